@@ -1,0 +1,357 @@
+"""Pins the CPU oracle against facts that do not come from the oracle itself:
+the reference's own fixture, library routines (torch/numpy) in the special cases
+where they compute the same thing, closed forms and brute force."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle as orc
+from oracle import ops as oops
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+rng = np.random.default_rng(1234)
+
+
+# ---------------------------------------------------------------- fp16 <-> fp32
+def test_f16_to_f32_exhaustive():
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([orc.f16_to_f32(int(v)) for v in h], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(nan, np.isnan(got))  # NaN payloads are not part of the contract
+    assert np.array_equal(want.view(np.uint32)[~nan], got.view(np.uint32)[~nan])
+
+
+def test_f32_to_f16_ties_and_random():
+    # every half value, the midpoint to its successor, and one fp32 ulp around the midpoint
+    h = np.arange(0, 0x7c00, dtype=np.uint16)
+    lo = h.view(np.float16).astype(np.float64)
+    hi = (h + 1).view(np.float16).astype(np.float64)
+    mid = ((lo + hi) / 2).astype(np.float32)
+    cands = np.concatenate([mid, np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf)),
+                            -mid, rng.standard_normal(20000).astype(np.float32) * 1000,
+                            np.array([0.0, -0.0, np.inf, -np.inf, 65504, 65519.99, 65520, 1e-8, 2.0 ** -25,
+                                      2.0 ** -24], dtype=np.float32)])
+    want = cands.astype(np.float16).view(np.uint16)
+    got = np.array([orc.f32_to_f16(v) for v in cands], dtype=np.uint16)
+    assert np.array_equal(want, got)
+
+
+# ---------------------------------------------------------------- positions (A3/A4)
+def _exact_pos(bw, scale):
+    qmax = 127 if bw == 8 else 32767
+    absmax = np.float32(qmax) / np.float32(scale)
+    return math.frexp(float(absmax))[1] - 1 - (bw - 2), float(absmax)
+
+
+def test_pos_from_scale_known_answers():
+    # absmax = 4 -> floor(log2 4) = 2 -> 2 - 6 ; absmax = 1 -> -6 ; absmax=0.4 -> -2-6
+    assert orc.pos_from_scale(8, 127.0 / 4.0) == -4
+    assert orc.pos_from_scale(8, 127.0) == -6
+    assert orc.pos_from_scale(8, 127.0 / 0.4) == -8
+    assert orc.pos_from_scale(16, 32767.0 / 3.0) == 1 - 14
+    assert orc.pos_from_scale(16, 32767.0 / 100.0) == 6 - 14
+
+
+def test_pos_from_scale_bruteforce_against_exponent():
+    for bw in (8, 16):
+        for s in np.exp(rng.uniform(-12, 12, 4000)).astype(np.float32):
+            want, absmax = _exact_pos(bw, s)
+            m = math.frexp(absmax)[0]  # in [0.5,1)
+            got = orc.pos_from_scale(bw, s)
+            if 0.5 + 1e-5 < m < 1 - 1e-5:
+                assert got == want
+            else:  # float log near an exact power of two may fall either side
+                assert abs(got - want) <= 1
+
+
+def test_quant_params_closed_form():
+    for bw in (8, 16):
+        qmax = 127 if bw == 8 else 32767
+        for s in np.exp(rng.uniform(-10, 10, 2000)).astype(np.float32):
+            pos, frac, sf = orc.quant_params(bw, s)
+            assert pos == orc.pos_from_scale(bw, s)
+            # scale_ = 2^pos * qmax / absmax lies in (qmax/2^(n-1), qmax/2^(n-2)]   (utils.cpp:97-100)
+            assert qmax / 2.0 ** (bw - 1) - 1e-5 <= frac <= qmax / 2.0 ** (bw - 2) + 1e-5
+            absmax = qmax / float(s)
+            assert math.isclose(frac, 2.0 ** pos * qmax / absmax, rel_tol=1e-5)
+            # scale_factor = absmax / qmax = 1/s
+            assert math.isclose(sf * float(s), 1.0, rel_tol=1e-5)
+
+
+def test_calib_scale():
+    assert orc.calib_scale(8, -2.0, 1.0) == 127.0 / 2.0
+    assert orc.calib_scale(16, -1.0, 4.0) == 32767.0 / 4.0
+    assert orc.calib_scale(8, 0.0, 0.0) == 1.0
+    assert orc.calib_scale(8, float("nan"), 1.0) == 1.0
+
+
+# ---------------------------------------------------------------- per-channel params (A7)
+def _fixture_rows():
+    rows = []
+    for line in open(os.path.join(GOLDEN, "inception_v3_qparams.txt")):
+        name, rest = line.split(" position: ")
+        pos, sc = rest.split(" scale: ")
+        sc = np.array(sc.split(), dtype=np.float32)
+        rows.append((name, int(pos), sc))
+    return rows
+
+
+def test_per_channel_params_reference_fixture():
+    """torch_mlu/csrc/test/data/test.txt holds, per Inception-v3 conv weight, the shared
+    position and the per-channel scales the reference's quantizer produced.  Feeding the
+    calibration scales they imply (s_c = new_scale_c * 2^-position) back through the
+    derivation must reproduce them; 43 of the 99 rows are exact half-way cases of
+    round((max+min)/2) and only round-half-to-even reproduces all of them."""
+    rows = [r for r in _fixture_rows() if r[2].size > 1]
+    assert len(rows) == 99
+    halfway = 0
+    for name, pos, sc in rows:
+        s = (sc.astype(np.float64) * 2.0 ** (-pos)).astype(np.float32)
+        new_pos, new_scale, sf = orc.per_channel_params(8, s)
+        assert new_pos == pos, name
+        np.testing.assert_allclose(new_scale, sc, rtol=2e-6, err_msg=name)
+        np.testing.assert_allclose(sf, 1.0 / s.astype(np.float64), rtol=2e-6, err_msg=name)
+        pc = np.floor(np.log2(127.0 / s.astype(np.float64))) - 6
+        if (pc.max() + pc.min()) % 2 != 0:
+            halfway += 1
+            # the two other common rounding rules disagree with the fixture on some rows
+    assert halfway == 43
+    up = sum(1 for _, pos, sc in rows if _np_round_rule(sc, pos, "half_up") != pos)
+    away = sum(1 for _, pos, sc in rows if _np_round_rule(sc, pos, "half_away") != pos)
+    assert up > 0 and away > 0
+
+
+def _np_round_rule(sc, pos, rule):
+    s = sc.astype(np.float64) * 2.0 ** (-pos)
+    pc = np.floor(np.log2(127.0 / s)) - 6
+    v = (pc.max() + pc.min()) / 2
+    if rule == "half_up":
+        return int(math.floor(v + 0.5))
+    return int(math.copysign(math.floor(abs(v) + 0.5), v))
+
+
+def test_per_channel_params_invariants():
+    for bw in (8, 16):
+        qmax = 127.0 if bw == 8 else 32767.0
+        s = np.exp(rng.uniform(-3, 9, 300)).astype(np.float32)
+        new_pos, new_scale, sf = orc.per_channel_params(bw, s)
+        pos_c = np.array([_exact_pos(bw, v)[0] for v in s])
+        scale_c = new_scale.astype(np.float64) * 2.0 ** (pos_c - new_pos)
+        lo, hi = qmax / 2.0 ** (bw - 1), qmax / 2.0 ** (bw - 2)
+        assert np.all(scale_c >= lo - 1e-5) and np.all(scale_c <= hi + 1e-5)
+        np.testing.assert_allclose(sf.astype(np.float64) * s, 1.0, rtol=3e-6)
+        assert new_pos == int(np.rint((pos_c.max() + pos_c.min()) / 2))
+        # one channel: shared position is that channel's own position
+        p1, ns1, _ = orc.per_channel_params(bw, s[:1])
+        assert p1 == pos_c[0] and lo - 1e-5 <= ns1[0] <= hi + 1e-5
+        np.testing.assert_allclose(ns1[0], 2.0 ** p1 * qmax / (qmax / float(s[0])), rtol=3e-6)
+
+
+# ---------------------------------------------------------------- quantize (A5)
+@pytest.mark.parametrize("bw", [8, 16, 31])
+def test_quantize_pos0_is_torch_round_clamp(bw):
+    qmin, qmax = {8: (-128, 127), 16: (-32768, 32767), 31: (-2 ** 30, 2 ** 30 - 1)}[bw]
+    x = np.concatenate([rng.standard_normal(50000) * 100, rng.standard_normal(5000) * 1e5,
+                        np.arange(-300, 300) + 0.5, [0.0, -0.0, 1e30, -1e30, np.inf, -np.inf]]).astype(np.float32)
+    want = torch.round(torch.from_numpy(x)).clamp(qmin, qmax).to(torch.int64).numpy()
+    got = orc.quantize(x, bw, 0).astype(np.int64)
+    assert np.array_equal(want, got)
+
+
+@pytest.mark.parametrize("bw", [8, 16])
+@pytest.mark.parametrize("pos", [-12, -7, -3, 0, 2, 5])
+def test_quantize_position_exact_vs_float64(bw, pos):
+    qmin, qmax = (-128, 127) if bw == 8 else (-32768, 32767)
+    k = np.arange(-400, 400)
+    ties = ((k + 0.5) * 2.0 ** pos).astype(np.float32)  # exactly representable half-way points
+    x = np.concatenate([ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+                        (rng.standard_normal(40000) * 2.0 ** (pos + 6)).astype(np.float32)])
+    want = np.clip(np.rint(x.astype(np.float64) * 2.0 ** (-pos)), qmin, qmax).astype(np.int64)
+    got = orc.quantize(x, bw, pos).astype(np.int64)
+    assert np.array_equal(want, got)
+    # half-to-even on the ties specifically: results are all even
+    t = orc.quantize(ties, 16, pos).astype(np.int64)
+    assert np.all(t % 2 == 0)
+
+
+def test_quantize_fp16_exhaustive():
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    for bw, pos in ((8, -4), (16, -9), (8, 0), (16, 3)):
+        qmin, qmax = (-128, 127) if bw == 8 else (-32768, 32767)
+        f = h.astype(np.float64)
+        want = np.where(np.isnan(f), 0, np.clip(np.rint(np.nan_to_num(f, nan=0.0) * 2.0 ** (-pos)), qmin, qmax))
+        got = orc.quantize(h, bw, pos)
+        assert np.array_equal(want.astype(np.int64), got.astype(np.int64))
+
+
+def test_quantize_fractional_scale_and_nan():
+    x = (rng.standard_normal(30000) * 3).astype(np.float32)
+    s = np.float32(1.3721)
+    want = np.clip(np.rint((x * s).astype(np.float32).astype(np.float64) * 2.0 ** 5), -128, 127)
+    assert np.array_equal(want.astype(np.int64), orc.quantize(x, 8, -5, s).astype(np.int64))
+    assert orc.quantize(np.array([np.nan], np.float32), 8, -3)[0] == 0
+    assert orc.quantize(np.zeros((0,), np.float32), 8, 0).size == 0
+
+
+def test_quantize_nchw_to_nhwc_matches_plain():
+    x = rng.standard_normal((2, 3, 5, 7)).astype(np.float32)
+    q = orc.quantize_nchw_to_nhwc(x, 8, -5, 1.0, cpad=4)
+    want = orc.quantize(np.transpose(x, (0, 2, 3, 1)), 8, -5)
+    assert np.array_equal(q[..., :3], want) and np.all(q[..., 3] == 0)
+
+
+@pytest.mark.parametrize("bw", [8, 16])
+def test_quantize_per_channel_is_round_div_clamp(bw):
+    """the reference spells the op chain out: clamp(round(input / scale_factor)) (quantify.cpp:100-105)"""
+    qmin, qmax = (-128, 127) if bw == 8 else (-32768, 32767)
+    w = (rng.standard_normal((17, 5, 3, 3)) * 0.05).astype(np.float32)
+    s = (qmax / np.abs(w).reshape(17, -1).max(1)).astype(np.float32)
+    _, _, sf = orc.per_channel_params(bw, s)
+    want = torch.clamp(torch.round(torch.from_numpy(w) / torch.from_numpy(sf).reshape(-1, 1, 1, 1)), qmin, qmax)
+    got = orc.quantize_per_channel(w, bw, sf)
+    assert np.array_equal(want.numpy().astype(np.int64), got.astype(np.int64))
+    assert np.abs(got.astype(np.int64)).max() >= qmax - 1  # the range is used
+
+
+def test_dequantize():
+    q = rng.integers(-128, 128, 1000).astype(np.int8)
+    np.testing.assert_array_equal(orc.dequantize(q, -5), q.astype(np.float32) * np.float32(2.0 ** -5))
+    q32 = rng.integers(-2 ** 20, 2 ** 20, 1000).astype(np.int32)
+    np.testing.assert_array_equal(orc.dequantize(q32, -9, 1.5),
+                                  (q32.astype(np.float32) * np.float32(2.0 ** -9)) / np.float32(1.5))
+
+
+# ---------------------------------------------------------------- int contraction (A9/A12)
+@pytest.mark.parametrize("bits", [(8, 8), (16, 8), (16, 16)])
+def test_gemm_nt_vs_torch_int64(bits):
+    lim = {8: 128, 16: 32768}
+    a = rng.integers(-lim[bits[0]], lim[bits[0]], (37, 129)).astype(np.int8 if bits[0] == 8 else np.int16)
+    b = rng.integers(-lim[bits[1]], lim[bits[1]], (23, 129)).astype(np.int8 if bits[1] == 8 else np.int16)
+    want = torch.from_numpy(a.astype(np.int64)) @ torch.from_numpy(b.astype(np.int64)).T
+    got, ovf = orc.gemm_nt(a, b)
+    assert ovf == 0 or bits == (16, 16)
+    assert np.array_equal(want.numpy(), got)
+
+
+def test_gemm_overflow_is_counted():
+    a = np.full((1, 600), 32767, np.int16)
+    b = np.full((1, 600), 127, np.int8)
+    acc, ovf = orc.gemm_nt(a, b)
+    assert ovf == 1 and acc[0, 0] == 32767 * 127 * 600
+
+
+CONV_CASES = [
+    # N, Ci, H, W, Co, kh, kw, pad, stride, dil, groups
+    (3, 64, 24, 24, 64, 3, 3, (3, 3), (3, 3), (1, 1), 1),  # the reference's qint grid (test_conv.py:104-131)
+    (2, 4, 6, 6, 16, 3, 3, (0, 0), (1, 1), (1, 1), 2),     # its groups case (test_conv.py:83-100)
+    (1, 3, 14, 14, 8, 2, 2, (0, 0), (1, 1), (1, 1), 1),
+    (2, 6, 9, 11, 10, 3, 2, (1, 2), (2, 1), (2, 1), 2),
+    (1, 8, 10, 10, 8, 3, 3, (1, 1), (2, 2), (1, 1), 8),    # depthwise
+    (1, 5, 7, 7, 4, 1, 1, (0, 0), (1, 1), (1, 1), 1),
+    (1, 16, 5, 5, 32, 5, 5, (2, 2), (1, 1), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("xbits", [8, 16])
+def test_conv2d_vs_torch_float64(case, xbits):
+    n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
+    lim = 128 if xbits == 8 else 32768
+    x = rng.integers(-lim, lim, (n, ci, h, w)).astype(np.int8 if xbits == 8 else np.int16)
+    wt = rng.integers(-128, 128, (co, ci // g, kh, kw)).astype(np.int8)
+    want = F.conv2d(torch.from_numpy(x.astype(np.float64)), torch.from_numpy(wt.astype(np.float64)), None,
+                    stride, pad, dil, g).numpy().astype(np.int64)
+    got, ovf = orc.conv2d_nhwc(np.transpose(x, (0, 2, 3, 1)), np.transpose(wt, (0, 2, 3, 1)), pad, stride, dil, g)
+    assert ovf == 0
+    assert np.array_equal(want, np.transpose(got, (0, 3, 1, 2)).astype(np.int64))
+    assert got.shape[1] == orc.conv_out_size(h, kh, pad[0], stride[0], dil[0])
+
+
+# ---------------------------------------------------------------- epilogue
+def test_epilogue_identity_and_order():
+    acc = rng.integers(-2 ** 26, 2 ** 26, (50, 12)).astype(np.int32)
+    assert np.array_equal(orc.epilogue(acc, 0), acc.astype(np.float32))
+    div = rng.uniform(0.5, 4, 12).astype(np.float32)
+    bias = rng.standard_normal(12).astype(np.float32)
+    res = rng.standard_normal((50, 12)).astype(np.float32)
+    v = acc.astype(np.float32) * np.float32(2.0 ** -11)
+    v = v / div
+    v = v + bias
+    v = v + res
+    relu = np.where(v > 0, v, np.float32(0))
+    assert np.array_equal(orc.epilogue(acc, -11, div, bias, res, 1), relu)
+    assert np.array_equal(orc.epilogue(acc, -11, div, bias, res, 2), np.minimum(relu, np.float32(6)))
+    assert np.array_equal(orc.epilogue(acc, -11, div, bias, res, 1, np.float16), relu.astype(np.float16))
+    # no fused multiply-add between the scaling and the bias: exact because 2^e scaling is exact
+    a1 = np.array([[2 ** 24 + 1]], np.int32)  # cvt rounds to 2^24, then exact scale, then add
+    assert orc.epilogue(a1, -24, None, np.array([1.0], np.float32))[0, 0] == np.float32(2.0)
+
+
+# ---------------------------------------------------------------- the reference's own acceptance metric
+def _rel_rms(a, b):  # test/common_utils.py:514-522 (use_MSE)
+    return math.sqrt(((a - b) ** 2).sum() / (a ** 2).sum())
+
+
+def _calibrate(x, w, bw, per_channel):
+    qmax = 127.0 if bw == 8 else 32767.0
+    s_in = orc.calib_scale(bw, x.min(), x.max())
+    if per_channel:
+        wf = w.reshape(w.shape[0], -1)
+        s_c = [orc.calib_scale(bw, lo, hi) for lo, hi in zip(wf.min(1), wf.max(1))]
+        return np.array([s_in, 0.0] + s_c, np.float32), np.array([3 if bw == 8 else 4], np.int32)
+    return np.array([s_in, orc.calib_scale(bw, w.min(), w.max())], np.float32), np.array([1 if bw == 8 else 2], np.int32)
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("bw", [8, 16])
+@pytest.mark.parametrize("per_channel", [True, False])
+@pytest.mark.parametrize("half", [False, True])
+def test_reference_conv_grid_rel_rms(bias, bw, per_channel, half):
+    """test/magicmind/op_test/test_conv.py:103-156: N=3 Ci=Co=64 HW=24 K=3 pad=3 stride=3, <= 0.02 vs float"""
+    g = torch.Generator().manual_seed(7)
+    conv = torch.nn.Conv2d(64, 64, 3, 3, 3, 1, 1, bias)
+    x = torch.randn(3, 64, 24, 24, generator=g)
+    with torch.no_grad():
+        want = conv(x).numpy()
+    w = conv.weight.detach().numpy()
+    b = conv.bias.detach().numpy() if bias else None
+    q_scale, q_mode = _calibrate(x.numpy(), w, bw, per_channel)
+    xin = x.numpy().astype(np.float16) if half else x.numpy()
+    r = oops.conv2d(xin, w, b, (3, 3), (3, 3), (1, 1), 1, q_scale, q_mode)
+    assert r["overflow"] == 0 or bw == 16  # int16 x int16 is defined on the exact (int64) sum
+    assert r["y"].dtype == (np.float16 if half else np.float32)
+    assert _rel_rms(want.astype(np.float64), r["y"].astype(np.float64)) <= 0.02
+
+
+@pytest.mark.parametrize("ni,ci,co", [(1, 10, 25), (10, 50, 75), (20, 100, 125)])
+@pytest.mark.parametrize("bw", [8, 16])
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_reference_linear_grid_rel_rms(ni, ci, co, bw, per_channel):
+    """test/magicmind/op_test/test_matmul.py:116-174, <= 0.02 vs float"""
+    g = torch.Generator().manual_seed(ni + ci)
+    lin = torch.nn.Linear(ci, co, True)
+    x = torch.rand(ni, ci, generator=g)
+    with torch.no_grad():
+        want = lin(x).numpy()
+    w, b = lin.weight.detach().numpy(), lin.bias.detach().numpy()
+    q_scale, q_mode = _calibrate(x.numpy(), w, bw, per_channel)
+    r = oops.linear(x.numpy(), w, b, q_scale, q_mode)
+    assert (r["overflow"] == 0 or bw == 16) and r["y"].dtype == np.float32
+    assert _rel_rms(want.astype(np.float64), r["y"].astype(np.float64)) <= 0.02
+
+
+def test_dequantized_float_conv_agrees():
+    """float conv of the dequantized integers == integer conv scaled by 2^(pos_x+pos_w)"""
+    x = rng.standard_normal((1, 8, 9, 9)).astype(np.float32)
+    w = (rng.standard_normal((6, 8, 3, 3)) * 0.1).astype(np.float32)
+    q_scale, q_mode = _calibrate(x, w, 8, False)
+    r = oops.conv2d(x, w, None, (1, 1), (1, 1), (1, 1), 1, q_scale, q_mode)
+    xd = orc.dequantize(np.transpose(r["qx"], (0, 3, 1, 2)), r["pos_x"]).astype(np.float64)
+    wd = orc.dequantize(np.transpose(r["qw"], (0, 3, 1, 2)), r["pos_w"]).astype(np.float64)
+    want = F.conv2d(torch.from_numpy(xd), torch.from_numpy(wd), None, 1, 1).numpy()
+    np.testing.assert_allclose(r["y"], want, rtol=1e-6, atol=1e-6)
