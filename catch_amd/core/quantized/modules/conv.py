@@ -1,0 +1,155 @@
+"""Quantized Conv2d module (counterpart of torch_mlu/core/quantized/modules/conv.py).
+
+On CPU tensors the module is the float convolution plus an input observer: that is the
+calibration pass (conv.py:174-177 in the reference).  On device tensors it calls
+``torch.ops.torch_mlu.conv2d`` with the packed q-params (conv.py:178-190)."""
+import logging
+
+import torch
+import torch.nn.functional as F
+from torch.nn.modules.conv import Conv2d as NNConv2d
+from torch.nn.modules.utils import _pair
+from torch.nn.parameter import Parameter
+
+from .mlumodel import MLUModel
+
+
+class MLUConv2d(torch.nn.Module, MLUModel):
+    # only the first convolution of a network may take the first-conv normalisation
+    is_first_layer = True
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1,
+                 bias=True, padding_mode="zeros"):
+        super().__init__()
+        if in_channels % groups != 0:
+            raise ValueError("in_channels must be divisible by groups")
+        if out_channels % groups != 0:
+            raise ValueError("out_channels    must be divisible by groups")
+        self.in_channels, self.out_channels, self.groups = in_channels, out_channels, groups
+        self.kernel_size, self.stride = _pair(kernel_size), _pair(stride)
+        self.padding, self.dilation = _pair(padding), _pair(dilation)
+        self.padding_mode = padding_mode
+        self.weight = Parameter(torch.empty(out_channels, in_channels // groups, *self.kernel_size))
+        if bias:
+            self.bias = Parameter(torch.empty(out_channels))
+        else:
+            self.register_parameter("bias", None)
+        self.scale = None
+        self.quantized_mode = None
+        self.use_symmetry = Parameter(torch.tensor([1]), requires_grad=False)
+        self.input_std = None
+        self.input_mean = None
+        self.quant = False
+        ref = NNConv2d(in_channels, out_channels, self.kernel_size, groups=groups, bias=bias)
+        with torch.no_grad():
+            self.weight.copy_(ref.weight)
+            if bias:
+                self.bias.copy_(ref.bias)
+
+    # -- calibration ----------------------------------------------------------------------------
+    def _observer_forward_hook(self, module, inputs, output):
+        return self.observer(*inputs)
+
+    def _float_forward(self, x):
+        if self.padding_mode == "circular":
+            ph, pw = self.padding
+            x = F.pad(x, ((pw + 1) // 2, pw // 2, (ph + 1) // 2, ph // 2), mode="circular")
+            return F.conv2d(x, self.weight, self.bias, self.stride, _pair(0), self.dilation, self.groups)
+        return F.conv2d(x, self.weight, self.bias, self.stride, self.padding, self.dilation, self.groups)
+
+    def forward(self, input):
+        if input.device.type == "cpu":
+            return self._float_forward(input)
+        if self.input_std is not None:
+            input = (input - self.input_mean) / self.input_std
+        return torch.ops.torch_mlu.conv2d(input, self.weight, self.bias, list(self.padding), list(self.stride),
+                                          list(self.dilation), self.groups, self.scale, self.quantized_mode)
+
+    # -- checkpoint format: weight, bias, scale, quantized_mode [, quantized_by_channel,
+    #    scale_weight_per_channel, input_mean, input_std] (conv.py:77-131) ---------------------------
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        if self.weight is not None:
+            destination[prefix + "weight"] = self.weight
+        if self.bias is not None:
+            destination[prefix + "bias"] = self.bias
+        if not self.quant:
+            return
+        weight_observer = self.qconfig.weight()
+        weight_observer(self.weight)
+        weight_observer.calculate_qparams()
+        self.observer.calculate_qparams()
+        self.set_quantized_mode(torch.Tensor([2 if self.observer.dtype == "int16" else 1]))
+        if weight_observer._get_name() == "MLUPerChannelMinMaxObserver":
+            destination[prefix + "quantized_by_channel"] = torch.tensor([1])
+            destination[prefix + "scale_weight_per_channel"] = torch.tensor(weight_observer.scales)
+            self.set_scale(torch.tensor([self.observer.scale, 0.0]))
+        else:
+            self.set_scale(torch.tensor([self.observer.scale, weight_observer.scale]))
+        destination[prefix + "scale"] = self.scale.data
+        destination[prefix + "quantized_mode"] = self.quantized_mode.data
+        if self.input_std is not None:
+            destination[prefix + "input_mean"] = self.input_mean.data.mul(255)
+            destination[prefix + "input_std"] = self.input_std.data.mul(255)
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, False, missing_keys, unexpected_keys,
+                                      error_msgs)
+        if prefix + "scale" in state_dict:
+            self.set_scale(state_dict[prefix + "scale"], state_dict.get(prefix + "scale_weight_per_channel"))
+        if prefix + "quantized_mode" in state_dict:
+            self.set_quantized_mode(state_dict[prefix + "quantized_mode"],
+                                    state_dict.get(prefix + "quantized_by_channel"))
+        if prefix + "input_mean" in state_dict and prefix + "input_std" in state_dict:
+            self.set_mean_std(state_dict[prefix + "input_mean"], state_dict[prefix + "input_std"])
+        if state_dict.get(prefix + "bias") is None:
+            self.set_bias_with_zeros(self.out_channels)
+        for lst in (missing_keys, unexpected_keys):  # the quantization keys are optional both ways
+            for k in [k for k in lst if k.startswith(prefix)]:
+                lst.remove(k)
+
+    def extra_repr(self):
+        return ("{in_channels}, {out_channels}, kernel_size={kernel_size}, stride={stride}, padding={padding}, "
+                "dilation={dilation}, groups={groups}").format(**self.__dict__) + \
+               ", scale={}, quantized_mode={}".format(self.scale, self.quantized_mode)
+
+    def _apply(self, fn, recurse=True):
+        # q_scale stays fp32 under .half(): int16 scales (32767/absmax) overflow fp16
+        kept = None if self.scale is None else self.scale.detach().clone()
+        super()._apply(fn)
+        if kept is not None and self.scale is not None and self.scale.dtype != torch.float32:
+            self.scale = Parameter(kept.detach().to(device=self.scale.device, dtype=torch.float32),
+                                   requires_grad=False)
+        return self
+
+    def _get_name(self):
+        return "MLUConv2d"
+
+    @classmethod
+    def from_float(cls, mod, gen_quant):
+        assert isinstance(mod, NNConv2d), "MLUConv2d only works for nn.Conv2d or its subclass"
+        assert hasattr(mod, "qconfig"), "Input float module must have qconfig defined"
+        q = cls(mod.in_channels, mod.out_channels, mod.kernel_size, mod.stride, mod.padding, mod.dilation,
+                mod.groups, mod.bias is not None, mod.padding_mode)
+        q.set_weight_bias(mod.weight, mod.bias)
+        if gen_quant:
+            q.quant = True
+            if cls.is_first_layer:
+                conf = mod.qconfig.activation().qscheme
+                if conf["firstconv"] is True:
+                    assert conf["mean"] is not None and conf["std"] is not None, \
+                        "You are using firstconv but forget setting mean or std, please set mean and std in qconfig!"
+                    assert q.in_channels in [1, 3, 4], \
+                        "firstconv needs 1 (GRAY), 3 (RGB) or 4 (RGBA) input channels, got {}".format(q.in_channels)
+                    assert min(conf["mean"]) >= 0 and max(conf["mean"]) <= 1 and \
+                        min(conf["std"]) >= 0 and max(conf["std"]) <= 1, \
+                        "firstconv mean and std must lie in [0.0, 1.0] (they are multiplied by 255 when saved)"
+                    if set(conf["mean"]) == {0} and set(conf["std"]) == {1}:
+                        logging.warning("firstconv with default mean [0,0,0] and std [1,1,1]: check that this is intended")
+                    q.set_mean_std(torch.Tensor(conf["mean"]), torch.Tensor(conf["std"]))
+                cls.is_first_layer = False
+            q.qconfig = mod.qconfig
+            q.observer = q.qconfig.activation()
+            q.register_forward_hook(q._observer_forward_hook)
+        return q

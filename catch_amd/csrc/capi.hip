@@ -1,0 +1,117 @@
+// C ABI entry points of the integer contractions: argument checks, then the route.
+#include <cstring>
+
+#include "catchq_common.h"
+
+namespace catchq {
+
+int gemm_nt_direct(const void *a, int a_bits, const void *b, int b_bits, int64_t M, int64_t N, int64_t K,
+                   const EpiDev &e, hipStream_t s);
+int conv2d_direct(const void *x, int x_bits, const void *w, int w_bits, const ConvDev &d, const EpiDev &e,
+                  hipStream_t s);
+int gemm_nt_mfma_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e,
+                    hipStream_t s);
+int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph,
+                   int pw, int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
+bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
+int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
+              int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
+
+enum Route { kDirect, kMfma, kDepthwise, kBad };
+
+static Route gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k, const void *a, const void *b) {
+  if (a_bits == 8 && b_bits == 8 && k % 16 == 0 && k >= 16 && m > 0 && n > 0 && k < (1ll << 31) &&
+      n < (1ll << 31) && (!a || aligned16(a)) && (!b || aligned16(b)))
+    return kMfma;
+  return kDirect;
+}
+
+static Route conv_route(int x_bits, int w_bits, const catchq_conv_desc_t *d, const void *x, const void *w) {
+  if (x_bits == 8 && w_bits == 8) {
+    // is_depthwise_conv: groups != 1, co % groups == 0, one input channel per group, groups == ci
+    if (d->groups != 1 && d->groups == d->ci && d->co == d->ci &&
+        dwconv_i8_supported(d->ci, d->kh, d->kw, d->stride_w, d->dil_w) && (!x || aligned16(x)))
+      return kDepthwise;
+    if (d->groups == 1 && d->ci % 16 == 0 && (!x || aligned16(x)) && (!w || aligned16(w))) return kMfma;
+  }
+  return kDirect;
+}
+
+static const char *route_name(Route r) {
+  switch (r) {
+    case kMfma: return "mfma";
+    case kDepthwise: return "depthwise";
+    case kDirect: return "direct";
+    default: return "invalid";
+  }
+}
+
+static int check_conv(const catchq_conv_desc_t *d, int *ho, int *wo) {
+  if (!d) return CATCHQ_ERR_ARG;
+  if (d->n < 0 || d->h <= 0 || d->w <= 0 || d->ci <= 0 || d->co <= 0 || d->kh <= 0 || d->kw <= 0)
+    return CATCHQ_ERR_SHAPE;
+  if (d->pad_h < 0 || d->pad_w < 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dil_h <= 0 || d->dil_w <= 0)
+    return CATCHQ_ERR_SHAPE;
+  if (d->groups <= 0 || d->ci % d->groups != 0 || d->co % d->groups != 0) return CATCHQ_ERR_SHAPE;
+  *ho = catchq_conv_out_size(d->h, d->kh, d->pad_h, d->stride_h, d->dil_h);
+  *wo = catchq_conv_out_size(d->w, d->kw, d->pad_w, d->stride_w, d->dil_w);
+  if (*ho <= 0 || *wo <= 0) return CATCHQ_ERR_SHAPE;
+  return CATCHQ_OK;
+}
+
+}  // namespace catchq
+
+using namespace catchq;
+
+CATCHQ_API const char *catchq_gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k) {
+  return route_name(gemm_route(a_bits, b_bits, m, n, k, nullptr, nullptr));
+}
+
+CATCHQ_API const char *catchq_conv2d_route(int x_bits, int w_bits, const catchq_conv_desc_t *desc) {
+  int ho, wo;
+  if (check_conv(desc, &ho, &wo) != CATCHQ_OK) return route_name(kBad);
+  return route_name(conv_route(x_bits, w_bits, desc, nullptr, nullptr));
+}
+
+CATCHQ_API int catchq_gemm_nt(const void *a, int a_bits, const void *b, int b_bits, int64_t m, int64_t n,
+                              int64_t k, const catchq_epilogue_t *epilogue, catchq_stream_t stream) {
+  if (m < 0 || n < 0 || k < 0) return CATCHQ_ERR_SHAPE;
+  if ((a_bits != 8 && a_bits != 16) || (b_bits != 8 && b_bits != 16)) return CATCHQ_ERR_BITWIDTH;
+  int st = check_epi(epilogue);
+  if (st != CATCHQ_OK) return st;
+  if (m == 0 || n == 0) return CATCHQ_OK;
+  if (k > 0 && (!a || !b)) return CATCHQ_ERR_ARG;
+  const EpiDev e = make_epi(epilogue);
+  hipStream_t s = as_stream(stream);
+  if (gemm_route(a_bits, b_bits, m, n, k, a, b) == kMfma) return gemm_nt_mfma_i8(a, b, m, n, k, e, s);
+  return gemm_nt_direct(a, a_bits, b, b_bits, m, n, k, e, s);
+}
+
+CATCHQ_API int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int w_bits,
+                                  const catchq_conv_desc_t *desc, const catchq_epilogue_t *epilogue,
+                                  catchq_stream_t stream) {
+  int ho, wo;
+  int st = check_conv(desc, &ho, &wo);
+  if (st != CATCHQ_OK) return st;
+  if ((x_bits != 8 && x_bits != 16) || (w_bits != 8 && w_bits != 16)) return CATCHQ_ERR_BITWIDTH;
+  st = check_epi(epilogue);
+  if (st != CATCHQ_OK) return st;
+  if (desc->n == 0) return CATCHQ_OK;
+  if (!x || !w) return CATCHQ_ERR_ARG;
+  const EpiDev e = make_epi(epilogue);
+  hipStream_t s = as_stream(stream);
+  const catchq_conv_desc_t &d = *desc;
+  switch (conv_route(x_bits, w_bits, desc, x, w)) {
+    case kDepthwise:
+      return dwconv_i8(x, w, d.n, d.h, d.w, d.ci, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h, d.stride_w, d.dil_h,
+                       d.dil_w, ho, wo, e, s);
+    case kMfma:
+      return conv2d_mfma_i8(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h,
+                            d.stride_w, d.dil_h, d.dil_w, ho, wo, e, s);
+    default: {
+      ConvDev cd = {d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h, d.stride_w,
+                    d.dil_h, d.dil_w, d.groups, ho, wo};
+      return conv2d_direct(x, x_bits, w, w_bits, cd, e, s);
+    }
+  }
+}

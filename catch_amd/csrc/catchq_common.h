@@ -1,0 +1,122 @@
+// Shared device helpers of the catchq kernels (gfx950 only).
+#pragma once
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "catchq.h"
+
+#define CATCHQ_API extern "C" __attribute__((visibility("default")))
+
+namespace catchq {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+inline hipStream_t as_stream(catchq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? CATCHQ_OK : CATCHQ_ERR_LAUNCH; }
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- the quantize rule: q = sat(rne(x * scale * 2^-pos)), NaN -> 0 -------------------------
+template <int BW>
+struct QRange;
+template <>
+struct QRange<8> {
+  typedef int8_t type;
+  static constexpr float lo = -128.0f, hi = 127.0f;
+};
+template <>
+struct QRange<16> {
+  typedef int16_t type;
+  static constexpr float lo = -32768.0f, hi = 32767.0f;
+};
+template <>
+struct QRange<31> {
+  typedef int32_t type;
+  static constexpr float lo = -1073741824.0f, hi = 1073741823.0f;
+};
+
+// x*scale is one fp32 rounding (exact for scale == 1), the scaling by 2^-pos is exact.
+template <int BW>
+__device__ __forceinline__ int quant1(float x, float scale, int neg_pos) {
+  float t = __builtin_ldexpf(x * scale, neg_pos);
+  float r = __builtin_rintf(t);
+  r = fminf(fmaxf(r, QRange<BW>::lo), QRange<BW>::hi);
+  return (t != t) ? 0 : (int)r;
+}
+
+struct ConvDev {
+  int N, H, W, Ci, Co, kh, kw, ph, pw, sh, sw, dh, dw, groups, Ho, Wo;
+};
+
+// ---- epilogue applied to one integer sum -----------------------------------------------------
+struct EpiDev {
+  int exp2;
+  const float *chan_div;
+  const float *bias;
+  const float *resid;
+  int act;
+  void *y;
+  int y_f16;
+  int32_t *acc_out;
+  void *q;
+  int q_bw;
+  int q_neg_pos;
+  float q_scale;
+};
+
+inline EpiDev make_epi(const catchq_epilogue_t *e) {
+  EpiDev d;
+  d.exp2 = e->exp2;
+  d.chan_div = e->chan_div;
+  d.bias = e->bias;
+  d.resid = e->resid;
+  d.act = e->act;
+  d.y = e->y;
+  d.y_f16 = (e->y_dtype == CATCHQ_F16);
+  d.acc_out = e->acc_out;
+  d.q = e->q;
+  d.q_bw = e->q_bitwidth;
+  d.q_neg_pos = -e->q_position;
+  d.q_scale = e->q_scale;
+  return d;
+}
+
+inline int check_epi(const catchq_epilogue_t *e) {
+  if (!e) return CATCHQ_ERR_ARG;
+  if (!e->y && !e->acc_out && !e->q) return CATCHQ_ERR_ARG;
+  if (e->y && e->y_dtype != CATCHQ_F32 && e->y_dtype != CATCHQ_F16) return CATCHQ_ERR_DTYPE;
+  if (e->q && e->q_bitwidth != 8 && e->q_bitwidth != 16) return CATCHQ_ERR_BITWIDTH;
+  if (e->act < CATCHQ_ACT_NONE || e->act > CATCHQ_ACT_RELU6) return CATCHQ_ERR_ARG;
+  if (e->exp2 < -126 || e->exp2 > 126) return CATCHQ_ERR_ARG;
+  if (e->q && (e->q_position < -126 || e->q_position > 126)) return CATCHQ_ERR_ARG;
+  return CATCHQ_OK;
+}
+
+// value after dequant / bias / residual / activation; facc = float(acc) (one RNE conversion)
+__device__ __forceinline__ float epi_value(float facc, int64_t idx, int c, const EpiDev &e) {
+  float v = __builtin_ldexpf(facc, e.exp2);
+  if (e.chan_div) v = v / e.chan_div[c];
+  if (e.bias) v = v + e.bias[c];
+  if (e.resid) v = v + e.resid[idx];
+  if (e.act >= CATCHQ_ACT_RELU) v = (v > 0.0f) ? v : 0.0f;
+  if (e.act == CATCHQ_ACT_RELU6) v = (v < 6.0f) ? v : 6.0f;
+  return v;
+}
+
+__device__ __forceinline__ void epi_store(float v, int64_t idx, const EpiDev &e) {
+  if (e.y) {
+    if (e.y_f16) reinterpret_cast<__half *>(e.y)[idx] = __float2half_rn(v);
+    else reinterpret_cast<float *>(e.y)[idx] = v;
+  }
+  if (e.q) {
+    if (e.q_bw == 8) reinterpret_cast<int8_t *>(e.q)[idx] = (int8_t)quant1<8>(v, e.q_scale, e.q_neg_pos);
+    else reinterpret_cast<int16_t *>(e.q)[idx] = (int16_t)quant1<16>(v, e.q_scale, e.q_neg_pos);
+  }
+}
+
+}  // namespace catchq

@@ -1,0 +1,104 @@
+// Host-side quantization-parameter math (scalars and per-channel vectors; no device work).
+#include <cmath>
+#include <vector>
+
+#include "catchq.h"
+
+#define CATCHQ_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+struct Range {
+  int n;
+  int qmin, qmax;
+};
+
+bool range_for(int bitwidth, Range *r) {
+  if (bitwidth == 8) {
+    *r = {8, -128, 127};
+    return true;
+  }
+  if (bitwidth == 16) {
+    *r = {16, -32768, 32767};
+    return true;
+  }
+  return false;
+}
+
+}  // namespace
+
+CATCHQ_API int catchq_version(void) { return 100; }
+
+CATCHQ_API const char *catchq_status_string(int status) {
+  switch (status) {
+    case CATCHQ_OK: return "ok";
+    case CATCHQ_ERR_ARG: return "invalid argument";
+    case CATCHQ_ERR_DTYPE: return "quantify only support input float/half";
+    case CATCHQ_ERR_BITWIDTH: return "bitwidth not support";
+    case CATCHQ_ERR_SHAPE: return "inconsistent shapes";
+    case CATCHQ_ERR_LAUNCH: return "kernel launch failed";
+    case CATCHQ_ERR_UNSUPPORTED: return "combination not supported";
+    default: return "unknown status";
+  }
+}
+
+// cnnl/cnnl_util.cpp:337-347 -- float absmax, float log over double log(2), floor, minus (bitwidth-2).
+CATCHQ_API int catchq_pos_from_scale(int bitwidth, float scale, int *position) {
+  Range r;
+  if (!position) return CATCHQ_ERR_ARG;
+  if (!range_for(bitwidth, &r)) return CATCHQ_ERR_BITWIDTH;
+  if (!(scale > 0.0f) || std::isinf(scale)) return CATCHQ_ERR_ARG;  // the logarithm below needs a finite absmax > 0
+  const float absmax = r.qmax / scale;
+  *position = static_cast<int>(std::floor(std::log(absmax) / std::log(2)) - (bitwidth - 2));
+  return CATCHQ_OK;
+}
+
+// jit/utils/utils.cpp:81-105 -- the intermediate values live in floats, the expressions in double.
+CATCHQ_API int catchq_quant_params(int bitwidth, float scale, int *position, float *scale_frac,
+                                   float *scale_factor) {
+  Range r;
+  if (!position || !scale_frac || !scale_factor) return CATCHQ_ERR_ARG;
+  if (!range_for(bitwidth, &r)) return CATCHQ_ERR_BITWIDTH;
+  if (!(scale > 0.0f) || std::isinf(scale)) return CATCHQ_ERR_ARG;
+  const float absmax = r.qmax / scale;
+  const float pos = std::floor(std::log(absmax) / std::log(2)) - (r.n - 2);
+  const float frac = std::pow(2, pos) * (std::pow(2, (r.n - 1)) - 1) / absmax;
+  const float factor = std::pow(2, pos) / frac;
+  *position = static_cast<int>(pos);
+  *scale_frac = frac;
+  *scale_factor = factor;
+  return CATCHQ_OK;
+}
+
+// operators/cnnl/quantify.cpp:55-98 -- every step is an fp32 tensor op there, so every step is
+// an fp32 scalar op here.
+CATCHQ_API int catchq_per_channel_params(int bitwidth, const float *scales, int co, int *new_position,
+                                         float *new_scale, float *scale_factor) {
+  Range r;
+  if (!scales || !new_position || !new_scale || !scale_factor || co <= 0) return CATCHQ_ERR_ARG;
+  if (!range_for(bitwidth, &r)) return CATCHQ_ERR_BITWIDTH;
+  const float qmax = static_cast<float>(r.qmax);
+  for (int c = 0; c < co; ++c)
+    if (!(scales[c] > 0.0f) || std::isinf(scales[c])) return CATCHQ_ERR_ARG;
+  std::vector<float> pos(co), chan_scale(co);
+  float pos_hi = 0.f, pos_lo = 0.f;
+  for (int c = 0; c < co; ++c) {
+    const float absmax = qmax / scales[c];
+    pos[c] = std::floor(std::log2(absmax)) - static_cast<float>(bitwidth - 2);
+    chan_scale[c] = (std::exp2(pos[c]) * qmax) / absmax;
+    pos_hi = (c == 0) ? pos[c] : std::fmax(pos_hi, pos[c]);
+    pos_lo = (c == 0) ? pos[c] : std::fmin(pos_lo, pos[c]);
+  }
+  const float shared = std::nearbyint((pos_hi + pos_lo) / 2.0f);  // half-to-even
+  for (int c = 0; c < co; ++c) {
+    new_scale[c] = chan_scale[c] * std::exp2(shared - pos[c]);
+    scale_factor[c] = std::exp2(shared) / new_scale[c];
+  }
+  *new_position = static_cast<int>(shared);
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_conv_out_size(int in, int k, int pad, int stride, int dil) {
+  const int kernel = dil * (k - 1) + 1;
+  return (in + 2 * pad - kernel) / stride + 1;
+}

@@ -1,0 +1,543 @@
+// PyTorch-ROCm front end of the catchq C ABI.
+//
+// Registers the reference's two custom-op schemas unchanged
+//   torch_mlu::conv2d(input, weight, bias, padding, stride, dilation, groups, q_scale, q_mode)
+//   torch_mlu::linear(input, weight, bias, q_scale, q_mode)
+// (torch_mlu/tools/mlu_functions.yaml:806-846, registered by tools/gen.py:38-43 in the reference)
+// plus helper ops that mirror the reference's C++-internal kernels
+// (tools/template/cnnl_kernel.h:48-72): quantize, quantize_per_channel, quantize_param, mm_q,
+// and the integer-in/integer-out building blocks qconv2d / qlinear used by fused pipelines.
+//
+// Device tensors only: there is deliberately no CPU implementation behind these ops (the
+// reference's own CPU fall-back for them returns its input, operators/op_methods.cpp:1019-1035).
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/DeviceGuard.h>
+#include <torch/library.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "catchq.h"
+
+namespace {
+
+using at::Tensor;
+
+void check_status(int st, const char *what) {
+  TORCH_CHECK(st == CATCHQ_OK, what, ": ", catchq_status_string(st));
+}
+
+catchq_stream_t current_stream() {
+  return reinterpret_cast<catchq_stream_t>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
+}
+
+int fp_dtype(const Tensor &t, const char *msg) {
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kHalf, msg);
+  return t.scalar_type() == at::kHalf ? CATCHQ_F16 : CATCHQ_F32;
+}
+
+at::ScalarType int_type(int64_t bitwidth) {
+  switch (bitwidth) {
+    case 8: return at::kChar;
+    case 16: return at::kShort;
+    case 31: return at::kInt;
+    default: TORCH_CHECK(false, "bitwidth not support");
+  }
+}
+
+int bits_of(const Tensor &t) {
+  switch (t.scalar_type()) {
+    case at::kChar: return 8;
+    case at::kShort: return 16;
+    case at::kInt: return 32;
+    default: TORCH_CHECK(false, "expected an int8/int16/int32 tensor, got ", t.scalar_type());
+  }
+}
+
+bool has_bias(const Tensor &b) { return b.defined() && b.numel() != 0 && b.dim() != 0; }
+
+// ------------------------------------------------------------------------------------------------
+// quantize family
+// ------------------------------------------------------------------------------------------------
+
+// cnnl_quantify_offline(input, bitwidth, int position): same shape and memory format as the input.
+Tensor quantize_op(const Tensor &x, int64_t bitwidth, int64_t position, double scale) {
+  const int dt = fp_dtype(x, "quantify only support input float/half");
+  c10::DeviceGuard guard(x.device());
+  Tensor xi = x.is_non_overlapping_and_dense() ? x : x.contiguous();
+  Tensor q = at::empty_like(xi, xi.options().dtype(int_type(bitwidth)));
+  check_status(catchq_quantize(xi.data_ptr(), dt, q.data_ptr(), (int)bitwidth, xi.numel(), (int)position,
+                               (float)scale, current_stream()),
+               "torch_mlu::quantize");
+  return q;
+}
+
+// cnnl_quantify_offline(input, bitwidth, Tensor position): position stays on the device.
+Tensor quantize_dev_op(const Tensor &x, int64_t bitwidth, const Tensor &position) {
+  const int dt = fp_dtype(x, "quantify only support input float/half");
+  TORCH_CHECK(position.scalar_type() == at::kInt && position.numel() == 1 && position.device() == x.device(),
+              "position must be a one-element int32 tensor on the input's device");
+  c10::DeviceGuard guard(x.device());
+  Tensor xi = x.is_non_overlapping_and_dense() ? x : x.contiguous();
+  Tensor q = at::empty_like(xi, xi.options().dtype(int_type(bitwidth)));
+  check_status(catchq_quantize_devpos(xi.data_ptr(), dt, q.data_ptr(), (int)bitwidth, xi.numel(),
+                                      position.data_ptr<int32_t>(), nullptr, current_stream()),
+               "torch_mlu::quantize_dev");
+  return q;
+}
+
+// cnnl_quantize_param(input, bitwidth, mode) -> (position int32[1], scale fp32[1], offset fp32[1])
+std::tuple<Tensor, Tensor, Tensor> quantize_param_op(const Tensor &x, int64_t bitwidth, int64_t mode) {
+  const int dt = fp_dtype(x, "quantize_param only support input float/half");
+  c10::DeviceGuard guard(x.device());
+  Tensor xi = x.is_non_overlapping_and_dense() ? x : x.contiguous();
+  size_t ws_bytes = 0;
+  check_status(catchq_quantize_param_workspace_size(xi.numel(), &ws_bytes), "torch_mlu::quantize_param");
+  Tensor ws = at::empty({(int64_t)ws_bytes}, xi.options().dtype(at::kChar));
+  Tensor pos = at::empty({1}, xi.options().dtype(at::kInt));
+  Tensor scale = at::ones({1}, xi.options().dtype(at::kFloat));
+  Tensor offset = at::zeros({1}, xi.options().dtype(at::kFloat));
+  check_status(catchq_quantize_param(xi.data_ptr(), dt, xi.numel(), (int)bitwidth, (int)mode, ws.data_ptr(),
+                                     ws_bytes, nullptr, pos.data_ptr<int32_t>(), scale.data_ptr<float>(),
+                                     offset.data_ptr<float>(), current_stream()),
+               "torch_mlu::quantize_param");
+  return std::make_tuple(pos, scale, offset);
+}
+
+struct PerChannel {
+  int new_pos = 0;
+  Tensor new_scale;     // device fp32 [Co]
+  Tensor scale_factor;  // device fp32 [Co]
+};
+
+PerChannel per_channel_params(const float *scales_host, int64_t co, int bw, const at::TensorOptions &dev_opts) {
+  std::vector<float> ns(co), sf(co);
+  PerChannel pc;
+  check_status(catchq_per_channel_params(bw, scales_host, (int)co, &pc.new_pos, ns.data(), sf.data()),
+               "per-channel parameters");
+  auto host = at::TensorOptions().dtype(at::kFloat);
+  pc.new_scale = at::from_blob(ns.data(), {co}, host).to(dev_opts.device(), /*non_blocking=*/false);
+  pc.scale_factor = at::from_blob(sf.data(), {co}, host).to(dev_opts.device(), false);
+  return pc;
+}
+
+Tensor quantize_weight_per_channel(const Tensor &w_dense, const PerChannel &pc, int bw) {
+  const int dt = fp_dtype(w_dense, "quantify only support input float/half");
+  Tensor q = at::empty_like(w_dense, w_dense.options().dtype(int_type(bw)));
+  const int64_t co = w_dense.size(0);
+  check_status(catchq_quantize_per_channel(w_dense.data_ptr(), dt, q.data_ptr(), bw, (int)co,
+                                           co ? w_dense.numel() / co : 0, pc.scale_factor.data_ptr<float>(),
+                                           current_stream()),
+               "torch_mlu::quantize_per_channel");
+  return q;
+}
+
+// cnnl_quantify_per_channel(input, scale_data, bitwidth) -> (quantized, new_position[1], new_scale[Co])
+std::tuple<Tensor, Tensor, Tensor> quantize_per_channel_op(const Tensor &w, const Tensor &scales, int64_t bitwidth) {
+  TORCH_CHECK(bitwidth == 8 || bitwidth == 16, "bitwidth not support");
+  TORCH_CHECK(w.dim() >= 1 && scales.numel() == w.size(0), "one scale per output channel expected");
+  c10::DeviceGuard guard(w.device());
+  Tensor s_host = scales.to(at::kCPU, at::kFloat).contiguous();
+  PerChannel pc = per_channel_params(s_host.data_ptr<float>(), s_host.numel(), (int)bitwidth, w.options());
+  // dim 0 must be the slowest-varying dimension of the memory: true for contiguous and channels-last
+  Tensor wd = w.is_non_overlapping_and_dense() && w.stride(0) * w.size(0) == w.numel() ? w : w.contiguous();
+  Tensor q = quantize_weight_per_channel(wd, pc, (int)bitwidth);
+  Tensor new_pos = at::full({1}, (double)pc.new_pos, w.options().dtype(at::kFloat));
+  return std::make_tuple(q, new_pos, pc.new_scale);
+}
+
+Tensor dequantize_op(const Tensor &q, int64_t position, double scale, bool half) {
+  c10::DeviceGuard guard(q.device());
+  Tensor qi = q.is_non_overlapping_and_dense() ? q : q.contiguous();
+  Tensor y = at::empty_like(qi, qi.options().dtype(half ? at::kHalf : at::kFloat));
+  check_status(catchq_dequantize(qi.data_ptr(), bits_of(qi), y.data_ptr(), half ? CATCHQ_F16 : CATCHQ_F32,
+                                 qi.numel(), (int)position, (float)scale, current_stream()),
+               "torch_mlu::dequantize");
+  return y;
+}
+
+// ------------------------------------------------------------------------------------------------
+// integer building blocks
+// ------------------------------------------------------------------------------------------------
+
+struct EpiArgs {
+  int64_t exp2 = 0;
+  c10::optional<Tensor> chan_div, bias, resid;
+  int64_t act = 0;
+  bool want_y = true, y_half = false, want_acc = false;
+  int64_t q_bitwidth = 0, q_position = 0;
+  double q_scale = 1.0;
+};
+
+struct EpiOut {
+  Tensor y, acc, q;
+};
+
+Tensor as_f32_vec(const c10::optional<Tensor> &t, int64_t n, const char *name) {
+  if (!t.has_value() || !t->defined()) return Tensor();
+  TORCH_CHECK(t->numel() == n, name, ": expected ", n, " elements, got ", t->numel());
+  return t->to(at::kFloat).contiguous();
+}
+
+// fills a catchq_epilogue_t; `keep` holds the temporaries alive until the launch is enqueued
+EpiOut prepare_epilogue(const EpiArgs &a, at::IntArrayRef out_shape, int64_t co, const at::TensorOptions &opts,
+                        catchq_epilogue_t *e, std::vector<Tensor> *keep) {
+  EpiOut o;
+  std::memset(e, 0, sizeof(*e));
+  TORCH_CHECK(a.exp2 >= -126 && a.exp2 <= 126, "position sum out of range");
+  e->exp2 = (int)a.exp2;
+  Tensor cd = as_f32_vec(a.chan_div, co, "chan_div"), bs = as_f32_vec(a.bias, co, "bias");
+  if (cd.defined()) { e->chan_div = cd.data_ptr<float>(); keep->push_back(cd); }
+  if (bs.defined()) { e->bias = bs.data_ptr<float>(); keep->push_back(bs); }
+  if (a.resid.has_value() && a.resid->defined()) {
+    TORCH_CHECK(a.resid->sizes() == out_shape && a.resid->scalar_type() == at::kFloat && a.resid->is_contiguous(),
+                "resid must be a contiguous fp32 tensor of the output's shape");
+    e->resid = a.resid->data_ptr<float>();
+  }
+  e->act = (int)a.act;
+  if (a.want_y) {
+    o.y = at::empty(out_shape, opts.dtype(a.y_half ? at::kHalf : at::kFloat));
+    e->y = o.y.data_ptr();
+    e->y_dtype = a.y_half ? CATCHQ_F16 : CATCHQ_F32;
+  }
+  if (a.want_acc) {
+    o.acc = at::empty(out_shape, opts.dtype(at::kInt));
+    e->acc_out = o.acc.data_ptr<int32_t>();
+  }
+  if (a.q_bitwidth != 0) {
+    TORCH_CHECK(a.q_bitwidth == 8 || a.q_bitwidth == 16, "bitwidth not support");
+    o.q = at::empty(out_shape, opts.dtype(int_type(a.q_bitwidth)));
+    e->q = o.q.data_ptr();
+    e->q_bitwidth = (int)a.q_bitwidth;
+    e->q_position = (int)a.q_position;
+    e->q_scale = (float)a.q_scale;
+  }
+  return o;
+}
+
+// qx [N,H,W,Ci] int8/int16 contiguous, qw [Co,kh,kw,Ci/g] contiguous -> outputs [N,Ho,Wo,Co]
+EpiOut qconv2d_impl(const Tensor &qx, const Tensor &qw, at::IntArrayRef padding, at::IntArrayRef stride,
+                    at::IntArrayRef dilation, int64_t groups, const EpiArgs &a) {
+  TORCH_CHECK(qx.dim() == 4 && qw.dim() == 4 && qx.is_contiguous() && qw.is_contiguous(),
+              "qconv2d expects contiguous NHWC activations and [Co,kh,kw,Ci/g] weights");
+  TORCH_CHECK(padding.size() == 2 && stride.size() == 2 && dilation.size() == 2, "2-d conv parameters expected");
+  TORCH_CHECK(groups > 0 && qx.size(3) == qw.size(3) * groups, "channel mismatch: input ", qx.size(3),
+              ", weight ", qw.size(3), " x groups ", groups);
+  catchq_conv_desc_t d;
+  d.n = (int)qx.size(0); d.h = (int)qx.size(1); d.w = (int)qx.size(2); d.ci = (int)qx.size(3);
+  d.co = (int)qw.size(0); d.kh = (int)qw.size(1); d.kw = (int)qw.size(2);
+  d.pad_h = (int)padding[0]; d.pad_w = (int)padding[1];
+  d.stride_h = (int)stride[0]; d.stride_w = (int)stride[1];
+  d.dil_h = (int)dilation[0]; d.dil_w = (int)dilation[1];
+  d.groups = (int)groups;
+  TORCH_CHECK(d.stride_h > 0 && d.stride_w > 0, "non-positive stride is not supported");
+  TORCH_CHECK(d.pad_h >= 0 && d.pad_w >= 0, "negative padding is not supported");
+  const int ho = catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h);
+  const int wo = catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w);
+  TORCH_CHECK(ho > 0 && wo > 0, "Calculated output size is too small");
+  catchq_epilogue_t e;
+  std::vector<Tensor> keep;
+  EpiOut o = prepare_epilogue(a, {d.n, ho, wo, d.co}, d.co, qx.options(), &e, &keep);
+  check_status(catchq_conv2d_nhwc(qx.data_ptr(), bits_of(qx), qw.data_ptr(), bits_of(qw), &d, &e, current_stream()),
+               "torch_mlu::conv2d");
+  return o;
+}
+
+EpiOut qlinear_impl(const Tensor &qx, const Tensor &qw, const EpiArgs &a) {
+  TORCH_CHECK(qx.dim() == 2 && qw.dim() == 2 && qx.is_contiguous() && qw.is_contiguous(), "dimension not support");
+  TORCH_CHECK(qx.size(1) == qw.size(1), "size mismatch: ", qx.sizes(), " x ", qw.sizes(), "^T");
+  catchq_epilogue_t e;
+  std::vector<Tensor> keep;
+  EpiOut o = prepare_epilogue(a, {qx.size(0), qw.size(0)}, qw.size(0), qx.options(), &e, &keep);
+  check_status(catchq_gemm_nt(qx.data_ptr(), bits_of(qx), qw.data_ptr(), bits_of(qw), qx.size(0), qw.size(0),
+                              qx.size(1), &e, current_stream()),
+               "torch_mlu::linear");
+  return o;
+}
+
+EpiArgs make_args(int64_t exp2, const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias,
+                  const c10::optional<Tensor> &resid, int64_t act, bool want_y, bool y_half, bool want_acc,
+                  int64_t q_bitwidth, int64_t q_position, double q_scale) {
+  EpiArgs a;
+  a.exp2 = exp2; a.chan_div = chan_div; a.bias = bias; a.resid = resid; a.act = act;
+  a.want_y = want_y; a.y_half = y_half; a.want_acc = want_acc;
+  a.q_bitwidth = q_bitwidth; a.q_position = q_position; a.q_scale = q_scale;
+  return a;
+}
+
+std::tuple<Tensor, Tensor, Tensor> tup(const EpiOut &o) { return std::make_tuple(o.y, o.q, o.acc); }
+
+std::tuple<Tensor, Tensor, Tensor> qconv2d_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
+                                              const c10::optional<Tensor> &chan_div,
+                                              const c10::optional<Tensor> &bias,
+                                              const c10::optional<Tensor> &resid, at::IntArrayRef padding,
+                                              at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups,
+                                              int64_t act, bool want_y, bool y_half, bool want_acc,
+                                              int64_t q_bitwidth, int64_t q_position, double q_scale) {
+  c10::DeviceGuard guard(qx.device());
+  return tup(qconv2d_impl(qx, qw, padding, stride, dilation, groups,
+                          make_args(exp2, chan_div, bias, resid, act, want_y, y_half, want_acc, q_bitwidth,
+                                    q_position, q_scale)));
+}
+
+std::tuple<Tensor, Tensor, Tensor> qlinear_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
+                                              const c10::optional<Tensor> &chan_div,
+                                              const c10::optional<Tensor> &bias, int64_t act, bool want_y,
+                                              bool y_half, bool want_acc, int64_t q_bitwidth,
+                                              int64_t q_position, double q_scale) {
+  c10::DeviceGuard guard(qx.device());
+  return tup(qlinear_impl(qx, qw,
+                          make_args(exp2, chan_div, bias, c10::nullopt, act, want_y, y_half, want_acc, q_bitwidth,
+                                    q_position, q_scale)));
+}
+
+// cnnl_mm(self, self_position, other, other_position, false, true): fp32 output
+Tensor mm_q_op(const Tensor &a, int64_t pos_a, const Tensor &b, int64_t pos_b) {
+  c10::DeviceGuard guard(a.device());
+  EpiArgs args;
+  args.exp2 = pos_a + pos_b;
+  return qlinear_impl(a.contiguous(), b.contiguous(), args).y;
+}
+
+// fp NCHW (or channels-last) activations -> NHWC integer tensor [N,H,W,cpad]
+Tensor quantize_to_nhwc(const Tensor &x, int bw, int pos, int64_t cpad) {
+  const int dt = fp_dtype(x, "quantify only support input float/half");
+  TORCH_CHECK(x.dim() == 4, "a 4-d activation tensor is expected");
+  const int64_t n = x.size(0), c = x.size(1), h = x.size(2), w = x.size(3);
+  if (cpad < c) cpad = c;
+  Tensor q = at::empty({n, h, w, cpad}, x.options().dtype(int_type(bw)));
+  if (cpad == c && x.is_contiguous(at::MemoryFormat::ChannelsLast)) {
+    check_status(catchq_quantize(x.data_ptr(), dt, q.data_ptr(), bw, x.numel(), pos, 1.0f, current_stream()),
+                 "torch_mlu::quantize");
+    return q;
+  }
+  Tensor xc = x.is_contiguous() ? x : x.contiguous();
+  check_status(catchq_quantize_nchw_to_nhwc(xc.data_ptr(), dt, q.data_ptr(), bw, (int)n, (int)c, (int)h, (int)w,
+                                            (int)cpad, pos, 1.0f, current_stream()),
+               "torch_mlu::quantize");
+  return q;
+}
+
+Tensor quantize_nhwc_op(const Tensor &x, int64_t bitwidth, int64_t position, int64_t cpad) {
+  c10::DeviceGuard guard(x.device());
+  return quantize_to_nhwc(x, (int)bitwidth, (int)position, cpad);
+}
+
+// ------------------------------------------------------------------------------------------------
+// the two reference ops
+// ------------------------------------------------------------------------------------------------
+
+// Decoded q_scale / q_mode plus the quantized weight, kept per weight tensor so that steady-state
+// calls neither copy the parameters to the host nor re-quantize the weight (the reference does both
+// on every call: quantify_conv_forward.cpp:74-75,100-101,114,119-120).  An entry is valid while the
+// same tensor objects, at the same versions, are passed again.
+struct Prepared {
+  c10::weak_intrusive_ptr<c10::TensorImpl> w_impl, s_impl, m_impl;
+  uint32_t w_ver = 0, s_ver = 0, m_ver = 0;
+  const void *w_ptr = nullptr;
+  int bw_x = 8, bw_w = 8, pos_x = 0, pos_w = 0;
+  bool per_channel = false;
+  Tensor qw;         // conv: [Co,kh,kw,Ci/g]; linear: [N,K]
+  Tensor new_scale;  // device fp32 [Co] when per_channel
+  Prepared() : w_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)),
+               s_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)),
+               m_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)) {}
+};
+
+uint32_t version_of(const Tensor &t) {
+  // inference tensors carry no version counter
+  return t.is_inference() ? 0u : t.unsafeGetTensorImpl()->version_counter().current_version();
+}
+
+bool cache_enabled() {
+  static const bool on = [] {
+    const char *v = std::getenv("CATCHQ_WEIGHT_CACHE");
+    return !(v && v[0] == '0');
+  }();
+  return on;
+}
+
+std::mutex g_cache_mutex;
+std::unordered_map<const c10::TensorImpl *, std::shared_ptr<Prepared>> g_cache;
+
+bool still_valid(const Prepared &p, const Tensor &w, const Tensor &s, const Tensor &m) {
+  auto same = [](const c10::weak_intrusive_ptr<c10::TensorImpl> &weak, const Tensor &t, uint32_t ver) {
+    return !weak.expired() && weak._unsafe_get_target() == t.unsafeGetTensorImpl() && version_of(t) == ver;
+  };
+  return same(p.w_impl, w, p.w_ver) && same(p.s_impl, s, p.s_ver) && same(p.m_impl, m, p.m_ver) &&
+         p.w_ptr == w.data_ptr();
+}
+
+c10::weak_intrusive_ptr<c10::TensorImpl> weak_of(const Tensor &t) {
+  return c10::weak_intrusive_ptr<c10::TensorImpl>(t.getIntrusivePtr());
+}
+
+// Decode the two q-param encodings and quantize the weight (dense, dim 0 slowest).
+std::shared_ptr<Prepared> prepare(const Tensor &w_dense, const Tensor &weight, const Tensor &q_scale,
+                                  const Tensor &q_mode) {
+  auto p = std::make_shared<Prepared>();
+  Tensor s_host = q_scale.to(at::kCPU).to(at::kFloat).contiguous();
+  Tensor m_host = q_mode.to(at::kCPU).to(at::kInt).contiguous();
+  const float *s = s_host.data_ptr<float>();
+  const int32_t *m = m_host.data_ptr<int32_t>();
+  if (m_host.numel() == 1) {
+    // CNML-compatible encoding: q_mode in {1:int8, 2:int16, 3:int8 per-channel, 4:int16 per-channel},
+    // q_scale = [s_in, s_w | 0, s_c0 ...]   (quantify_conv_forward.cpp:77-131; linear.cpp:81-144)
+    const int mode = m[0];
+    TORCH_CHECK(mode >= 1 && mode <= 4, "quantized_mode must be 1, 2, 3 or 4, got ", mode);
+    const int bw = (mode == 1 || mode == 3) ? 8 : 16;
+    p->bw_x = p->bw_w = bw;
+    p->per_channel = mode > 2;
+    TORCH_CHECK(s_host.numel() >= 2, "q_scale needs at least [input_scale, weight_scale]");
+    check_status(catchq_pos_from_scale(bw, s[0], &p->pos_x), "input position");
+    if (!p->per_channel) {
+      check_status(catchq_pos_from_scale(bw, s[1], &p->pos_w), "weight position");
+      p->qw = quantize_op(w_dense, bw, p->pos_w, 1.0);
+    } else {
+      const int64_t co = w_dense.size(0);
+      TORCH_CHECK(s_host.numel() == 2 + co, "per-channel q_scale must hold 2 + ", co, " values, got ", s_host.numel());
+      PerChannel pc = per_channel_params(s + 2, co, bw, w_dense.options());
+      p->pos_w = pc.new_pos;
+      p->new_scale = pc.new_scale;
+      p->qw = quantize_weight_per_channel(w_dense, pc, bw);
+    }
+  } else {
+    // CNNL encoding: q_scale = [bitwidth_in, bitwidth_w], q_mode = [pos_in, pos_w]
+    // (quantify_conv_forward.cpp:132-145; linear.cpp:145-166)
+    TORCH_CHECK(m_host.numel() == 2 && s_host.numel() == 2, "q_scale/q_mode must hold two values each");
+    p->bw_x = (int)s[0];
+    p->bw_w = (int)s[1];
+    TORCH_CHECK((p->bw_x == 8 || p->bw_x == 16) && (p->bw_w == 8 || p->bw_w == 16), "bitwidth not support");
+    p->pos_x = m[0];
+    p->pos_w = m[1];
+    p->qw = quantize_op(w_dense, p->bw_w, p->pos_w, 1.0);
+  }
+  p->w_impl = weak_of(weight); p->s_impl = weak_of(q_scale); p->m_impl = weak_of(q_mode);
+  p->w_ver = version_of(weight); p->s_ver = version_of(q_scale); p->m_ver = version_of(q_mode);
+  p->w_ptr = weight.data_ptr();
+  return p;
+}
+
+template <typename MakeDense>
+std::shared_ptr<Prepared> prepared_for(const Tensor &weight, const Tensor &q_scale, const Tensor &q_mode,
+                                       MakeDense make_dense) {
+  const bool use_cache = cache_enabled();
+  const c10::TensorImpl *key = weight.unsafeGetTensorImpl();
+  if (use_cache) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_cache.find(key);
+    if (it != g_cache.end()) {
+      if (still_valid(*it->second, weight, q_scale, q_mode)) return it->second;
+      g_cache.erase(it);
+    }
+  }
+  auto p = prepare(make_dense(weight), weight, q_scale, q_mode);
+  if (use_cache) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    if (g_cache.size() > 4096) {  // drop entries whose weight is gone
+      for (auto it = g_cache.begin(); it != g_cache.end();)
+        it = it->second->w_impl.expired() ? g_cache.erase(it) : std::next(it);
+    }
+    g_cache[key] = p;
+  }
+  return p;
+}
+
+void clear_cache_op() {
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  g_cache.clear();
+}
+
+Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, at::IntArrayRef padding,
+                 at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups, const Tensor &q_scale,
+                 const Tensor &q_mode) {
+  TORCH_CHECK(input.dim() > 2, "Input's dim must greater than 2!");
+  TORCH_CHECK(input.dim() == 4 && weight.dim() == 4, "torch_mlu::conv2d expects 4-d input and weight");
+  const bool half = fp_dtype(input, "quantify only support input float/half") == CATCHQ_F16;
+  c10::DeviceGuard guard(input.device());
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w) {
+    // the memory of a channels-last [Co,Ci/g,kh,kw] tensor is [Co][kh][kw][Ci/g]
+    return w.contiguous(at::MemoryFormat::ChannelsLast);
+  });
+  Tensor qx = quantize_to_nhwc(input, prep->bw_x, prep->pos_x, input.size(1));
+  Tensor qw = prep->qw.permute({0, 2, 3, 1});  // view of the same memory as [Co,kh,kw,Ci/g], contiguous
+  EpiArgs a;
+  a.exp2 = prep->pos_x + prep->pos_w;
+  if (prep->per_channel) a.chan_div = prep->new_scale;
+  if (has_bias(bias)) a.bias = bias;
+  a.y_half = half;
+  EpiOut o = qconv2d_impl(qx, qw, padding, stride, dilation, groups, a);
+  return o.y.permute({0, 3, 1, 2});  // logical NCHW over channels-last memory, like the reference
+}
+
+Tensor linear_op(const Tensor &input, const Tensor &weight, const Tensor &bias, const Tensor &q_scale,
+                 const Tensor &q_mode) {
+  TORCH_CHECK(weight.dim() == 2, "we only support the  dim of weight is 2");
+  fp_dtype(input, "quantify only support input float/half");
+  TORCH_CHECK(input.dim() >= 1 && input.size(-1) == weight.size(1), "size mismatch: input ", input.sizes(),
+              ", weight ", weight.sizes());
+  c10::DeviceGuard guard(input.device());
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w) { return w.contiguous(); });
+  Tensor x2 = input.contiguous().view({-1, input.size(-1)});
+  Tensor qx = quantize_op(x2, prep->bw_x, prep->pos_x, 1.0);
+  EpiArgs a;  // output is fp32 whatever the input type (operators/cnnl/matmul.cpp:72-74)
+  a.exp2 = prep->pos_x + prep->pos_w;
+  if (prep->per_channel) a.chan_div = prep->new_scale;
+  if (has_bias(bias)) a.bias = bias;
+  EpiOut o = qlinear_impl(qx, prep->qw, a);
+  std::vector<int64_t> shape(input.sizes().begin(), input.sizes().end() - 1);
+  shape.push_back(weight.size(0));
+  return o.y.view(shape);
+}
+
+std::string conv2d_route_op(int64_t x_bits, int64_t w_bits, at::IntArrayRef in_nhwc, at::IntArrayRef w_ohwi,
+                            at::IntArrayRef padding, at::IntArrayRef stride, at::IntArrayRef dilation,
+                            int64_t groups) {
+  catchq_conv_desc_t d = {(int)in_nhwc[0], (int)in_nhwc[1], (int)in_nhwc[2], (int)in_nhwc[3], (int)w_ohwi[0],
+                          (int)w_ohwi[1], (int)w_ohwi[2], (int)padding[0], (int)padding[1], (int)stride[0],
+                          (int)stride[1], (int)dilation[0], (int)dilation[1], (int)groups};
+  return catchq_conv2d_route((int)x_bits, (int)w_bits, &d);
+}
+
+}  // namespace
+
+TORCH_LIBRARY(torch_mlu, m) {
+  m.def("conv2d(Tensor input, Tensor weight, Tensor bias, int[] padding, int[] stride, int[] dilation, "
+        "int groups, Tensor q_scale, Tensor q_mode) -> Tensor");
+  m.def("linear(Tensor input, Tensor weight, Tensor bias, Tensor q_scale, Tensor q_mode) -> Tensor");
+  m.def("quantize(Tensor x, int bitwidth, int position, float scale=1.0) -> Tensor");
+  m.def("quantize_dev(Tensor x, int bitwidth, Tensor position) -> Tensor");
+  m.def("quantize_nhwc(Tensor x, int bitwidth, int position, int cpad=0) -> Tensor");
+  m.def("quantize_param(Tensor x, int bitwidth, int mode) -> (Tensor, Tensor, Tensor)");
+  m.def("quantize_per_channel(Tensor w, Tensor scales, int bitwidth) -> (Tensor, Tensor, Tensor)");
+  m.def("dequantize(Tensor q, int position, float scale=1.0, bool half=False) -> Tensor");
+  m.def("mm_q(Tensor a, int pos_a, Tensor b, int pos_b) -> Tensor");
+  m.def("qconv2d(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, Tensor? resid, "
+        "int[] padding, int[] stride, int[] dilation, int groups, int act=0, bool want_y=True, "
+        "bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0) "
+        "-> (Tensor, Tensor, Tensor)");
+  m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
+        "bool want_y=True, bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, "
+        "float q_scale=1.0) -> (Tensor, Tensor, Tensor)");
+  m.def("clear_weight_cache() -> ()", &clear_cache_op);
+  m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
+        "int[] dilation, int groups) -> str", &conv2d_route_op);
+}
+
+TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA key
+  m.impl("conv2d", &conv2d_op);
+  m.impl("linear", &linear_op);
+  m.impl("quantize", &quantize_op);
+  m.impl("quantize_dev", &quantize_dev_op);
+  m.impl("quantize_nhwc", &quantize_nhwc_op);
+  m.impl("quantize_param", &quantize_param_op);
+  m.impl("quantize_per_channel", &quantize_per_channel_op);
+  m.impl("dequantize", &dequantize_op);
+  m.impl("mm_q", &mm_q_op);
+  m.impl("qconv2d", &qconv2d_op);
+  m.impl("qlinear", &qlinear_op);
+}

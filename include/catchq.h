@@ -1,0 +1,168 @@
+/*
+ * catchq.h -- C ABI of the MI355X (gfx950) fixed-point quantized-inference kernels.
+ *
+ * Drop-in boundary for the quantized hot path of Cambricon/catch (torch_mlu): each
+ * entry point replaces one vendor-library call (or one group of small tensor ops)
+ * that the reference's op wrappers make.  Citations are file:line in the
+ * reference tree, below torch_mlu/csrc/aten/ unless a longer path is given.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every device buffer (inputs, outputs,
+ *     workspace) is owned by the caller; nothing here allocates or frees;
+ *   - all device entry points are asynchronous on `stream` (a hipStream_t passed
+ *     as void*; NULL = the null stream) and keep no mutable global state;
+ *   - the return value is a status (0 = CATCHQ_OK); no exception crosses the
+ *     boundary; catchq_status_string() names a status;
+ *   - activations are NHWC, convolution weights [Co][kh][kw][Ci/groups]
+ *     (= the memory of a channels-last [Co,Ci/g,kh,kw] tensor), GEMM operands
+ *     row-major with K contiguous (A [M,K], B [N,K]).
+ */
+#ifndef CATCHQ_H_
+#define CATCHQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *catchq_stream_t;
+
+enum {
+  CATCHQ_OK = 0,
+  CATCHQ_ERR_ARG = 1,         /* null pointer, negative size, bad enum */
+  CATCHQ_ERR_DTYPE = 2,       /* "quantify only support input float/half" (operators/cnnl/internal/quantify.cpp:73-74) */
+  CATCHQ_ERR_BITWIDTH = 3,    /* "bitwidth not support" (operators/cnnl/internal/quantify.cpp:63) */
+  CATCHQ_ERR_SHAPE = 4,       /* inconsistent shapes (groups, output extent <= 0, ...) */
+  CATCHQ_ERR_LAUNCH = 5,      /* the HIP runtime refused the launch */
+  CATCHQ_ERR_UNSUPPORTED = 6  /* combination not implemented */
+};
+
+enum { CATCHQ_F32 = 0, CATCHQ_F16 = 1 };
+enum { CATCHQ_ACT_NONE = 0, CATCHQ_ACT_RELU = 1, CATCHQ_ACT_RELU6 = 2 };
+/* cnnlQuantizeMode_t values used by the reference (operators/cnnl/internal/quantize_param.cpp:70-78) */
+enum { CATCHQ_QUANTIZE_POSITION = 0, CATCHQ_QUANTIZE_POSITION_SCALE = 1, CATCHQ_QUANTIZE_POSITION_SCALE_OFFSET = 2 };
+
+int catchq_version(void);
+const char *catchq_status_string(int status);
+
+/* ------------------------------------------------------------------ host q-param math */
+
+/* get_pos_from_scale_data(bitwidth, scale_data)            cnnl/cnnl_util.cpp:337-347 */
+int catchq_pos_from_scale(int bitwidth, float scale, int *position);
+
+/* setQuantizedParams(scale, qmode, ...)                    torch_mlu/csrc/jit/utils/utils.cpp:81-105
+ * position, fractional scale 2^pos*qmax/absmax and scale_factor 2^pos/scale_. */
+int catchq_quant_params(int bitwidth, float scale, int *position, float *scale_frac, float *scale_factor);
+
+/* the parameter part of cnnl_quantify_per_channel          operators/cnnl/quantify.cpp:55-98
+ * scales[co] (= qmax/absmax_c) -> shared new_position, new_scale[co], scale_factor[co] (host arrays). */
+int catchq_per_channel_params(int bitwidth, const float *scales, int co, int *new_position,
+                              float *new_scale, float *scale_factor);
+
+/* ------------------------------------------------------------------ quantize / dequantize */
+
+/* cnnl_quantify_offline_internal(input, bitwidth, int position) -> cnnlQuantizeV1
+ *                                                          operators/cnnl/internal/quantify.cpp:69-101
+ * q[i] = sat(rne(x[i] * scale * 2^-position)); x fp32/fp16, q int8 / int16 / int32 (bitwidth 8/16/31).
+ * The reference's eager path passes scale = 1. */
+int catchq_quantize(const void *x, int x_dtype, void *q, int bitwidth, int64_t n, int position,
+                    float scale, catchq_stream_t stream);
+
+/* cnnl_quantify_offline_internal(input, bitwidth, Tensor position) -> cnnlQuantizeV2
+ *                                                          operators/cnnl/internal/quantify.cpp:103-137
+ * same, position (and optionally scale) read from device memory: no host sync. scale_dev may be NULL (=1). */
+int catchq_quantize_devpos(const void *x, int x_dtype, void *q, int bitwidth, int64_t n,
+                           const int32_t *position_dev, const float *scale_dev, catchq_stream_t stream);
+
+/* cnnl_contiguous(input, ChannelsLast) followed by cnnl_quantify_offline
+ *                                                          operators/cnnl/quantify_conv_forward.cpp:62-63,97
+ * x [N,C,H,W] contiguous -> q [N,H,W,cpad] (channels C..cpad-1 zero), in one pass. */
+int catchq_quantize_nchw_to_nhwc(const void *x, int x_dtype, void *q, int bitwidth, int n, int c, int h,
+                                 int w, int cpad, int position, float scale, catchq_stream_t stream);
+
+/* cnnlGetQuantizeParamWorkspaceSize + cnnl_quantize_param -> cnnlQuantizeParam
+ *                                                          operators/cnnl/internal/quantize_param.cpp:39-96
+ * max-abs reduction, then position (mode 0), + scale (1), + offset = 0 (2) written to device memory.
+ * absmax_dev / scale_dev / offset_dev may be NULL.  The vendor formula is not in the reference tree;
+ * defined as position = floor(log2(absmax)) - (bitwidth-2), scale = 2^position*qmax/absmax. */
+int catchq_quantize_param_workspace_size(int64_t n, size_t *bytes);
+int catchq_quantize_param(const void *x, int x_dtype, int64_t n, int bitwidth, int mode, void *workspace,
+                          size_t workspace_bytes, float *absmax_dev, int32_t *position_dev,
+                          float *scale_dev, float *offset_dev, catchq_stream_t stream);
+
+/* the elementwise part of cnnl_quantify_per_channel        operators/cnnl/quantify.cpp:100-112
+ * q[c, i] = sat(rne(w[c, i] / scale_factor[c])), w [co, inner] fp32/fp16, scale_factor on the device. */
+int catchq_quantize_per_channel(const void *w, int w_dtype, void *q, int bitwidth, int co, int64_t inner,
+                                const float *scale_factor_dev, catchq_stream_t stream);
+
+/* explicit form of the dequantization the reference leaves to the vendor conv/matmul descriptors
+ * (cnnl/cnnlTensorDescriptors.cpp:175-184) : y[i] = q[i] * 2^position / scale; q int8/int16/int32
+ * (bits 8/16/32), y fp32/fp16. */
+int catchq_dequantize(const void *q, int bits, void *y, int y_dtype, int64_t n, int position, float scale,
+                      catchq_stream_t stream);
+
+/* ------------------------------------------------------------------ integer contraction + epilogue */
+
+/* What happens to each integer sum acc[r][c] (r = output row / pixel, c = output channel):
+ *   v = float(acc) * 2^exp2                 positions of both operands (matmul_internal.cpp:93-96;
+ *                                           convolution_forward_internal.cpp:85-88)
+ *   v = v / chan_div[c]   if chan_div       "output / new_scale" (quantify_conv_forward.cpp:127; linear.cpp:56)
+ *   v = v + bias[c]       if bias           (quantify_conv_forward.cpp:129; linear.cpp:57-59)
+ *   v = v + resid[r][c]   if resid          residual branch of the caller's graph (fp32)
+ *   v = act(v)
+ * then any of: y[r][c] = v (fp32, or fp16 by one RNE conversion); acc_out[r][c] = acc;
+ * q[r][c] = sat(rne(v * q_scale * 2^-q_position)) for the next layer (q_bitwidth 8/16).
+ * All fp32, no fused multiply-add, true division. */
+typedef struct catchq_epilogue {
+  int exp2;
+  const float *chan_div; /* device [co] or NULL */
+  const float *bias;     /* device [co] or NULL */
+  const float *resid;    /* device [rows, co] fp32 or NULL */
+  int act;               /* CATCHQ_ACT_* */
+  void *y;               /* device [rows, co] or NULL */
+  int y_dtype;           /* CATCHQ_F32 / CATCHQ_F16 */
+  int32_t *acc_out;      /* device [rows, co] or NULL */
+  void *q;               /* device [rows, co] int8/int16 or NULL */
+  int q_bitwidth;
+  int q_position;
+  float q_scale;
+} catchq_epilogue_t;
+
+/* cnnl_mm(self, self_position, other, other_position, false, true) -> cnnlMatMul
+ *                                                          operators/cnnl/matmul.cpp:69-75;
+ *                                                          operators/cnnl/internal/matmul_internal.cpp:46-120
+ * acc[m][n] = sum_k a[m][k] * b[n][k]; a [M,K], b [N,K]; a_bits/b_bits in {8,16}.
+ * int8 x int8 and int16 x int8 accumulate in int32; int16 x int16 in int64 (acc_out unsupported there). */
+int catchq_gemm_nt(const void *a, int a_bits, const void *b, int b_bits, int64_t m, int64_t n, int64_t k,
+                   const catchq_epilogue_t *epilogue, catchq_stream_t stream);
+
+typedef struct catchq_conv_desc {
+  int n, h, w, ci;  /* input  [n,h,w,ci] */
+  int co, kh, kw;   /* weight [co,kh,kw,ci/groups] */
+  int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, groups;
+} catchq_conv_desc_t;
+
+/* conv_output_size()                                       operators/cnnl/internal/convolution_forward_internal.cpp:40-54 */
+int catchq_conv_out_size(int in, int k, int pad, int stride, int dil);
+
+/* cnnl_quantify_convolution_internal -> cnnlConvolutionForward
+ *                                                          operators/cnnl/internal/convolution_forward_internal.cpp:56-180
+ * integer cross-correlation with zero padding and groups; the output rows are the pixels
+ * (n,ho,wo) in that order, so y/acc_out/q/resid are NHWC [n,ho,wo,co].
+ * Depthwise layers (is_depthwise_conv, operators/cnnl/convolution_overrideable.cpp:41-54) run a
+ * stencil kernel, dense int8 layers with ci % 16 == 0 an MFMA implicit GEMM, everything else a
+ * direct kernel; the arithmetic is the same in all of them. */
+int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int w_bits, const catchq_conv_desc_t *desc,
+                       const catchq_epilogue_t *epilogue, catchq_stream_t stream);
+
+/* Name of the kernel family catchq_conv2d_nhwc / catchq_gemm_nt would use ("mfma", "direct",
+ * "depthwise", ...): for logs and tests; not part of the arithmetic. */
+const char *catchq_conv2d_route(int x_bits, int w_bits, const catchq_conv_desc_t *desc);
+const char *catchq_gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CATCHQ_H_ */

@@ -1,0 +1,133 @@
+"""Thin test-side wrappers: call the C ABI of include/catchq.h on torch device tensors."""
+import ctypes
+
+import numpy as np
+import torch
+
+from catch_amd import _native
+from catch_amd._native import ConvDesc, Epilogue, check
+
+F32, F16 = 0, 1
+_INT = {8: torch.int8, 16: torch.int16, 31: torch.int32, 32: torch.int32}
+
+
+def lib():
+    return _native.kernel_lib()
+
+
+def stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def dt(t):
+    return F16 if t.dtype == torch.float16 else F32
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def quantize(x, bw, pos, scale=1.0):
+    q = torch.empty(x.shape, dtype=_INT[bw], device=x.device)
+    check(lib().catchq_quantize(ptr(x), dt(x), ptr(q), bw, x.numel(), pos, scale, stream()))
+    return q
+
+
+def quantize_devpos(x, bw, pos_t, scale_t=None):
+    q = torch.empty(x.shape, dtype=_INT[bw], device=x.device)
+    check(lib().catchq_quantize_devpos(ptr(x), dt(x), ptr(q), bw, x.numel(), ptr(pos_t), ptr(scale_t), stream()))
+    return q
+
+
+def quantize_nchw_to_nhwc(x, bw, pos, scale=1.0, cpad=None):
+    n, c, h, w = x.shape
+    cpad = cpad or c
+    q = torch.empty((n, h, w, cpad), dtype=_INT[bw], device=x.device)
+    check(lib().catchq_quantize_nchw_to_nhwc(ptr(x), dt(x), ptr(q), bw, n, c, h, w, cpad, pos, scale, stream()))
+    return q
+
+
+def quantize_param(x, bw, mode=2):
+    sz = ctypes.c_size_t()
+    check(lib().catchq_quantize_param_workspace_size(x.numel(), ctypes.byref(sz)))
+    ws = torch.empty(max(sz.value, 4), dtype=torch.int8, device=x.device)
+    absmax = torch.empty(1, dtype=torch.float32, device=x.device)
+    pos = torch.empty(1, dtype=torch.int32, device=x.device)
+    scale = torch.ones(1, dtype=torch.float32, device=x.device)
+    off = torch.ones(1, dtype=torch.float32, device=x.device)
+    check(lib().catchq_quantize_param(ptr(x), dt(x), x.numel(), bw, mode, ptr(ws), sz.value, ptr(absmax), ptr(pos),
+                                      ptr(scale), ptr(off), stream()))
+    return absmax, pos, scale, off
+
+
+def quantize_per_channel(w, bw, sf):
+    q = torch.empty(w.shape, dtype=_INT[bw], device=w.device)
+    co = w.shape[0]
+    check(lib().catchq_quantize_per_channel(ptr(w), dt(w), ptr(q), bw, co, w.numel() // max(co, 1), ptr(sf), stream()))
+    return q
+
+
+def dequantize(q, pos, scale=1.0, half=False):
+    bits = q.element_size() * 8
+    y = torch.empty(q.shape, dtype=torch.float16 if half else torch.float32, device=q.device)
+    check(lib().catchq_dequantize(ptr(q), bits, ptr(y), F16 if half else F32, q.numel(), pos, scale, stream()))
+    return y
+
+
+def _epilogue(shape, device, exp2, chan_div, bias, resid, act, y_dtype, want_acc, q_bw, q_pos, q_scale):
+    e = Epilogue()
+    out = {}
+    e.exp2 = exp2
+    e.chan_div, e.bias, e.resid = ptr(chan_div), ptr(bias), ptr(resid)
+    e.act = act
+    if y_dtype is not None:
+        out["y"] = torch.empty(shape, dtype=y_dtype, device=device)
+        e.y, e.y_dtype = ptr(out["y"]), (F16 if y_dtype == torch.float16 else F32)
+    if want_acc:
+        out["acc"] = torch.empty(shape, dtype=torch.int32, device=device)
+        e.acc_out = ptr(out["acc"])
+    if q_bw:
+        out["q"] = torch.empty(shape, dtype=_INT[q_bw], device=device)
+        e.q, e.q_bitwidth, e.q_position, e.q_scale = ptr(out["q"]), q_bw, q_pos, q_scale
+    return e, out
+
+
+def gemm_nt(a, b, exp2=0, chan_div=None, bias=None, act=0, y_dtype=torch.float32, want_acc=True, q_bw=0,
+            q_pos=0, q_scale=1.0):
+    m, k = a.shape
+    n = b.shape[0]
+    e, out = _epilogue((m, n), a.device, exp2, chan_div, bias, None, act, y_dtype, want_acc, q_bw, q_pos, q_scale)
+    check(lib().catchq_gemm_nt(ptr(a), a.element_size() * 8, ptr(b), b.element_size() * 8, m, n, k,
+                               ctypes.byref(e), stream()))
+    return out
+
+
+def conv_desc(x_shape, w_shape, padding, stride, dilation, groups):
+    n, h, w, ci = x_shape
+    co, kh, kw, _ = w_shape
+    return ConvDesc(n, h, w, ci, co, kh, kw, padding[0], padding[1], stride[0], stride[1], dilation[0],
+                    dilation[1], groups)
+
+
+def conv2d_nhwc(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1, exp2=0, chan_div=None, bias=None,
+                resid=None, act=0, y_dtype=torch.float32, want_acc=True, q_bw=0, q_pos=0, q_scale=1.0):
+    d = conv_desc(x.shape, w.shape, padding, stride, dilation, groups)
+    ho = lib().catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h)
+    wo = lib().catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w)
+    e, out = _epilogue((d.n, ho, wo, d.co), x.device, exp2, chan_div, bias, resid, act, y_dtype, want_acc, q_bw,
+                       q_pos, q_scale)
+    check(lib().catchq_conv2d_nhwc(ptr(x), x.element_size() * 8, ptr(w), w.element_size() * 8, ctypes.byref(d),
+                                   ctypes.byref(e), stream()))
+    return out
+
+
+def conv_route(x_bits, w_bits, x_shape, w_shape, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1):
+    d = conv_desc(x_shape, w_shape, padding, stride, dilation, groups)
+    return lib().catchq_conv2d_route(x_bits, w_bits, ctypes.byref(d)).decode()

@@ -1,0 +1,236 @@
+"""GPU tests of the drop-in ops torch.ops.torch_mlu.{conv2d,linear} and of the module-swap flow,
+replaying the reference's own test grids (test/magicmind/op_test/test_conv.py:103-156,
+test/magicmind/op_test/test_matmul.py:116-174, test/magicmind/test_quantization.py:42-72) with
+the CPU oracle as the exact expectation and the reference's rel-RMS <= 0.02 vs float as a
+secondary check."""
+import math
+import sys
+from itertools import product
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import oracle as orc
+from oracle import ops as oops
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    import catch_amd  # noqa: F401  (registers the ops)
+    from catch_amd.core.mlu_quantize import quantize_dynamic_mlu
+
+torch.set_grad_enabled(False)
+
+
+def note(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def rel_rms(a, b):  # test/common_utils.py:514-522
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    return math.sqrt(((a - b) ** 2).sum() / (a ** 2).sum())
+
+
+def same_bits(a, b):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    return a.shape == b.shape and a.dtype == b.dtype and np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def calibrate(model, x, bw, per_channel):
+    qconfig = {"use_avg": False, "data_scale": 1.0, "per_channel": per_channel, "firstconv": False}
+    calib = quantize_dynamic_mlu(model, qconfig, dtype=bw, gen_quant=True)
+    calib(x)
+    return calib.state_dict()
+
+
+@pytest.mark.parametrize("bias,bw,per_channel,half",
+                         list(product([True, False], ["int8", "int16"], [True, False], [False, True])))
+def test_conv2d_qint_grid(bias, bw, per_channel, half):
+    note("conv2d_qint", bias, bw, per_channel, half)
+    torch.manual_seed(11)
+    model = nn.Sequential(nn.Conv2d(64, 64, 3, 3, 3, 1, 1, bias)).eval().float()
+    x = torch.randn(3, 64, 24, 24)
+    want_float = model(x).numpy()
+    ckpt = calibrate(model, x, bw, per_channel)
+    qmodel = quantize_dynamic_mlu(model)
+    qmodel.load_state_dict(ckpt)
+    conv = qmodel[0]
+    assert conv.quantized_mode.item() == {("int8", False): 1, ("int16", False): 2, ("int8", True): 3,
+                                          ("int16", True): 4}[(bw, per_channel)]
+    assert conv.scale.numel() == (2 + 64 if per_channel else 2)
+    xin = x.half() if half else x
+    if half:
+        qmodel.half()
+    qmodel.to("cuda")
+    got = qmodel(xin.to("cuda"))
+    assert got.shape == (3, 64, 10, 10) and got.dtype == xin.dtype
+    assert got.is_contiguous(memory_format=torch.channels_last)
+    b = conv.bias.detach().float().cpu().numpy()
+    ref = oops.conv2d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), b, (3, 3), (3, 3), (1, 1), 1,
+                      conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
+    if not half:  # a half model carries half weights: the oracle sees the same rounded values above
+        assert same_bits(ref["y"], got.cpu().numpy())
+    else:
+        assert same_bits(ref["y"], got.cpu().numpy())
+    assert rel_rms(want_float, got.float().cpu().numpy()) <= 0.02
+
+
+@pytest.mark.parametrize("bias,ni,ci,co", list(product([True, False], [1, 10, 20], [10, 50, 100], [25, 75, 125])))
+def test_linear_qint_grid(bias, ni, ci, co):
+    note("linear_qint", bias, ni, ci, co)
+    torch.manual_seed(ni * 1000 + ci * 10 + co)
+    model = nn.Sequential(nn.Linear(ci, co, bias)).eval().float()
+    x = torch.rand(ni, ci)
+    want_float = model(x).numpy()
+    for bw, per_channel, half in product(["int8", "int16"], [True, False], [False, True]):
+        ckpt = calibrate(model, x, bw, per_channel)
+        qmodel = quantize_dynamic_mlu(model)
+        qmodel.load_state_dict(ckpt)
+        lin = qmodel[0]
+        xin = x.half() if half else x
+        if half:
+            qmodel.half()
+        qmodel.to("cuda")
+        got = qmodel(xin.to("cuda"))
+        assert got.dtype == torch.float32 and got.shape == (ni, co)  # fp32 whatever the input type
+        ref = oops.linear(xin.numpy(), lin.weight.detach().float().cpu().numpy(),
+                          lin.bias.detach().float().cpu().numpy(), lin.scale.detach().float().cpu().numpy(),
+                          lin.quantized_mode.cpu().numpy())
+        assert same_bits(ref["y"], got.cpu().numpy()), (bw, per_channel, half)
+        assert rel_rms(want_float, got.cpu().numpy()) <= 0.02, (bw, per_channel, half)
+
+
+def test_linear_leading_dims_and_no_bias_tensor():
+    note("linear leading dims")
+    torch.manual_seed(3)
+    w = torch.randn(48, 32) * 0.1
+    x = torch.randn(2, 5, 32)
+    q_scale = torch.tensor([127 / x.abs().max().item(), 127 / w.abs().max().item()])
+    q_mode = torch.tensor([1], dtype=torch.int32)
+    zero_dim_bias = torch.tensor(0.0)  # bias.dim() == 0 means "no bias" (linear.cpp:57)
+    got = torch.ops.torch_mlu.linear(x.cuda(), w.cuda(), zero_dim_bias.cuda(), q_scale.cuda(), q_mode.cuda())
+    ref = oops.linear(x.numpy(), w.numpy(), None, q_scale.numpy(), q_mode.numpy())
+    assert got.shape == (2, 5, 48) and same_bits(ref["y"], got.cpu().numpy())
+    with pytest.raises(RuntimeError, match="we only support the  dim of weight is 2"):
+        torch.ops.torch_mlu.linear(x.cuda(), w.cuda()[None], zero_dim_bias.cuda(), q_scale.cuda(), q_mode.cuda())
+
+
+def test_conv2d_cnnl_encoding_int16_act_int8_weight():
+    """q_scale = [bitwidth_in, bitwidth_w], q_mode = [pos_in, pos_w] (quantify_conv_forward.cpp:132-145)"""
+    note("conv2d encoding B")
+    torch.manual_seed(5)
+    x = torch.rand(2, 32, 13, 13)
+    w = torch.randn(48, 32, 3, 3) * 0.05
+    b = torch.randn(48)
+    q_scale = torch.tensor([16.0, 8.0])
+    q_mode = torch.tensor([-14, -9], dtype=torch.int32)
+    got = torch.ops.torch_mlu.conv2d(x.cuda(), w.cuda(), b.cuda(), [1, 1], [1, 1], [1, 1], 1, q_scale, q_mode)
+    ref = oops.conv2d(x.numpy(), w.numpy(), b.numpy(), (1, 1), (1, 1), (1, 1), 1, q_scale.numpy(), q_mode.numpy())
+    assert ref["overflow"] == 0 and ref["qx"].dtype == np.int16 and ref["qw"].dtype == np.int8
+    assert same_bits(ref["y"], got.cpu().numpy())
+    want = F.conv2d(x, w, b, 1, 1).numpy()
+    assert rel_rms(want, got.cpu().numpy()) <= 0.02
+
+
+@pytest.mark.parametrize("groups,ci,co", [(2, 4, 16), (8, 8, 8), (32, 32, 32)])
+def test_conv2d_groups_and_layouts(groups, ci, co):
+    note("conv2d groups", groups, ci, co)
+    torch.manual_seed(groups)
+    x = torch.randn(2, ci, 12, 12)
+    w = torch.randn(co, ci // groups, 3, 3) * 0.2
+    b = torch.randn(co)
+    wf = w.reshape(co, -1)
+    q_scale = torch.cat([torch.tensor([127 / x.abs().max().item(), 0.0]), 127 / wf.abs().max(1)[0]])
+    q_mode = torch.tensor([3], dtype=torch.int32)
+    ref = oops.conv2d(x.numpy(), w.numpy(), b.numpy(), (1, 1), (2, 2), (1, 1), groups, q_scale.numpy(), q_mode.numpy())
+    for xin in (x.cuda(), x.cuda().contiguous(memory_format=torch.channels_last), x.cuda().transpose(2, 3).contiguous().transpose(2, 3)):
+        got = torch.ops.torch_mlu.conv2d(xin, w.cuda(), b.cuda(), [1, 1], [2, 2], [1, 1], groups, q_scale.cuda(), q_mode.cuda())
+        assert same_bits(ref["y"], got.cpu().numpy())
+    with pytest.raises(RuntimeError, match="Input's dim must greater than 2!"):
+        torch.ops.torch_mlu.conv2d(x.cuda()[0, 0], w.cuda(), b.cuda(), [1, 1], [2, 2], [1, 1], groups, q_scale.cuda(), q_mode.cuda())
+
+
+def test_weight_cache_follows_inplace_updates():
+    note("weight cache")
+    torch.manual_seed(8)
+    x = torch.randn(1, 16, 8, 8).cuda()
+    w = (torch.randn(16, 16, 3, 3) * 0.1).cuda()
+    b = torch.zeros(16).cuda()
+    q_scale = torch.tensor([127 / 4.0, 127 / 0.5]).cuda()
+    q_mode = torch.tensor([1], dtype=torch.int32).cuda()
+    args = ([1, 1], [1, 1], [1, 1], 1)
+    y1 = torch.ops.torch_mlu.conv2d(x, w, b, *args, q_scale, q_mode)
+    y1b = torch.ops.torch_mlu.conv2d(x, w, b, *args, q_scale, q_mode)  # served from the cache
+    assert torch.equal(y1, y1b)
+    w.mul_(0.5)  # bumps the version counter -> re-quantized
+    y2 = torch.ops.torch_mlu.conv2d(x, w, b, *args, q_scale, q_mode)
+    ref = oops.conv2d(x.cpu().numpy(), w.cpu().numpy(), None, (1, 1), (1, 1), (1, 1), 1, q_scale.cpu().numpy(),
+                      q_mode.cpu().numpy())
+    assert same_bits(ref["y"], y2.cpu().numpy()) and not torch.equal(y1, y2)
+    q_scale[0] = 127 / 8.0  # parameter change is seen too
+    y3 = torch.ops.torch_mlu.conv2d(x, w, b, *args, q_scale, q_mode)
+    ref = oops.conv2d(x.cpu().numpy(), w.cpu().numpy(), None, (1, 1), (1, 1), (1, 1), 1, q_scale.cpu().numpy(),
+                      q_mode.cpu().numpy())
+    assert same_bits(ref["y"], y3.cpu().numpy())
+
+
+def test_cpu_tensors_are_refused():
+    note("cpu refused")
+    x, w, b = torch.randn(1, 4, 4, 4), torch.randn(4, 4, 1, 1), torch.zeros(4)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        torch.ops.torch_mlu.conv2d(x, w, b, [0, 0], [1, 1], [1, 1], 1, torch.tensor([1.0, 1.0]),
+                                   torch.tensor([1], dtype=torch.int32))
+
+
+class _SmallNet(nn.Module):  # test/magicmind/test_quantization.py:22-40
+    def __init__(self, ci):
+        super().__init__()
+        self.block1 = nn.Sequential(nn.Conv2d(ci, 16, 3, 1, 0, 1, 1, bias=False), nn.BatchNorm2d(16, affine=False),
+                                    nn.ReLU())
+
+    def forward(self, x):
+        y = self.block1(x)
+        z = F.max_pool2d(y + y, 2)
+        return torch.transpose(z, 0, 3)
+
+
+@pytest.mark.parametrize("ci", [1, 3, 10])
+def test_quantized_model(ci):
+    note("quantized model", ci)
+    torch.manual_seed(ci)
+    net = _SmallNet(ci).eval().float()
+    x = torch.rand(1, ci, 64, 64)
+    want = net(x).numpy()
+    ckpt = calibrate(net, x, "int8", True)
+    qnet = quantize_dynamic_mlu(net)
+    qnet.load_state_dict(ckpt)
+    got = qnet.to("cuda")(x.to("cuda")).cpu().numpy()
+    assert rel_rms(want, got) <= 0.02
+
+
+def test_helper_ops():
+    note("helper ops")
+    torch.manual_seed(2)
+    x = torch.randn(3, 5, 7, 9).cuda()
+    q = torch.ops.torch_mlu.quantize(x, 8, -5)
+    assert same_bits(orc.quantize(x.cpu().numpy(), 8, -5), q.cpu().numpy())
+    pos, scale, off = torch.ops.torch_mlu.quantize_param(x, 8, 1)
+    p, s, _ = orc.quantize_param(orc.absmax(x.cpu().numpy()), 8)
+    assert pos.item() == p and np.float32(scale.item()) == s
+    assert same_bits(torch.ops.torch_mlu.quantize_dev(x, 8, pos).cpu().numpy(), orc.quantize(x.cpu().numpy(), 8, p))
+    w = (torch.randn(6, 5, 3, 3) * 0.1).cuda()
+    s_c = 127 / w.reshape(6, -1).abs().max(1)[0]
+    qw, new_pos, new_scale = torch.ops.torch_mlu.quantize_per_channel(w, s_c, 8)
+    op, ons, osf = orc.per_channel_params(8, s_c.cpu().numpy())
+    assert new_pos.item() == op and same_bits(ons, new_scale.cpu().numpy())
+    assert same_bits(orc.quantize_per_channel(w.cpu().numpy(), 8, osf), qw.cpu().numpy())
+    d = torch.ops.torch_mlu.dequantize(q, -5)
+    assert same_bits(orc.dequantize(q.cpu().numpy(), -5), d.cpu().numpy())
+    a = torch.randint(-128, 128, (9, 32), dtype=torch.int8).cuda()
+    b = torch.randint(-128, 128, (11, 32), dtype=torch.int8).cuda()
+    acc, _ = orc.gemm_nt(a.cpu().numpy(), b.cpu().numpy())
+    assert same_bits(orc.epilogue(acc, -7), torch.ops.torch_mlu.mm_q(a, -3, b, -4).cpu().numpy())

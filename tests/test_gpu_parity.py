@@ -1,0 +1,281 @@
+"""GPU parity: every HIP kernel, called through the C ABI, against the CPU oracle on the same
+seeded inputs.  Bit-exact for integer outputs; floating outputs are compared bit-exactly too
+where the oracle fixes the operation order, and within 1e-3 of the output range otherwise."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from oracle import ops as oops
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    import cabi
+
+
+def note(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def same_bits(a, b):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    assert a.shape == b.shape and a.dtype == b.dtype
+    return np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def assert_float_close(got, want, what=""):
+    """max-abs <= 1e-3 * output range (the tolerance the target states for fp outputs)"""
+    got, want = got.astype(np.float64), want.astype(np.float64)
+    span = max(want.max() - want.min(), 1e-30) if want.size else 1.0
+    err = np.abs(got - want).max() if want.size else 0.0
+    assert err <= 1e-3 * span, "%s: max-abs %g > 1e-3 * range %g" % (what, err, span)
+
+
+# ------------------------------------------------------------------------------ quantize
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bw", [8, 16, 31])
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 1023, 4096 * 37 + 5])
+def test_quantize_flat(dtype, bw, n):
+    note("quantize_flat", dtype.__name__, bw, n)
+    r = rng(n + bw)
+    pos = -5 if bw == 8 else -11 if bw == 16 else -20
+    x = (r.standard_normal(n) * 3).astype(dtype)
+    if n > 600:
+        k = np.arange(-300, 300)
+        x[:600] = ((k + 0.5) * 2.0 ** pos).astype(dtype)  # exact ties
+        x[600:606] = [np.inf, -np.inf, np.nan, 1e4, -1e4, 0.0]
+    want = orc.quantize(x, bw, pos)
+    got = cabi.quantize(cabi.dev(x), bw, pos).cpu().numpy()
+    assert same_bits(want, got)
+
+
+def test_quantize_fp16_exhaustive_and_scale():
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    for bw, pos, scale in ((8, -4, 1.0), (16, -9, 1.0), (8, 2, 1.0), (16, -3, 1.3721)):
+        note("quantize_fp16_exhaustive", bw, pos, scale)
+        want = orc.quantize(h, bw, pos, scale)
+        got = cabi.quantize(cabi.dev(h), bw, pos, scale).cpu().numpy()
+        assert same_bits(want, got)
+    x = (rng(5).standard_normal(100003) * 2).astype(np.float32)
+    assert same_bits(orc.quantize(x, 8, -6, 1.61803), cabi.quantize(cabi.dev(x), 8, -6, 1.61803).cpu().numpy())
+
+
+def test_quantize_unaligned_and_devpos():
+    x = (rng(6).standard_normal(50001) * 4).astype(np.float32)
+    xd = cabi.dev(x)
+    note("quantize unaligned")
+    got = cabi.quantize(xd[1:], 8, -4).cpu().numpy()  # 4-byte aligned only -> scalar kernel
+    assert same_bits(orc.quantize(x[1:], 8, -4), got)
+    note("quantize devpos")
+    pos = torch.tensor([-4], dtype=torch.int32, device="cuda")
+    assert same_bits(orc.quantize(x, 16, -4), cabi.quantize_devpos(xd, 16, pos).cpu().numpy())
+    sc = torch.tensor([1.25], dtype=torch.float32, device="cuda")
+    assert same_bits(orc.quantize(x, 8, -4, 1.25), cabi.quantize_devpos(xd, 8, pos, sc).cpu().numpy())
+
+
+@pytest.mark.parametrize("shape,cpad", [((2, 3, 17, 19), 4), ((1, 3, 224, 224), 4), ((2, 1, 9, 9), 4),
+                                         ((2, 5, 7, 9), 8), ((2, 70, 5, 6), 70), ((1, 3, 8, 8), 3),
+                                         ((1, 130, 9, 9), 144)])
+@pytest.mark.parametrize("bw", [8, 16])
+def test_quantize_nchw_to_nhwc(shape, cpad, bw):
+    note("quantize_nchw_to_nhwc", shape, cpad, bw)
+    x = rng(sum(shape)).standard_normal(shape).astype(np.float32)
+    want = orc.quantize_nchw_to_nhwc(x, bw, -5, 1.0, cpad)
+    got = cabi.quantize_nchw_to_nhwc(cabi.dev(x), bw, -5, 1.0, cpad).cpu().numpy()
+    assert same_bits(want, got)
+    if bw == 8:
+        goth = cabi.quantize_nchw_to_nhwc(cabi.dev(x.astype(np.float16)), bw, -5, 1.0, cpad).cpu().numpy()
+        assert same_bits(orc.quantize_nchw_to_nhwc(x.astype(np.float16).astype(np.float32), bw, -5, 1.0, cpad), goth)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("n", [1, 7, 100000, 4096 * 300 + 3])
+def test_quantize_param(dtype, n):
+    note("quantize_param", dtype.__name__, n)
+    x = (rng(n).standard_normal(n) * 2.5).astype(dtype)
+    if n > 10:
+        x[n // 2] = np.nan  # ignored by the reduction
+    for bw in (8, 16):
+        absmax, pos, scale, off = cabi.quantize_param(cabi.dev(x), bw)
+        am = orc.absmax(x)
+        p, s, o = orc.quantize_param(am, bw)
+        assert absmax.item() == am and pos.item() == p and np.float32(scale.item()) == s and off.item() == 0.0
+        assert am == np.nanmax(np.abs(x.astype(np.float32)))
+    z = torch.zeros(100, device="cuda")
+    absmax, pos, scale, _ = cabi.quantize_param(z, 8)
+    assert (absmax.item(), pos.item(), scale.item()) == (0.0, 0, 1.0)
+
+
+@pytest.mark.parametrize("bw", [8, 16])
+@pytest.mark.parametrize("shape", [(64, 64, 3, 3), (7, 5), (130, 33, 1, 1)])
+def test_quantize_per_channel(bw, shape):
+    note("quantize_per_channel", bw, shape)
+    r = rng(bw + len(shape))
+    w = (r.standard_normal(shape) * 0.05 * r.uniform(0.2, 3, (shape[0],) + (1,) * (len(shape) - 1))).astype(np.float32)
+    qmax = 127.0 if bw == 8 else 32767.0
+    s = (qmax / np.abs(w).reshape(shape[0], -1).max(1)).astype(np.float32)
+    new_pos, new_scale, sf = orc.per_channel_params(bw, s)
+    got = cabi.quantize_per_channel(cabi.dev(w), bw, cabi.dev(sf)).cpu().numpy()
+    assert same_bits(orc.quantize_per_channel(w, bw, sf), got)
+
+
+def test_dequantize():
+    r = rng(9)
+    for bits, dtype in ((8, np.int8), (16, np.int16), (32, np.int32)):
+        note("dequantize", bits)
+        q = r.integers(-2 ** (bits - 2), 2 ** (bits - 2), 10007).astype(dtype)
+        assert same_bits(orc.dequantize(q, -7), cabi.dequantize(cabi.dev(q), -7).cpu().numpy())
+        assert same_bits(orc.dequantize(q, -7, 1.7), cabi.dequantize(cabi.dev(q), -7, 1.7).cpu().numpy())
+        h = cabi.dequantize(cabi.dev(q), -7, 1.7, half=True).cpu().numpy()
+        assert same_bits(orc.dequantize(q, -7, 1.7).astype(np.float16), h)
+
+
+# ------------------------------------------------------------------------------ GEMM
+def _ints(r, shape, bits):
+    lim = 2 ** (bits - 1)
+    return r.integers(-lim, lim, shape).astype(np.int8 if bits == 8 else np.int16)
+
+
+GEMM_SHAPES = [(1, 1, 16), (5, 7, 16), (128, 128, 64), (130, 70, 80), (257, 129, 1040), (64, 1000, 2048),
+               (300, 64, 48), (1, 10, 10), (20, 125, 100), (33, 17, 7)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_gemm_i8_acc_and_epilogue(m, n, k):
+    note("gemm_i8", m, n, k, cabi.lib().catchq_gemm_route(8, 8, m, n, k))
+    r = rng(m * 7 + n * 3 + k)
+    a, b = _ints(r, (m, k), 8), _ints(r, (n, k), 8)
+    div = r.uniform(0.6, 3.5, n).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    acc, ovf = orc.gemm_nt(a, b)
+    assert ovf == 0
+    ad, bd = cabi.dev(a), cabi.dev(b)
+    out = cabi.gemm_nt(ad, bd, exp2=-9, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=1)
+    assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
+    assert same_bits(orc.epilogue(acc, -9, div, bias, None, 1), out["y"].cpu().numpy())
+    out = cabi.gemm_nt(ad, bd, exp2=-9, bias=cabi.dev(bias), act=0, y_dtype=torch.float16, want_acc=False,
+                       q_bw=8, q_pos=-2)
+    y = orc.epilogue(acc, -9, None, bias, None, 0)
+    assert same_bits(y.astype(np.float16), out["y"].cpu().numpy())
+    assert same_bits(orc.quantize(y, 8, -2), out["q"].cpu().numpy())
+
+
+@pytest.mark.parametrize("bits", [(16, 8), (16, 16)])
+@pytest.mark.parametrize("m,n,k", [(20, 125, 100), (64, 64, 128), (3, 5, 600)])
+def test_gemm_wide(bits, m, n, k):
+    note("gemm_wide", bits, m, n, k)
+    r = rng(k + bits[1])
+    a, b = _ints(r, (m, k), bits[0]), _ints(r, (n, k), bits[1])
+    bias = r.standard_normal(n).astype(np.float32)
+    acc, ovf = orc.gemm_nt(a, b)
+    out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=-20, bias=cabi.dev(bias), want_acc=(bits == (16, 8)))
+    if bits == (16, 8):
+        assert ovf == 0
+        assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
+    assert same_bits(orc.epilogue(acc, -20, None, bias), out["y"].cpu().numpy())
+
+
+def test_gemm_full_size_properties():
+    """Config-2 sizes: too big for the oracle in seconds, so check what the integers must satisfy:
+    rows of A that are copies give equal rows of C, and a sampled set of entries equals the
+    oracle's dot products."""
+    for (m, n, k) in ((4096, 3072, 768), (4096, 768, 3072)):
+        note("gemm_full", m, n, k)
+        r = rng(k)
+        a, b = _ints(r, (m, k), 8), _ints(r, (n, k), 8)
+        a[1234] = a[17]
+        out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), y_dtype=None)
+        acc = out["acc"].cpu().numpy()
+        assert np.array_equal(acc[1234], acc[17])
+        rows = r.integers(0, m, 64)
+        want, _ = orc.gemm_nt(a[rows], b)
+        assert np.array_equal(want.astype(np.int32), acc[rows])
+        # linearity in A: (a1 + a2) B^T = a1 B^T + a2 B^T with halves that cannot overflow int8
+        a1, a2 = (a // 2).astype(np.int8), (a - a // 2).astype(np.int8)
+        s = cabi.gemm_nt(cabi.dev(a1), cabi.dev(b), y_dtype=None)["acc"] + \
+            cabi.gemm_nt(cabi.dev(a2), cabi.dev(b), y_dtype=None)["acc"]
+        assert torch.equal(s, out["acc"])
+
+
+# ------------------------------------------------------------------------------ conv
+CONV_CASES = [
+    # N, Ci, H, W, Co, kh, kw, pad, stride, dil, groups
+    (3, 64, 24, 24, 64, 3, 3, (3, 3), (3, 3), (1, 1), 1),      # reference qint grid
+    (2, 4, 6, 6, 16, 3, 3, (0, 0), (1, 1), (1, 1), 2),         # reference groups case
+    (1, 3, 14, 14, 8, 2, 2, (0, 0), (1, 1), (1, 1), 1),
+    (2, 6, 9, 11, 10, 3, 2, (1, 2), (2, 1), (2, 1), 2),
+    (2, 16, 9, 11, 24, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # MFMA, K=144 (tail step)
+    (2, 64, 14, 14, 128, 1, 1, (0, 0), (1, 1), (1, 1), 1),     # 1x1
+    (2, 64, 15, 15, 160, 1, 1, (0, 0), (2, 2), (1, 1), 1),     # 1x1 stride 2 (downsample)
+    (2, 32, 13, 13, 64, 3, 3, (1, 1), (2, 2), (1, 1), 1),      # 3x3 stride 2
+    (1, 48, 10, 12, 40, 3, 3, (2, 2), (1, 1), (2, 2), 1),      # dilation
+    (1, 128, 7, 7, 256, 3, 3, (1, 1), (1, 1), (1, 1), 1),
+    (1, 16, 5, 5, 32, 5, 5, (2, 2), (1, 1), (1, 1), 1),
+    (1, 80, 8, 8, 16, 7, 1, (3, 0), (1, 1), (1, 1), 1),        # asymmetric kernel
+    (2, 32, 12, 12, 32, 3, 3, (1, 1), (1, 1), (1, 1), 32),     # depthwise s1
+    (2, 96, 15, 15, 96, 3, 3, (1, 1), (2, 2), (1, 1), 96),     # depthwise s2
+    (1, 8, 10, 10, 8, 3, 3, (1, 1), (2, 2), (1, 1), 8),        # depthwise, few channels
+    (1, 36, 40, 40, 36, 5, 5, (2, 2), (1, 1), (1, 1), 36),     # depthwise 5x5, several strips
+    (1, 6, 7, 7, 6, 3, 3, (1, 1), (1, 1), (1, 1), 6),          # depthwise C%4 != 0 -> direct
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_i8_acc_and_epilogue(case):
+    n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
+    route = cabi.conv_route(8, 8, (n, h, w, ci), (co, kh, kw, ci // g), pad, stride, dil, g)
+    note("conv_i8", case, route)
+    r = rng(sum(case[:7]))
+    x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, kh, kw, ci // g), 8)
+    acc, ovf = orc.conv2d_nhwc(x, wt, pad, stride, dil, g)
+    assert ovf == 0
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = r.standard_normal(co).astype(np.float32)
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    xd, wd = cabi.dev(x), cabi.dev(wt)
+    out = cabi.conv2d_nhwc(xd, wd, pad, stride, dil, g, exp2=-10, chan_div=cabi.dev(div), bias=cabi.dev(bias),
+                           resid=cabi.dev(resid), act=1, q_bw=8, q_pos=-3)
+    assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
+    y = orc.epilogue(acc, -10, div, bias, resid, 1)
+    assert same_bits(y, out["y"].cpu().numpy())
+    assert same_bits(orc.quantize(y, 8, -3), out["q"].cpu().numpy())
+    out = cabi.conv2d_nhwc(xd, wd, pad, stride, dil, g, exp2=-10, act=2, y_dtype=torch.float16, want_acc=False)
+    assert same_bits(orc.epilogue(acc, -10, None, None, None, 2, np.float16), out["y"].cpu().numpy())
+
+
+@pytest.mark.parametrize("bits", [(16, 8), (16, 16)])
+@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[4], CONV_CASES[12]])
+def test_conv_wide(bits, case):
+    n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
+    note("conv_wide", bits, case)
+    r = rng(sum(case[:7]) + bits[1])
+    x, wt = _ints(r, (n, h, w, ci), bits[0]), _ints(r, (co, kh, kw, ci // g), bits[1])
+    acc, ovf = orc.conv2d_nhwc(x, wt, pad, stride, dil, g)
+    bias = r.standard_normal(co).astype(np.float32)
+    out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), pad, stride, dil, g, exp2=-22, bias=cabi.dev(bias),
+                           want_acc=(bits == (16, 8)))
+    if bits == (16, 8):
+        assert ovf == 0 and same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
+    assert same_bits(orc.epilogue(acc, -22, None, bias), out["y"].cpu().numpy())
+
+
+def test_error_statuses():
+    note("error statuses")
+    x = torch.zeros(16, device="cuda")
+    q = torch.zeros(16, dtype=torch.int8, device="cuda")
+    L = cabi.lib()
+    assert L.catchq_quantize(cabi.ptr(x), 0, cabi.ptr(q), 7, 16, 0, 1.0, cabi.stream()) == 3  # bitwidth
+    assert L.catchq_quantize(cabi.ptr(x), 5, cabi.ptr(q), 8, 16, 0, 1.0, cabi.stream()) == 2  # dtype
+    assert L.catchq_quantize(None, 0, cabi.ptr(q), 8, 16, 0, 1.0, cabi.stream()) == 1          # null
+    assert L.catchq_quantize(None, 0, None, 8, 0, 0, 1.0, cabi.stream()) == 0                  # empty is fine
+    with pytest.raises(Exception):
+        cabi.conv2d_nhwc(torch.zeros((1, 2, 2, 4), dtype=torch.int8, device="cuda"),
+                         torch.zeros((4, 3, 3, 4), dtype=torch.int8, device="cuda"))  # output extent <= 0
