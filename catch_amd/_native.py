@@ -47,11 +47,13 @@ SIGNATURES = {
     "catchq_gemm_nt": (_I, [_P, _I, _P, _I, _I64, _I64, _I64, ctypes.POINTER(Epilogue), _P]),
     "catchq_conv_out_size": (_I, [_I] * 5),
     "catchq_conv2d_nhwc": (_I, [_P, _I, _P, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Epilogue), _P]),
+    "catchq_maxpool_nhwc": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "catchq_global_avgpool_nhwc": (_I, [_P, _P, _I, _I, _I, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
 }
 
-_BUILD_HINT = "build it with `python -m catch_amd.build` (hipcc cross-compiles gfx950 without a GPU)"
+_BUILD_HINT = "build it with `python catch_amd/build.py` (hipcc cross-compiles gfx950 without a GPU)"
 
 
 def kernel_lib():

@@ -3,7 +3,8 @@
   catch_amd/lib/libcatchq.so        hand-written gfx950 HIP kernels behind the C ABI of include/catchq.h
   catch_amd/lib/_catchq_torch.so    PyTorch-ROCm extension registering the torch_mlu::* ops on top of it
 
-hipcc cross-compiles for gfx950 without a GPU.  Run ``python -m catch_amd.build``.
+hipcc cross-compiles for gfx950 without a GPU.  Run ``python catch_amd/build.py [kernels|torch|all]`` (by path: the package itself cannot be
+imported before its libraries exist).
 """
 import os
 import subprocess
@@ -18,7 +19,7 @@ INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
-KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "dwconv_i8.hip", "capi.hip",
+KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "dwconv_i8.hip", "pool.hip", "capi.hip",
                   "host_math.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from the fp32 epilogue math.

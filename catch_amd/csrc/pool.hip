@@ -1,0 +1,122 @@
+// Pooling on NHWC tensors for pipelines that keep activations quantized between layers.
+//   max pooling (int8 / int16 / fp32): quantization is monotonic, so pooling the integers equals
+//     quantizing the pooled floats;
+//   global average pooling (fp32): sequential sum over (h, w) in that order, then one division --
+//     a fixed order, so the result is reproducible bit for bit.
+#include "catchq_common.h"
+
+namespace catchq {
+
+template <typename T>
+struct Lowest;
+template <>
+struct Lowest<int8_t> {
+  static __device__ int8_t value() { return -128; }
+};
+template <>
+struct Lowest<int16_t> {
+  static __device__ int16_t value() { return -32768; }
+};
+template <>
+struct Lowest<float> {
+  static __device__ float value() { return -__builtin_inff(); }
+};
+
+// one thread = one output pixel x VEC consecutive channels (VEC * sizeof(T) = 16 bytes, or VEC = 1)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const T *__restrict__ x, T *__restrict__ y, int N, int H,
+                                                          int W, int C, int k, int stride, int pad, int Ho,
+                                                          int Wo) {
+  const int cv = C / VEC;
+  const int64_t total = (int64_t)N * Ho * Wo * cv;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
+    const int c = (int)(idx % cv) * VEC;
+    int64_t p = idx / cv;
+    const int wo = (int)(p % Wo);
+    p /= Wo;
+    const int ho = (int)(p % Ho);
+    const int n = (int)(p / Ho);
+    T m[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m[j] = Lowest<T>::value();
+    for (int r = 0; r < k; ++r) {
+      const int hi = ho * stride - pad + r;
+      if ((unsigned)hi >= (unsigned)H) continue;
+      for (int q = 0; q < k; ++q) {
+        const int wi = wo * stride - pad + q;
+        if ((unsigned)wi >= (unsigned)W) continue;
+        const T *src = x + (((int64_t)n * H + hi) * W + wi) * C + c;
+        T v[VEC];
+        if constexpr (VEC == 1) v[0] = src[0];
+        else *reinterpret_cast<v4i *>(v) = *reinterpret_cast<const v4i *>(src);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) m[j] = (v[j] > m[j]) ? v[j] : m[j];
+      }
+    }
+    T *dst = y + (((int64_t)n * Ho + ho) * Wo + wo) * C + c;
+    if constexpr (VEC == 1) dst[0] = m[0];
+    else *reinterpret_cast<v4i *>(dst) = *reinterpret_cast<v4i *>(m);
+  }
+}
+
+template <typename T>
+static int launch_maxpool(const void *x, void *y, int N, int H, int W, int C, int k, int stride, int pad, int Ho,
+                          int Wo, hipStream_t s) {
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec = (C % VEC == 0) && aligned16(x) && aligned16(y);
+  const int64_t total = (int64_t)N * Ho * Wo * (vec ? C / VEC : C);
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks < 1) blocks = 1;
+  if (vec)
+    maxpool_nhwc_kernel<T, VEC><<<(int)blocks, 256, 0, s>>>((const T *)x, (T *)y, N, H, W, C, k, stride, pad, Ho, Wo);
+  else
+    maxpool_nhwc_kernel<T, 1><<<(int)blocks, 256, 0, s>>>((const T *)x, (T *)y, N, H, W, C, k, stride, pad, Ho, Wo);
+  return launch_status();
+}
+
+__global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                 int N, int HW, int C) {
+  const int64_t total = (int64_t)N * C;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(idx % C);
+    const int64_t n = idx / C;
+    const float *src = x + n * HW * C + c;
+    float s = 0.0f;
+    for (int p = 0; p < HW; ++p) s = s + src[(int64_t)p * C];
+    y[idx] = s / (float)HW;
+  }
+}
+
+}  // namespace catchq
+
+using namespace catchq;
+
+CATCHQ_API int catchq_maxpool_nhwc(const void *x, void *y, int elem_bits, int n, int h, int w, int c, int k,
+                                   int stride, int pad, catchq_stream_t stream) {
+  if (n < 0 || h <= 0 || w <= 0 || c <= 0 || k <= 0 || stride <= 0 || pad < 0 || 2 * pad > k) return CATCHQ_ERR_SHAPE;
+  const int ho = (h + 2 * pad - k) / stride + 1, wo = (w + 2 * pad - k) / stride + 1;
+  if (ho <= 0 || wo <= 0) return CATCHQ_ERR_SHAPE;
+  if (n == 0) return CATCHQ_OK;
+  if (!x || !y) return CATCHQ_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (elem_bits) {
+    case 8: return launch_maxpool<int8_t>(x, y, n, h, w, c, k, stride, pad, ho, wo, s);
+    case 16: return launch_maxpool<int16_t>(x, y, n, h, w, c, k, stride, pad, ho, wo, s);
+    case 32: return launch_maxpool<float>(x, y, n, h, w, c, k, stride, pad, ho, wo, s);
+    default: return CATCHQ_ERR_BITWIDTH;
+  }
+}
+
+CATCHQ_API int catchq_global_avgpool_nhwc(const float *x, float *y, int n, int hw, int c, catchq_stream_t stream) {
+  if (n < 0 || hw <= 0 || c <= 0) return CATCHQ_ERR_SHAPE;
+  if (n == 0) return CATCHQ_OK;
+  if (!x || !y) return CATCHQ_ERR_ARG;
+  const int64_t total = (int64_t)n * c;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 65536) blocks = 65536;
+  global_avgpool_nhwc_kernel<<<blocks, 256, 0, as_stream(stream)>>>(x, y, n, hw, c);
+  return launch_status();
+}

@@ -494,6 +494,38 @@ Tensor linear_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   return o.y.view(shape);
 }
 
+// x [N,H,W,C] contiguous int8 / int16 / fp32
+Tensor maxpool_nhwc_op(const Tensor &x, int64_t k, int64_t stride, int64_t pad) {
+  TORCH_CHECK(x.dim() == 4 && x.is_contiguous(), "maxpool_nhwc expects a contiguous [N,H,W,C] tensor");
+  int bits = 0;
+  switch (x.scalar_type()) {
+    case at::kChar: bits = 8; break;
+    case at::kShort: bits = 16; break;
+    case at::kFloat: bits = 32; break;
+    default: TORCH_CHECK(false, "maxpool_nhwc: int8, int16 or float32 expected");
+  }
+  c10::DeviceGuard guard(x.device());
+  const int64_t ho = (x.size(1) + 2 * pad - k) / stride + 1, wo = (x.size(2) + 2 * pad - k) / stride + 1;
+  TORCH_CHECK(ho > 0 && wo > 0, "Calculated output size is too small");
+  Tensor y = at::empty({x.size(0), ho, wo, x.size(3)}, x.options());
+  check_status(catchq_maxpool_nhwc(x.data_ptr(), y.data_ptr(), bits, (int)x.size(0), (int)x.size(1), (int)x.size(2),
+                                   (int)x.size(3), (int)k, (int)stride, (int)pad, current_stream()),
+               "torch_mlu::maxpool_nhwc");
+  return y;
+}
+
+// x [N,H,W,C] contiguous fp32 -> [N,C]
+Tensor global_avgpool_nhwc_op(const Tensor &x) {
+  TORCH_CHECK(x.dim() == 4 && x.is_contiguous() && x.scalar_type() == at::kFloat,
+              "global_avgpool_nhwc expects a contiguous fp32 [N,H,W,C] tensor");
+  c10::DeviceGuard guard(x.device());
+  Tensor y = at::empty({x.size(0), x.size(3)}, x.options());
+  check_status(catchq_global_avgpool_nhwc(x.data_ptr<float>(), y.data_ptr<float>(), (int)x.size(0),
+                                          (int)(x.size(1) * x.size(2)), (int)x.size(3), current_stream()),
+               "torch_mlu::global_avgpool_nhwc");
+  return y;
+}
+
 std::string conv2d_route_op(int64_t x_bits, int64_t w_bits, at::IntArrayRef in_nhwc, at::IntArrayRef w_ohwi,
                             at::IntArrayRef padding, at::IntArrayRef stride, at::IntArrayRef dilation,
                             int64_t groups) {
@@ -523,6 +555,8 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
         "bool want_y=True, bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, "
         "float q_scale=1.0) -> (Tensor, Tensor, Tensor)");
+  m.def("maxpool_nhwc(Tensor x, int k, int stride, int pad) -> Tensor");
+  m.def("global_avgpool_nhwc(Tensor x) -> Tensor");
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
         "int[] dilation, int groups) -> str", &conv2d_route_op);
@@ -540,4 +574,6 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("mm_q", &mm_q_op);
   m.impl("qconv2d", &qconv2d_op);
   m.impl("qlinear", &qlinear_op);
+  m.impl("maxpool_nhwc", &maxpool_nhwc_op);
+  m.impl("global_avgpool_nhwc", &global_avgpool_nhwc_op);
 }

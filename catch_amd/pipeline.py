@@ -1,0 +1,235 @@
+"""Fused int8/int16 execution of a calibrated network.
+
+The drop-in ops (``torch_mlu::conv2d`` / ``linear``) take and return floating tensors, so a model
+built from them writes every activation in fp32, reads it back, quantizes it, and runs ReLU and
+the residual add as separate float kernels.  This module compiles the same network -- the layer
+list of ``catch_amd.nets`` plus a checkpoint in the reference's format (``scale``,
+``quantized_mode`` per layer) -- into a plan in which each convolution's epilogue applies
+dequantization, bias, residual add and activation and writes the *next* layer's quantized input
+directly; fp32 copies are written only where a residual branch, the global average pool or a
+network output needs them.  Max pooling runs on the integers (quantization is monotonic).
+
+Every value is computed by the same arithmetic, in the same order, as the unfused sequence
+quantize -> integer conv -> dequant+bias -> add -> activation -> quantize, so all quantized
+tensors, int32 accumulators and fp32 outputs are identical to it bit for bit.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _native
+from .nets import outputs_of
+
+_ACT_CODE = {"none": 0, "relu": 1, "relu6": 2}
+_PASS = ("maxpool", "upsample", "concat")
+
+
+def _key(name):
+    return "mods." + name.replace(".", "_") + "."
+
+
+def pos_from_scale(bw, scale):
+    p = ctypes.c_int()
+    _native.check(_native.kernel_lib().catchq_pos_from_scale(int(bw), float(scale), ctypes.byref(p)), "position")
+    return p.value
+
+
+class _LayerQ(object):
+    """decoded q-params and the quantized weight of one conv / fc layer"""
+    __slots__ = ("bw_x", "bw_w", "pos_x", "pos_w", "qw", "chan_div", "bias", "exp2", "cpad")
+
+
+def _decode(layer, sd, device):
+    q = _LayerQ()
+    k = _key(layer.name)
+    w = sd[k + "weight"].to(device=device, dtype=torch.float32)
+    scale = sd[k + "scale"].detach().float().cpu()
+    mode = sd[k + "quantized_mode"].detach().cpu().to(torch.int32).reshape(-1)
+    bias = sd.get(k + "bias")
+    q.bias = None if bias is None else bias.to(device=device, dtype=torch.float32).contiguous()
+    q.chan_div = None
+    if layer.kind == "conv":
+        w = w.contiguous(memory_format=torch.channels_last)  # memory [Co][kh][kw][Ci/g]
+    if mode.numel() == 1:
+        m = int(mode[0])
+        bw = 8 if m in (1, 3) else 16
+        q.bw_x = q.bw_w = bw
+        q.pos_x = pos_from_scale(bw, scale[0].item())
+        if m > 2:
+            qw, new_pos, new_scale = torch.ops.torch_mlu.quantize_per_channel(w, scale[2:].to(device), bw)
+            q.pos_w, q.chan_div = int(new_pos.item()), new_scale
+        else:
+            q.pos_w = pos_from_scale(bw, scale[1].item())
+            qw = torch.ops.torch_mlu.quantize(w, bw, q.pos_w)
+    else:
+        q.bw_x, q.bw_w = int(scale[0].item()), int(scale[1].item())
+        q.pos_x, q.pos_w = int(mode[0]), int(mode[1])
+        qw = torch.ops.torch_mlu.quantize(w, q.bw_w, q.pos_w)
+    q.exp2 = q.pos_x + q.pos_w
+    q.cpad = 0
+    if layer.kind == "conv":
+        qw = qw.permute(0, 2, 3, 1)  # [Co,kh,kw,Ci/g] view of the same memory
+        if layer.groups == 1 and layer.ci < 4:  # few-channel network input: pad channels to 4 (zeros)
+            q.cpad = 4
+            qw = torch.nn.functional.pad(qw, (0, 4 - layer.ci))
+        qw = qw.contiguous()
+    q.qw = qw
+    return q
+
+
+class FusedNet(object):
+    def __init__(self, layers, state_dict, device="cuda", out_half=False):
+        self.layers = list(layers)
+        self.device = torch.device(device)
+        self.outputs = outputs_of(self.layers)
+        self.out_half = out_half
+        self.q = {l.name: _decode(l, state_dict, self.device) for l in self.layers if l.kind in ("conv", "fc")}
+        self._plan_demands()
+        self._graph = None
+
+    # which forms of every tensor are needed: 'f' (fp32 NHWC) and/or quantized at (bitwidth, position)
+    def _plan_demands(self):
+        names = ["input"] + [l.name for l in self.layers]
+        self.q_demand = {n: [] for n in names}
+        self.f_demand = {n: False for n in names}
+        for o in self.outputs:
+            self.f_demand[o] = True
+
+        def want_q(t, d):
+            if d not in self.q_demand[t]:
+                self.q_demand[t].append(d)
+
+        for l in reversed(self.layers):
+            if l.kind in ("conv", "fc"):
+                lq = self.q[l.name]
+                want_q(l.src, (lq.bw_x, lq.pos_x))
+                if l.add:
+                    self.f_demand[l.add] = True
+            elif l.kind == "gap":
+                self.f_demand[l.src] = True
+            elif l.kind in _PASS:
+                for s in ((l.src,) if isinstance(l.src, str) else l.src):
+                    for d in self.q_demand[l.name]:
+                        want_q(s, d)
+                    self.f_demand[s] = self.f_demand[s] or self.f_demand[l.name]
+        # a conv epilogue writes one quantized form; further ones are quantized from the fp32 copy
+        for l in self.layers:
+            if l.kind in ("conv", "fc") and len(self.q_demand[l.name]) > 1:
+                self.f_demand[l.name] = True
+
+    # ------------------------------------------------------------------------------------------
+    def forward(self, x, trace=None):
+        """x: [N,3,H,W] fp32 (NCHW) on the device.  trace: optional dict filled with, per conv/fc
+        layer, its quantized input, int32 accumulators and fp32 output (as NHWC tensors)."""
+        ops = torch.ops.torch_mlu
+        env = {}
+        tracing = trace is not None
+        for d in self.q_demand["input"]:
+            first = self.layers[0]
+            cpad = self.q[first.name].cpad if first.kind == "conv" else 0
+            env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], cpad)
+        for l in self.layers:
+            name = l.name
+            if l.kind == "conv":
+                lq = self.q[name]
+                qx = env[(l.src, lq.bw_x, lq.pos_x)]
+                resid = env[(l.add, "f")] if l.add else None
+                qd = self.q_demand[name][0] if self.q_demand[name] else None
+                want_y = self.f_demand[name] or tracing or qd is None
+                y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
+                                        [l.stride, l.stride], [1, 1], l.groups, _ACT_CODE[l.act], want_y,
+                                        self.out_half and name in self.outputs, tracing,
+                                        qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
+                if want_y:
+                    env[(name, "f")] = y
+                if qd:
+                    env[(name,) + qd] = q
+                for d in self.q_demand[name][1:]:
+                    env[(name,) + d] = ops.quantize(y, d[0], d[1])
+                if tracing:
+                    trace[name] = dict(qx=qx, acc=acc, y=y)
+            elif l.kind == "fc":
+                lq = self.q[name]
+                qx = env[(l.src, lq.bw_x, lq.pos_x)]
+                qx2 = qx.reshape(qx.shape[0], -1)
+                y, _, acc = ops.qlinear(qx2, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, tracing, 0, 0, 1.0)
+                env[(name, "f")] = y
+                if tracing:
+                    trace[name] = dict(qx=qx2, acc=acc, y=y)
+            elif l.kind == "maxpool":
+                for form in self._forms(name):
+                    env[(name,) + form] = ops.maxpool_nhwc(env[(l.src,) + form], l.k, l.stride, l.pad)
+            elif l.kind == "gap":
+                g = ops.global_avgpool_nhwc(env[(l.src, "f")])
+                env[(name, "f")] = g.reshape(g.shape[0], 1, 1, g.shape[1])
+                for d in self.q_demand[name]:
+                    env[(name,) + d] = ops.quantize(env[(name, "f")], d[0], d[1])
+            elif l.kind == "upsample":
+                for form in self._forms(name):
+                    t = env[(l.src,) + form]
+                    env[(name,) + form] = t.repeat_interleave(2, 1).repeat_interleave(2, 2)
+            elif l.kind == "concat":
+                for form in self._forms(name):
+                    env[(name,) + form] = torch.cat([env[(s,) + form] for s in l.src], 3)
+            else:
+                raise ValueError(l.kind)
+        outs = []
+        for o in self.outputs:
+            y = env[(o, "f")]
+            outs.append(y.permute(0, 3, 1, 2) if y.dim() == 4 else y)  # logical NCHW over NHWC memory
+        return outs[0] if len(outs) == 1 else tuple(outs)
+
+    __call__ = forward
+
+    def _forms(self, name):
+        forms = [tuple(d) for d in self.q_demand[name]]
+        if self.f_demand[name]:
+            forms.append(("f",))
+        return forms
+
+    # ------------------------------------------------------------------------------------------
+    def capture(self, example):
+        """Record one forward pass into a HIP graph; returns (static_input, replay) where replay()
+        re-runs the whole network on whatever static_input holds and returns the static output(s)."""
+        static_in = example.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                self.forward(static_in)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = self.forward(static_in)
+        self._graph = graph
+
+        def replay():
+            graph.replay()
+            return static_out
+
+        return static_in, replay
+
+
+def calibrate(float_net, x_cpu, dtype="int8", per_channel=True):
+    """Run the reference-style calibration flow on the CPU and return the checkpoint
+    (weights + scale / quantized_mode / scale_weight_per_channel per layer)."""
+    from .core.mlu_quantize import quantize_dynamic_mlu
+    spec = {"use_avg": False, "data_scale": 1.0, "per_channel": per_channel, "firstconv": False, "iteration": 1}
+    calib = quantize_dynamic_mlu(float_net, spec, dtype=dtype, gen_quant=True)
+    with torch.no_grad():
+        calib(x_cpu)
+    sd = calib.state_dict()
+    # merge the per-channel scales the way the modules do when they load the checkpoint
+    out = {}
+    for k, v in sd.items():
+        out[k] = v
+    for k in list(sd.keys()):
+        if k.endswith(".scale"):
+            p = k[:-len("scale")]
+            if p + "scale_weight_per_channel" in sd:
+                out[k] = torch.cat((sd[k], sd[p + "scale_weight_per_channel"])).float()
+                m = int(sd[p + "quantized_mode"].item())
+                out[p + "quantized_mode"] = torch.tensor([m + 2 if m in (1, 2) else m], dtype=torch.int32)
+    return out

@@ -157,6 +157,20 @@ int catchq_conv_out_size(int in, int k, int pad, int stride, int dil);
 int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int w_bits, const catchq_conv_desc_t *desc,
                        const catchq_epilogue_t *epilogue, catchq_stream_t stream);
 
+/* ------------------------------------------------------------------ neighbours of the convolutions */
+
+/* Max pooling over an NHWC tensor whose elements are int8, int16 (quantized activations) or fp32
+ * (elem_bits 8 / 16 / 32); windows k x k, zero-size padding never wins (2*pad <= k).  The reference
+ * pools in float between its quantized ops (cnnl_max_pool2d, operators/cnnl/pooling.cpp); because
+ * quantization is monotonic, pooling the integers gives the same integers. */
+int catchq_maxpool_nhwc(const void *x, void *y, int elem_bits, int n, int h, int w, int c, int k, int stride,
+                        int pad, catchq_stream_t stream);
+
+/* Global average pooling of an fp32 NHWC tensor [n, hw, c] -> [n, c]: sequential fp32 sum over the
+ * pixels in storage order, then one division by hw (adaptive_avg_pool2d((1,1)) in the reference's
+ * models, operators/cnnl/pooling.cpp). */
+int catchq_global_avgpool_nhwc(const float *x, float *y, int n, int hw, int c, catchq_stream_t stream);
+
 /* Name of the kernel family catchq_conv2d_nhwc / catchq_gemm_nt would use ("mfma", "direct",
  * "depthwise", ...): for logs and tests; not part of the arithmetic. */
 const char *catchq_conv2d_route(int x_bits, int w_bits, const catchq_conv_desc_t *desc);

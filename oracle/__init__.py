@@ -51,6 +51,7 @@ def _load():
         "orc_conv2d_nhwc": (c_i64, [c_p, c_i, c_p, c_i] + [c_i] * 14 + [c_p]),
         "orc_epilogue_f32": (None, [c_p, c_i64, c_i64, c_i, c_p, c_p, c_p, c_i, c_p]),
         "orc_epilogue_f16": (None, [c_p, c_i64, c_i64, c_i, c_p, c_p, c_p, c_i, c_p]),
+        "orc_global_avgpool_nhwc_f32": (None, [c_p, c_i, c_i, c_i, c_p]),
         "orc_maxpool_nhwc_f32": (None, [c_p, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_p]),
     }
     for name, (res, args) in sig.items():
@@ -223,4 +224,13 @@ def maxpool_nhwc(x, k, stride, pad):
     ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
     y = np.empty((n, ho, wo, c), np.float32)
     _lib.orc_maxpool_nhwc_f32(_ptr(x), n, h, w, c, k, stride, pad, _ptr(y))
+    return y
+
+
+def global_avgpool_nhwc(x):
+    """x [N,H,W,C] fp32 -> [N,C]"""
+    x = _c(x, np.float32)
+    n, h, w, c = x.shape
+    y = np.empty((n, c), np.float32)
+    _lib.orc_global_avgpool_nhwc_f32(_ptr(x), n, h * w, c, _ptr(y))
     return y

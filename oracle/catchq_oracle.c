@@ -478,6 +478,18 @@ ORC_API void orc_epilogue_f16(const int64_t *acc, int64_t rows, int64_t co, int 
           orc_f32_to_f16(orc_epi1(acc[r * co + c], exp2, chan_div, bias, resid, r * co + c, c, act));
 }
 
+/* Global average pooling of an NHWC fp32 tensor: sequential fp32 sum over the pixels in storage
+ * order, one division.  The order is this build's definition (floating-point sums depend on it). */
+ORC_API void orc_global_avgpool_nhwc_f32(const float *x, int N, int HW, int C, float *y) {
+#pragma omp parallel for
+  for (int64_t i = 0; i < (int64_t)N * C; ++i) {
+    int64_t n = i / C, c = i % C;
+    float s = 0.0f;
+    for (int p = 0; p < HW; ++p) s = s + x[(n * HW + p) * C + c];
+    y[i] = s / (float)HW;
+  }
+}
+
 /* 2-D max pooling over an NHWC fp32 tensor (-inf padding), used by the model
  * level checks; not part of the quantized arithmetic itself. */
 ORC_API void orc_maxpool_nhwc_f32(const float *x, int N, int H, int W, int C, int k, int stride,

@@ -1,0 +1,133 @@
+"""Model-level parity: the fused int8 pipeline on the GPU against the oracle's unfused,
+layer-by-layer execution of the same calibrated network -- every layer's quantized input and
+int32 accumulators bit-exact, outputs within 1e-3 of their range (they are in fact identical),
+and the module-swap drop-in flow against both."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import netref
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    import catch_amd  # noqa: F401
+    from catch_amd import nets, pipeline
+    from catch_amd.core.mlu_quantize import quantize_dynamic_mlu
+
+torch.set_grad_enabled(False)
+
+
+def note(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def np_sd(sd):
+    return {k: v.detach().cpu().numpy() for k, v in sd.items()}
+
+
+def check_against_oracle(layers, sd, x, fused):
+    t, rec = netref.run(layers, np_sd(sd), x.numpy())
+    trace = {}
+    out = fused.forward(x.cuda(), trace=trace)
+    torch.cuda.synchronize()
+    for l in layers:
+        if l.kind not in ("conv", "fc"):
+            continue
+        r, g = rec[l.name], trace[l.name]
+        assert r["overflow"] == 0, l.name
+        qx = g["qx"].cpu().numpy()
+        if qx.ndim == 4 and qx.shape[-1] != r["qx"].shape[-1]:  # channel-padded network input
+            assert not qx[..., r["qx"].shape[-1]:].any()
+            qx = qx[..., :r["qx"].shape[-1]]
+        assert np.array_equal(r["qx"].reshape(qx.shape), qx), "quantized input of " + l.name
+        assert np.array_equal(r["acc"].astype(np.int32), g["acc"].cpu().numpy().reshape(r["acc"].shape)), \
+            "accumulators of " + l.name
+        assert np.array_equal(r["y"].reshape(-1), g["y"].float().cpu().numpy().reshape(-1)), "output of " + l.name
+    outs = out if isinstance(out, tuple) else (out,)
+    for name, o in zip(fused.outputs, outs):
+        want = t[name]
+        got = o.float().cpu().numpy()
+        got = np.transpose(got, (0, 2, 3, 1)) if got.ndim == 4 else got.reshape(want.shape)
+        span = float(want.max() - want.min())
+        assert np.abs(got - want).max() <= 1e-3 * span
+    # the untraced run (fp32 copies only where needed) gives the same outputs
+    out2 = fused.forward(x.cuda())
+    outs2 = out2 if isinstance(out2, tuple) else (out2,)
+    for a, b in zip(outs, outs2):
+        assert torch.equal(a, b)
+    return outs
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_resnet18_bs1(per_channel):
+    """ResNet-18, 1x3x224x224 N(0,1), weights N(0,0.05), int8 weights and activations."""
+    note("resnet18", per_channel)
+    layers = nets.resnet(18)
+    net = nets.FloatNet(layers, seed=0).eval()
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(1))
+    sd = pipeline.calibrate(net, x, "int8", per_channel)
+    fused = pipeline.FusedNet(layers, sd)
+    check_against_oracle(layers, sd, x, fused)
+
+
+def test_resnet50_small_batch_and_graph_replay():
+    note("resnet50 bs2 112x112")
+    layers = nets.resnet(50)
+    net = nets.FloatNet(layers, seed=0).eval()
+    x = torch.randn(2, 3, 112, 112, generator=torch.Generator().manual_seed(2))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd)
+    (logits,) = check_against_oracle(layers, sd, x, fused)
+    # HIP graph: several replays, with eager work in between, all equal to the eager result
+    static_in, replay = fused.capture(x.cuda())
+    for i in range(3):
+        static_in.copy_(x.cuda())
+        out = replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, logits), "replay %d" % i
+        _ = fused.forward(torch.randn(2, 3, 112, 112, device="cuda"))
+        torch.cuda.synchronize()
+
+
+def test_dropin_modules_match_fused_pipeline():
+    """quantize_dynamic_mlu flow (torch_mlu::conv2d/linear + ATen relu/add/pool in float) gives
+    the same logits as the fused plan, up to the global-average-pool summation order."""
+    note("drop-in vs fused")
+    layers = nets.resnet(18)
+    net = nets.FloatNet(layers, seed=3).eval()
+    x = torch.randn(2, 3, 96, 96, generator=torch.Generator().manual_seed(4))
+    spec = {"use_avg": False, "data_scale": 1.0, "per_channel": True, "firstconv": False}
+    calib = quantize_dynamic_mlu(net, spec, dtype="int8", gen_quant=True)
+    calib(x)
+    ckpt = calib.state_dict()
+    qnet = quantize_dynamic_mlu(net)
+    qnet.load_state_dict(ckpt)
+    got = qnet.to("cuda")(x.cuda())
+    fused = pipeline.FusedNet(layers, pipeline.calibrate(net, x, "int8", True))
+    want = fused.forward(x.cuda())
+    span = (want.max() - want.min()).item()
+    assert (got - want).abs().max().item() <= 1e-3 * span
+
+
+def test_pool_kernels():
+    note("pool kernels")
+    import oracle as orc
+    g = np.random.default_rng(0)
+    for shape, k, s, p in (((2, 9, 11, 64), 3, 2, 1), ((1, 8, 8, 6), 2, 2, 0), ((2, 7, 7, 16), 3, 1, 1)):
+        x = g.standard_normal(shape).astype(np.float32)
+        want = orc.maxpool_nhwc(x, k, s, p)
+        got = torch.ops.torch_mlu.maxpool_nhwc(torch.from_numpy(x).cuda(), k, s, p).cpu().numpy()
+        assert np.array_equal(want, got)
+        q = orc.quantize(x, 8, -5)
+        gq = torch.ops.torch_mlu.maxpool_nhwc(torch.from_numpy(q).cuda(), k, s, p).cpu().numpy()
+        assert np.array_equal(orc.quantize(want, 8, -5), gq)  # pooling commutes with quantization
+        q16 = orc.quantize(x, 16, -12)
+        gq16 = torch.ops.torch_mlu.maxpool_nhwc(torch.from_numpy(q16).cuda(), k, s, p).cpu().numpy()
+        assert np.array_equal(orc.quantize(want, 16, -12), gq16)
+    x = (g.standard_normal((3, 7, 7, 130)) * 100).astype(np.float32)
+    got = torch.ops.torch_mlu.global_avgpool_nhwc(torch.from_numpy(x).cuda()).cpu().numpy()
+    assert np.array_equal(orc.global_avgpool_nhwc(x), got)

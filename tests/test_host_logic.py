@@ -197,5 +197,5 @@ def test_missing_native_library_is_loud(tmp_path, monkeypatch):
     from catch_amd import _native
     monkeypatch.setattr(_native, "_lib", None)
     monkeypatch.setattr(_native, "KERNEL_LIB", str(tmp_path / "nope.so"))
-    with pytest.raises(ImportError, match="catch_amd.build"):
+    with pytest.raises(ImportError, match="catch_amd/build.py"):
         _native.kernel_lib()
