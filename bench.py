@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference hot path on one MI355X.
+
+A step is one forward pass of the fused int8 pipeline over one batch that is already resident in
+HBM (fp32 NCHW input -> fp32 logits), replayed from a HIP graph.  Default workload: ResNet-50 v1.5,
+batch 64, 3x224x224 N(0,1) inputs, per-channel int8 weights / per-tensor int8 activations,
+random-init seeded weights N(0,0.05) with batch norm folded.
+
+Prints ONE JSON line: images/s, plus
+  roofline      achieved algorithmic GB/s of the dominant kernel family (the int8 implicit-GEMM
+                convolutions) against the 8 TB/s HBM peak, from HIP-event timings of every launch;
+  cpu_baseline  the CPU oracle (a port of the reference's formulas) on a bounded sample of the
+                same batch, on the host cores of this box;
+  extras        int8 GEMM TOPS on the standalone-linear shapes and quantize-kernel GB/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "resnet18", "mobilenet_v2"])
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--calib-images", type=int, default=8)
+    ap.add_argument("--cpu-images", type=int, default=2)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    return ap.parse_args()
+
+
+def event_time(fn, iters, warm=3):
+    """average seconds per call, HIP events on the current stream (the one the kernels run on)"""
+    import torch
+    for _ in range(warm):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    e.synchronize()
+    return s.elapsed_time(e) * 1e-3 / iters
+
+
+def layer_profile(fused, x, iters=20):
+    """Time every kernel launch of one forward pass separately (HIP events, `iters` back-to-back
+    launches each) and attach the algorithmic bytes / ops of each conv / fc launch."""
+    import torch
+    ops = torch.ops.torch_mlu
+    rows = []
+    trace = {}
+    fused.forward(x, trace=trace)  # materialise every layer's quantized input once
+    torch.cuda.synchronize()
+    for l in fused.layers:
+        if l.kind not in ("conv", "fc"):
+            continue
+        lq = fused.q[l.name]
+        qx = trace[l.name]["qx"]
+        qd = fused.q_demand[l.name][0] if fused.q_demand[l.name] else None
+        want_y = fused.f_demand[l.name] or qd is None
+        if l.kind == "conv":
+            resid = torch.zeros_like(trace[l.name]["y"]) if l.add else None
+
+            def run(l=l, lq=lq, qx=qx, qd=qd, want_y=want_y, resid=resid):
+                return ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
+                                   [l.stride, l.stride], [1, 1], l.groups, {"none": 0, "relu": 1, "relu6": 2}[l.act],
+                                   want_y, False, False, qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
+            route = ops.conv2d_route(8, 8, list(qx.shape), list(lq.qw.shape[:3]) + [lq.qw.shape[3]],
+                                     [l.pad, l.pad], [l.stride, l.stride], [1, 1], l.groups)
+        else:
+            def run(lq=lq, qx=qx):
+                return ops.qlinear(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, False, 0, 0, 1.0)
+            resid = None
+            route = "gemm"
+        y = trace[l.name]["y"]
+        n_out = y.numel()
+        macs = n_out * (lq.qw.numel() // lq.qw.shape[0])
+        bytes_alg = qx.numel() * qx.element_size() + lq.qw.numel() * lq.qw.element_size()
+        bytes_alg += (4 * n_out if want_y else 0) + (n_out * (qd[0] // 8) if qd else 0) + (4 * n_out if resid is not None else 0)
+        t = event_time(run, iters)
+        rows.append(dict(name=l.name, route=route, t=t, ops=2 * macs, bytes=bytes_alg))
+    return rows
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (every box has one GPU, "
+              "the path shards by batch with no communication)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    torch.set_grad_enabled(False)
+    import catch_amd  # noqa: F401  (fails loudly if the HIP extension is missing)
+    from catch_amd import nets, pipeline
+
+    batch = args.batch or {"resnet50": 64, "resnet18": 64, "mobilenet_v2": 128}[args.workload]
+    layers = nets.NETS[args.workload]()
+    net = nets.FloatNet(layers, seed=0).eval()
+    x = torch.randn(batch, 3, 224, 224, generator=torch.Generator().manual_seed(1))
+    t0 = time.time()
+    sd = pipeline.calibrate(net, x[:args.calib_images], "int8", True)
+    t_cal = time.time() - t0
+    fused = pipeline.FusedNet(layers, sd)
+    xg = x.cuda()
+    static_in, replay = fused.capture(xg)
+    static_in.copy_(xg)
+    for _ in range(args.warmup):
+        replay()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(args.steps):
+        out = replay()
+    e.record()
+    torch.cuda.synchronize()
+    ms_per_step = s.elapsed_time(e) / args.steps
+    value = batch / (ms_per_step * 1e-3)
+    logits = out.float().cpu()
+    assert torch.isfinite(logits).all()
+
+    # ---- per-kernel roofline of the dominant family: the implicit-GEMM convolutions ------------
+    rows = layer_profile(fused, xg)
+    conv_rows = [r for r in rows if r["route"] == "mfma"]
+    t_conv = sum(r["t"] for r in conv_rows)
+    b_conv = sum(r["bytes"] for r in conv_rows)
+    o_conv = sum(r["ops"] for r in conv_rows)
+    t_all = sum(r["t"] for r in rows)
+    if args.layers:
+        for r in rows:
+            print("%-12s %-9s %8.1f us %7.1f GB/s %7.1f TOPS" % (r["name"], r["route"], r["t"] * 1e6,
+                                                                r["bytes"] / r["t"] / 1e9, r["ops"] / r["t"] / 1e12),
+                  file=sys.stderr)
+        print("sum of conv/fc launches: %.1f us; graph step: %.1f us" % (t_all * 1e6, ms_per_step * 1e3), file=sys.stderr)
+    roofline = {"bound": "hbm", "kernel": "igemm_i8_kernel (all %d launches of one step)" % len(conv_rows),
+                "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                "avg_launch_us": round(t_conv / max(len(conv_rows), 1) * 1e6, 2),
+                "algorithmic_bytes_per_step": b_conv, "int8_tops": round(o_conv / t_conv / 1e12, 1),
+                "mfma_frac": round(o_conv / t_conv / 1e12 / INT8_PEAK_TOPS, 4)}
+
+    result = {"metric": "int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
+              else "int8 %s images/sec" % args.workload,
+              "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+              "dtype": "int8", "data": "synthetic",
+              "config": {"workload": "%s int8 (per-channel W, per-tensor act), batch %d, 3x224x224 N(0,1), fused "
+                                     "requant pipeline replayed from a HIP graph" % (args.workload, batch),
+                         "global_batch": batch, "calibration_images": args.calib_images,
+                         "gop_per_step": round(2 * nets.conv_macs(layers, batch, 224, 224) / 1e9, 1)},
+              "roofline": roofline}
+
+    if not args.no_extras:
+        result["extras"] = extras()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(layers, sd, x[:args.cpu_images], out[:args.cpu_images].float().cpu())
+    result["calibration_s"] = round(t_cal, 2)
+    print(json.dumps(result))
+
+
+def extras():
+    """standalone kernels: int8 linear (config shapes) and quantize streaming rate"""
+    import ctypes
+    import torch
+    ops = torch.ops.torch_mlu
+    out = {}
+    for (m, n, k) in ((4096, 3072, 768), (4096, 768, 3072)):
+        a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
+        b = torch.randint(-128, 128, (n, k), dtype=torch.int8, device="cuda")
+        bias = torch.randn(n, device="cuda")
+        div = torch.rand(n, device="cuda") + 0.5
+        t = event_time(lambda: ops.qlinear(a, b, -10, div, bias, 1, True, True, False, 0, 0, 1.0), 200, 20)
+        out["linear_%dx%dx%d" % (m, n, k)] = {"us": round(t * 1e6, 2), "tops": round(2 * m * n * k / t / 1e12, 1),
+                                             "mfma_frac": round(2 * m * n * k / t / 1e12 / INT8_PEAK_TOPS, 4),
+                                             "epilogue": "per-channel dequant + bias + ReLU, fp16 out"}
+    n = 64 * 256 * 56 * 56  # one ResNet-50 stage-1 activation, 822 MB of fp32: larger than the 256 MB cache
+    x = torch.randn(n, device="cuda")
+    t = event_time(lambda: ops.quantize(x, 8, -5, 1.0), 20, 3)
+    out["quantize_f32_to_i8"] = {"elements": n, "us": round(t * 1e6, 1), "gbs": round(5 * n / t / 1e9, 1),
+                                 "hbm_frac": round(5 * n / t / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
+
+
+def cpu_baseline(layers, sd, x_sample, gpu_logits):
+    """the oracle's unfused execution of the same network on a few images of the same batch"""
+    import numpy as np
+    import oracle as orc
+    from oracle import netref
+    sdn = {k: v.detach().cpu().numpy() for k, v in sd.items()}
+    t0 = time.time()
+    t, _ = netref.run(layers, sdn, x_sample.numpy())
+    dt = time.time() - t0
+    want = t[layers[-1].name].reshape(gpu_logits.shape)
+    span = float(want.max() - want.min())
+    err = float(np.abs(want - gpu_logits.numpy()).max())
+    return {"value": round(x_sample.shape[0] / dt, 3), "unit": "images/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": "%d images of the same batch through the whole network (oracle, OpenMP)" % x_sample.shape[0],
+            "gpu_vs_oracle_max_abs": err, "output_range": span, "within_1e-3_of_range": bool(err <= 1e-3 * span)}
+
+
+if __name__ == "__main__":
+    main()

@@ -33,6 +33,8 @@ static Route conv_route(int x_bits, int w_bits, const catchq_conv_desc_t *d, con
         dwconv_i8_supported(d->ci, d->kh, d->kw, d->stride_w, d->dil_w) && (!x || aligned16(x)))
       return kDepthwise;
     if (d->groups == 1 && d->ci % 16 == 0 && (!x || aligned16(x)) && (!w || aligned16(w))) return kMfma;
+    // four-channel inputs (an RGB image padded to 4): one pixel per dword
+    if (d->groups == 1 && d->ci == 4 && d->dil_w == 1 && (!x || aligned16(x)) && (!w || aligned16(w))) return kMfma;
   }
   return kDirect;
 }

@@ -220,6 +220,12 @@ CONV_CASES = [
     (1, 128, 7, 7, 256, 3, 3, (1, 1), (1, 1), (1, 1), 1),
     (1, 16, 5, 5, 32, 5, 5, (2, 2), (1, 1), (1, 1), 1),
     (1, 80, 8, 8, 16, 7, 1, (3, 0), (1, 1), (1, 1), 1),        # asymmetric kernel
+    (2, 4, 30, 30, 64, 7, 7, (3, 3), (2, 2), (1, 1), 1),       # 4-channel input, 7x7 s2 (network stem)
+    (1, 4, 9, 13, 24, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # 4-channel input, 3x3
+    (2, 4, 11, 10, 40, 5, 2, (2, 0), (1, 1), (2, 1), 1),       # 4-channel input, 5x2, vertical dilation
+    (1, 4, 6, 6, 8, 1, 1, (0, 0), (1, 1), (1, 1), 1),          # 4-channel input, 1x1
+    (1, 64, 9, 9, 72, 1, 1, (0, 0), (1, 1), (1, 1), 1),        # Co % 64 != 0
+    (1, 32, 5, 5, 30, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # Co % 4 != 0 -> scalar epilogue
     (2, 32, 12, 12, 32, 3, 3, (1, 1), (1, 1), (1, 1), 32),     # depthwise s1
     (2, 96, 15, 15, 96, 3, 3, (1, 1), (2, 2), (1, 1), 96),     # depthwise s2
     (1, 8, 10, 10, 8, 3, 3, (1, 1), (2, 2), (1, 1), 8),        # depthwise, few channels

@@ -103,6 +103,7 @@ def test_routes(lib):
         return lib.catchq_conv2d_route(bits[0], bits[1], ctypes.byref(d)).decode()
     assert route(64, 64, 3, 1) == "mfma"
     assert route(3, 64, 7, 1) == "direct"
+    assert route(4, 64, 7, 1) == "mfma"
     assert route(32, 32, 3, 32) == "depthwise"
     assert route(4, 16, 3, 2) == "direct"
     assert route(64, 64, 3, 1, (16, 16)) == "direct"
