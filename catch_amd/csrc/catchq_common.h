@@ -40,13 +40,36 @@ struct QRange<31> {
   static constexpr float lo = -1073741824.0f, hi = 1073741823.0f;
 };
 
+// v_cvt_i32_f32 saturates out-of-range values and converts NaN to 0: with an integer clamp after
+// it that is exactly "NaN -> 0, otherwise saturate".
+__device__ __forceinline__ int cvt_i32_sat(float r) {
+  int i;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(i) : "v"(r));
+  return i;
+}
+
 // x*scale is one fp32 rounding (exact for scale == 1), the scaling by 2^-pos is exact.
 template <int BW>
 __device__ __forceinline__ int quant1(float x, float scale, int neg_pos) {
-  float t = __builtin_ldexpf(x * scale, neg_pos);
-  float r = __builtin_rintf(t);
-  r = fminf(fmaxf(r, QRange<BW>::lo), QRange<BW>::hi);
-  return (t != t) ? 0 : (int)r;
+  const float t = __builtin_ldexpf(x * scale, neg_pos);
+  const int i = cvt_i32_sat(__builtin_rintf(t));
+  constexpr int lo = (int)QRange<BW>::lo, hi = (int)QRange<BW>::hi;
+  return min(max(i, lo), hi);
+}
+
+// same with scale == 1 known (x * 1.0f == x bit for bit, so the multiply is dropped)
+template <int BW>
+__device__ __forceinline__ int quant1_unit(float x, int neg_pos) {
+  const int i = cvt_i32_sat(__builtin_rintf(__builtin_ldexpf(x, neg_pos)));
+  constexpr int lo = (int)QRange<BW>::lo, hi = (int)QRange<BW>::hi;
+  return min(max(i, lo), hi);
+}
+
+// v / d through the precomputed correctly rounded reciprocal r (see include/catchq.h)
+__device__ __forceinline__ float div_by_rcp(float v, float d, float r) {
+  const float q = v * r;
+  const float err = __builtin_fmaf(-q, d, v);
+  return __builtin_fmaf(err, r, q);
 }
 
 struct ConvDev {
@@ -57,6 +80,7 @@ struct ConvDev {
 struct EpiDev {
   int exp2;
   const float *chan_div;
+  const float *chan_rcp;  // only set when the fused reciprocal form may be used
   const float *bias;
   const float *resid;
   int act;
@@ -73,6 +97,7 @@ inline EpiDev make_epi(const catchq_epilogue_t *e) {
   EpiDev d;
   d.exp2 = e->exp2;
   d.chan_div = e->chan_div;
+  d.chan_rcp = (e->chan_div && e->chan_rcp && e->exp2 >= -64 && e->exp2 <= 64) ? e->chan_rcp : nullptr;
   d.bias = e->bias;
   d.resid = e->resid;
   d.act = e->act;

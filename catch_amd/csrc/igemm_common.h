@@ -1,0 +1,233 @@
+// Pieces shared by the int8 implicit-GEMM kernels: parameters, the LDS swizzle, and the epilogue.
+#pragma once
+#include <type_traits>
+
+#include "catchq_common.h"
+
+namespace catchq {
+
+struct IgemmParams {
+  int64_t M;
+  int N, K;
+  int H, W, Ci, Ho, Wo, kh, kw, ph, pw, sh, sw, dh, dw;
+  int kwq;  // LOAD_C4: chunks (groups of 4 taps) per filter row
+  int tiles_n;
+  int nblocks;
+};
+
+constexpr int BK = 64;  // bytes of K per pipeline step (one LDS row)
+enum { LOAD_GEMM = 0, LOAD_CONV = 1, LOAD_C4 = 2 };
+
+// LDS rows are 64 bytes = four 16-byte chunks; the chunk index is XOR-ed with (row>>2)&3 so that
+// 16 consecutive rows at one logical chunk fall into 16 different 16-byte bank groups
+// (measured: 176 B/clk/CU with the swizzle, 62 B/clk/CU without).
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 2) & 3); }
+
+// block id -> tile index, XCD-aware: ids that land on one XCD (id % 8) take a contiguous run of
+// tiles, so neighbouring tiles (same A rows, same weights) share that XCD's L2.
+__device__ __forceinline__ int xcd_remap(int bid, int nb) {
+  const int xcd = bid & 7, local = bid >> 3;
+  const int q = nb >> 3, rem = nb & 7;
+  return xcd * q + (xcd < rem ? xcd : rem) + local;
+}
+
+inline bool vec_epilogue_ok(int N, const EpiDev &e) {
+  return N % 4 == 0 && aligned16(e.chan_div) && aligned16(e.chan_rcp) && aligned16(e.bias) && aligned16(e.resid) && aligned16(e.y) &&
+         aligned16(e.acc_out) && aligned16(e.q);
+}
+
+// What an epilogue instance knows at compile time.  A field of -1 is decided at run time from the
+// EpiDev (the generic instance); fixed fields let the compiler drop every untaken branch, which
+// matters because the epilogue is VALU-bound (about a dozen fp32 operations per output element).
+//   DIV  0 none, 1 reciprocal form, 2 true division      BIAS, RESID  0/1
+//   ACT  CATCHQ_ACT_*       YM  0 none, 1 fp32, 2 fp16     QM  0 none, 8, 16     ACC 0/1
+template <int DIV, int BIAS, int RESID, int ACT, int YM, int QM, int ACC>
+struct EpiSpec {
+  static constexpr bool kGeneric = DIV < 0;
+  static __device__ __forceinline__ bool rcp(const EpiDev &e) { return DIV < 0 ? e.chan_rcp != nullptr : DIV == 1; }
+  static __device__ __forceinline__ bool truediv(const EpiDev &e) {
+    return DIV < 0 ? (e.chan_div != nullptr && e.chan_rcp == nullptr) : DIV == 2;
+  }
+  static __device__ __forceinline__ bool bias(const EpiDev &e) { return BIAS < 0 ? e.bias != nullptr : BIAS == 1; }
+  static __device__ __forceinline__ bool resid(const EpiDev &e) { return RESID < 0 ? e.resid != nullptr : RESID == 1; }
+  static __device__ __forceinline__ int act(const EpiDev &e) { return ACT < 0 ? e.act : ACT; }
+  static __device__ __forceinline__ bool y32(const EpiDev &e) { return YM < 0 ? (e.y && !e.y_f16) : YM == 1; }
+  static __device__ __forceinline__ bool y16(const EpiDev &e) { return YM < 0 ? (e.y && e.y_f16) : YM == 2; }
+  static __device__ __forceinline__ bool q8(const EpiDev &e) { return QM < 0 ? (e.q && e.q_bw == 8) : QM == 8; }
+  static __device__ __forceinline__ bool q16(const EpiDev &e) { return QM < 0 ? (e.q && e.q_bw == 16) : QM == 16; }
+  static __device__ __forceinline__ bool acc(const EpiDev &e) { return ACC < 0 ? e.acc_out != nullptr : ACC == 1; }
+};
+typedef EpiSpec<-1, -1, -1, -1, -1, -1, -1> EpiGeneric;
+
+// epilogue variants a kernel can be instantiated with
+enum {
+  EPI_SCALAR = 0,   // any N / alignment: one element at a time, straight from the accumulators
+  EPI_VECTOR = 1,   // generic, vectorised through LDS (N % 4 == 0, 16-byte aligned pointers)
+  EPI_Q8_RELU = 2,  // reciprocal-form dequant + bias + ReLU -> int8                 (conv feeding a conv)
+  EPI_RES_Y_Q8 = 3, // ... + residual + ReLU -> fp32 and int8                         (end of a residual block)
+  EPI_Y32 = 4,      // reciprocal-form dequant + bias -> fp32                         (projection shortcut)
+  EPI_RES_Y = 5,    // ... + residual + ReLU -> fp32                                   (last block)
+  EPI_Y16_RELU = 6, // reciprocal-form dequant + bias + ReLU -> fp16                  (standalone linear)
+  EPI_Q8_RELU6 = 7, // reciprocal-form dequant + bias + ReLU6 -> int8
+  EPI_COUNT = 8
+};
+template <int EPI> struct EpiOf { typedef EpiGeneric type; };
+template <> struct EpiOf<EPI_Q8_RELU> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_RELU, 0, 8, 0> type; };
+template <> struct EpiOf<EPI_RES_Y_Q8> { typedef EpiSpec<1, 1, 1, CATCHQ_ACT_RELU, 1, 8, 0> type; };
+template <> struct EpiOf<EPI_Y32> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_NONE, 1, 0, 0> type; };
+template <> struct EpiOf<EPI_RES_Y> { typedef EpiSpec<1, 1, 1, CATCHQ_ACT_RELU, 1, 0, 0> type; };
+template <> struct EpiOf<EPI_Y16_RELU> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_RELU, 2, 0, 0> type; };
+template <> struct EpiOf<EPI_Q8_RELU6> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_RELU6, 0, 8, 0> type; };
+
+// which variant serves this launch (the specialised ones also need a unit requantization scale)
+inline int pick_epilogue(int N, const EpiDev &e) {
+  if (!vec_epilogue_ok(N, e)) return EPI_SCALAR;
+  const bool rcp = e.chan_rcp != nullptr, bias = e.bias != nullptr, resid = e.resid != nullptr;
+  const int ym = !e.y ? 0 : (e.y_f16 ? 2 : 1);
+  const int qm = !e.q ? 0 : e.q_bw;
+  if (!rcp || !bias || e.acc_out || (qm && e.q_scale != 1.0f)) return EPI_VECTOR;
+  if (!resid && e.act == CATCHQ_ACT_RELU && ym == 0 && qm == 8) return EPI_Q8_RELU;
+  if (resid && e.act == CATCHQ_ACT_RELU && ym == 1 && qm == 8) return EPI_RES_Y_Q8;
+  if (!resid && e.act == CATCHQ_ACT_NONE && ym == 1 && qm == 0) return EPI_Y32;
+  if (resid && e.act == CATCHQ_ACT_RELU && ym == 1 && qm == 0) return EPI_RES_Y;
+  if (!resid && e.act == CATCHQ_ACT_RELU && ym == 2 && qm == 0) return EPI_Y16_RELU;
+  if (!resid && e.act == CATCHQ_ACT_RELU6 && ym == 0 && qm == 8) return EPI_Q8_RELU6;
+  return EPI_VECTOR;
+}
+
+// Epilogue of one wave.  acc[i][j] are 32x32 MFMA tiles: lane holds column (lane&31) and rows
+// 8*(r/4) + 4*(lane>>5) + (r&3).  (m_w, n_w) = global row / column of the wave tile's origin.
+// Vector variants: the wave transposes 32 rows at a time through its private LDS area `stage` so
+// that a lane owns four consecutive channels of one pixel.
+template <int TM, int TN, int EPI>
+__device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
+                                               const IgemmParams &p, const EpiDev &e) {
+  typedef typename EpiOf<EPI>::type S;
+  constexpr int WN = TN * 32;
+  constexpr int EPI_STRIDE = WN + 8;  // +8 ints: the two half-waves write different banks
+  const int frow = lane & 31, fhalf = lane >> 5;
+  if constexpr (EPI == EPI_SCALAR) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = n_w + j * 32 + frow;
+        if (n >= p.N) continue;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t m = m_w + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
+          if (m >= p.M) continue;
+          const int64_t idx = m * p.N + n;
+          const int a = acc[i][j][r];
+          if (e.acc_out) e.acc_out[idx] = a;
+          epi_store(epi_value((float)a, idx, n, e), idx, e);
+        }
+      }
+    }
+  } else {
+    constexpr int CPR = WN / 4;    // 4-channel groups per staged row
+    constexpr int RPI = 64 / CPR;  // rows the wave moves per iteration
+    const int cg = lane % CPR, rsub = lane / CPR;
+    const int n = n_w + cg * 4;
+    const bool n_ok = n < p.N;
+    const bool use_rcp = S::rcp(e), use_div = S::truediv(e), use_bias = S::bias(e), use_res = S::resid(e);
+    const int act = S::act(e);
+    // per-channel constants of this lane.  Reciprocal form with the power of two folded in:
+    //   v = (f*2^e)/d  ==  q = f*(r*2^e); err = fma(-q, d*2^-e, f); fma(err, r*2^e, q)
+    // (scaling by 2^e is exact, so every intermediate is the scaled image of the unfolded one)
+    v4f div = {1.f, 1.f, 1.f, 1.f}, rcp = {1.f, 1.f, 1.f, 1.f}, bias = {0.f, 0.f, 0.f, 0.f};
+    if (n_ok && (use_rcp || use_div)) div = *reinterpret_cast<const v4f *>(e.chan_div + n);
+    if (n_ok && use_rcp) {
+      rcp = *reinterpret_cast<const v4f *>(e.chan_rcp + n);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        rcp[t] = __builtin_ldexpf(rcp[t], e.exp2);
+        div[t] = __builtin_ldexpf(div[t], -e.exp2);
+      }
+    }
+    if (n_ok && use_bias) bias = *reinterpret_cast<const v4f *>(e.bias + n);
+    const bool unit_q = S::kGeneric ? (e.q_scale == 1.0f) : true;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      // residual rows of this 32-row block: all loads in flight before the staging below
+      v4f resv[32 / RPI];
+      if (use_res) {
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+          const int64_t m = m_w + i * 32 + it * RPI + rsub;
+          resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
+          if (n_ok && m < p.M) resv[it] = *reinterpret_cast<const v4f *>(e.resid + m * p.N + n);
+        }
+      }
+      // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
+      const int64_t mbase = m_w + i * 32;
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int row = it * RPI + rsub;
+        const int64_t m = mbase + row;
+        const v4i a = *reinterpret_cast<const v4i *>(stage + row * EPI_STRIDE + cg * 4);
+        if (!n_ok || m >= p.M) continue;
+        const int64_t idx = m * p.N + n;
+        if (S::acc(e)) *reinterpret_cast<v4i *>(e.acc_out + idx) = a;
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          float x = (float)a[t];
+          if (use_rcp) x = div_by_rcp(x, div[t], rcp[t]);
+          else {
+            x = __builtin_ldexpf(x, e.exp2);
+            if (use_div) x = x / div[t];
+          }
+          if (use_bias) x = x + bias[t];
+          if (use_res) x = x + resv[it][t];
+          if (act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
+          if (act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
+          v[t] = x;
+        }
+        if (S::y16(e)) {
+          __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
+                          __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
+          *reinterpret_cast<v2i *>(reinterpret_cast<__half *>(e.y) + idx) = *reinterpret_cast<v2i *>(h);
+        } else if (S::y32(e)) {
+          v4f o = {v[0], v[1], v[2], v[3]};
+          *reinterpret_cast<v4f *>(reinterpret_cast<float *>(e.y) + idx) = o;
+        }
+        if (S::q8(e)) {
+          int b[4];
+          if (unit_q) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) b[t] = quant1_unit<8>(v[t], e.q_neg_pos);
+          } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) b[t] = quant1<8>(v[t], e.q_scale, e.q_neg_pos);
+          }
+          // four clamped values -> four bytes: two byte permutes and a merge
+          const unsigned lo = __builtin_amdgcn_perm((unsigned)b[1], (unsigned)b[0], 0x0c0c0400u);
+          const unsigned hi = __builtin_amdgcn_perm((unsigned)b[3], (unsigned)b[2], 0x04000c0cu);
+          *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = lo | hi;
+        } else if (S::q16(e)) {
+          v2i pk;
+          unsigned h[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            h[t] = (unsigned)(unit_q ? quant1_unit<16>(v[t], e.q_neg_pos) : quant1<16>(v[t], e.q_scale, e.q_neg_pos)) & 0xffffu;
+          pk[0] = (int)(h[0] | (h[1] << 16));
+          pk[1] = (int)(h[2] | (h[3] << 16));
+          *reinterpret_cast<v2i *>(reinterpret_cast<int16_t *>(e.q) + idx) = pk;
+        }
+      }
+    }
+  }
+}
+
+// launchers of the LDS-DMA pipelined kernel (igemm_i8_dma.hip); return -1 when the shape is not
+// eligible (operand of 2 GiB or more, four-channel stem) and the caller takes the register-staged kernel
+int igemm_dma_launch(int load, const void *a, const void *b, IgemmParams p, const EpiDev &e, int64_t a_bytes,
+                     int64_t b_bytes, hipStream_t s);
+
+}  // namespace catchq

@@ -17,23 +17,11 @@
 // Epilogue: each wave transposes its accumulators through LDS (32 rows at a time) so that a lane
 // owns four consecutive output channels of one pixel; residual loads and all stores are then
 // 16-byte (fp32) / 4-byte (int8) vectors and whole output rows are written contiguously.
-#include "catchq_common.h"
+#include <cstdlib>
+
+#include "igemm_common.h"
 
 namespace catchq {
-
-struct IgemmParams {
-  int64_t M;
-  int N, K;
-  int H, W, Ci, Ho, Wo, kh, kw, ph, pw, sh, sw, dh, dw;
-  int kwq;  // LOAD_C4: chunks (groups of 4 taps) per filter row
-  int tiles_n;
-  int nblocks;
-};
-
-constexpr int BK = 64;
-enum { LOAD_GEMM = 0, LOAD_CONV = 1, LOAD_C4 = 2 };
-
-__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 2) & 3); }
 
 // 16 bytes from a 4-byte aligned address
 __device__ __forceinline__ v4i load16_a4(const int8_t *p) {
@@ -41,7 +29,7 @@ __device__ __forceinline__ v4i load16_a4(const int8_t *p) {
   return reinterpret_cast<const P *>(p)->v;
 }
 
-template <int BM, int BN, int LOAD, bool VEC_EPI>
+template <int BM, int BN, int LOAD, int EPI>
 __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict__ A,
                                                       const int8_t *__restrict__ B, IgemmParams p,
                                                       EpiDev e) {
@@ -50,7 +38,7 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
   constexpr int LA = BM / 64, LB = BN / 64;  // 16-byte chunks each thread loads per K step
   constexpr int EPI_STRIDE = WN + 8;         // ints per staged row (+8: the two half-waves hit different banks)
   constexpr int PIPE_BYTES = 2 * (BM + BN) * BK;
-  constexpr int EPI_BYTES = VEC_EPI ? 4 * 32 * EPI_STRIDE * 4 : 0;
+  constexpr int EPI_BYTES = EPI != EPI_SCALAR ? 4 * 32 * EPI_STRIDE * 4 : 0;
   constexpr int LDS_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
   __shared__ __attribute__((aligned(16))) int8_t lds_raw[LDS_BYTES];
   int8_t(*lds)[(BM + BN) * BK] = reinterpret_cast<int8_t(*)[(BM + BN) * BK]>(lds_raw);
@@ -60,15 +48,7 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
   const int wave = tid >> 6;
   const int wave_m = wave >> 1, wave_n = wave & 1;
 
-  // block id -> tile, XCD-aware: ids that land on one XCD (id % 8) take a contiguous run of
-  // tiles, so neighbouring tiles (same A rows, same weights) share that XCD's L2.
-  int logical;
-  {
-    const int bid = blockIdx.x, nb = p.nblocks;
-    const int xcd = bid & 7, local = bid >> 3;
-    const int q = nb >> 3, rem = nb & 7;
-    logical = xcd * q + (xcd < rem ? xcd : rem) + local;
-  }
+  const int logical = xcd_remap(blockIdx.x, p.nblocks);
   const int tile_n = logical % p.tiles_n;
   const int tile_m = logical / p.tiles_n;
   const int64_t m0 = (int64_t)tile_m * BM;
@@ -120,8 +100,12 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
     while (kq >= p.kwq) { kq -= p.kwq; ++kr; }
   }
 
-  v4i ra[LA], rb[LB];
-  auto load_global = [&]() {
+  // Register ring: the loads of step s+D are issued while step s is multiplied, so D-1 whole steps
+  // of work cover the memory latency of every load.
+  constexpr int D = 4;
+  v4i ra[D][LA], rb[D][LB];
+  auto load_global = [&](auto slot_c) {
+    constexpr int slot = decltype(slot_c)::value;
     const bool k_ok = k_lin < p.K;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
@@ -145,7 +129,7 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
       } else {
         if (k_ok && a_ok[i]) v = *reinterpret_cast<const v4i *>(a_ptr[i] + k_lin);
       }
-      ra[i] = v;
+      ra[slot][i] = v;
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
@@ -160,7 +144,7 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
       } else {
         if (k_ok && b_ok[i]) v = *reinterpret_cast<const v4i *>(b_ptr[i] + k_lin);
       }
-      rb[i] = v;
+      rb[slot][i] = v;
     }
   };
   auto advance_k = [&]() {
@@ -176,18 +160,19 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
       while (kq >= p.kwq) { kq -= p.kwq; ++kr; }
     }
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](int buf, auto slot_c) {
+    constexpr int slot = decltype(slot_c)::value;
     int8_t *la = lds[buf];
     int8_t *lb = lds[buf] + BM * BK;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
       const int row = lr + 64 * i;
-      *reinterpret_cast<v4i *>(la + row * BK + swz(row, lc) * 16) = ra[i];
+      *reinterpret_cast<v4i *>(la + row * BK + swz(row, lc) * 16) = ra[slot][i];
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
       const int row = lr + 64 * i;
-      *reinterpret_cast<v4i *>(lb + row * BK + swz(row, lc) * 16) = rb[i];
+      *reinterpret_cast<v4i *>(lb + row * BK + swz(row, lc) * 16) = rb[slot][i];
     }
   };
 
@@ -200,20 +185,10 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
   const int nsteps = (p.K + BK - 1) / BK;
-  load_global();
-  advance_k();
-  store_lds(0);
-  __syncthreads();
-
   const int frow = lane & 31;   // operand row within a 32-row MFMA tile
   const int fhalf = lane >> 5;  // which 16-byte half of the 32-byte K slice
 
-  for (int step = 0; step < nsteps; ++step) {
-    const int buf = step & 1;
-    if (step + 1 < nsteps) {
-      load_global();
-      advance_k();
-    }
+  auto compute = [&](int buf) {
     const int8_t *la = lds[buf];
     const int8_t *lb = lds[buf] + BM * BK;
 #pragma unroll
@@ -236,105 +211,45 @@ __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict_
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
-    if (step + 1 < nsteps) store_lds(buf ^ 1);
+  };
+
+  // prologue: steps 0..D-1 in flight, step 0 into LDS
+  {
+    auto issue = [&](auto slot_c) {
+      if (decltype(slot_c)::value < nsteps) {
+        load_global(slot_c);
+        advance_k();
+      }
+    };
+    issue(std::integral_constant<int, 0>{});
+    issue(std::integral_constant<int, 1>{});
+    issue(std::integral_constant<int, 2>{});
+    issue(std::integral_constant<int, 3>{});
+    store_lds(0, std::integral_constant<int, 0>{});
     __syncthreads();
+  }
+  // one ring position: slot d held step `step` (already in LDS), so it is free for step+D
+  auto ring_step = [&](int step, auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    if (step >= nsteps) return;
+    if (step + D < nsteps) {
+      load_global(d_c);
+      advance_k();
+    }
+    compute(d & 1);
+    if (step + 1 < nsteps) store_lds((d + 1) & 1, std::integral_constant<int, (d + 1) % D>{});
+    __syncthreads();
+  };
+  for (int base = 0; base < nsteps; base += D) {
+    ring_step(base + 0, std::integral_constant<int, 0>{});
+    ring_step(base + 1, std::integral_constant<int, 1>{});
+    ring_step(base + 2, std::integral_constant<int, 2>{});
+    ring_step(base + 3, std::integral_constant<int, 3>{});
   }
 
   // ---- epilogue -------------------------------------------------------------------------------
-  // accumulator layout: lane holds column (lane&31), rows 8*(r/4) + 4*(lane>>5) + (r&3)
-  if constexpr (!VEC_EPI) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int n = n0 + wave_n * WN + j * 32 + frow;
-        if (n >= p.N) continue;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t m = m0 + wave_m * WM + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-          if (m >= p.M) continue;
-          const int64_t idx = m * p.N + n;
-          const int a = acc[i][j][r];
-          if (e.acc_out) e.acc_out[idx] = a;
-          epi_store(epi_value((float)a, idx, n, e), idx, e);
-        }
-      }
-    }
-  } else {
-    // N % 4 == 0 and all pointers 16-byte aligned (checked on the host)
-    constexpr int CPR = WN / 4;    // 4-channel groups per staged row
-    constexpr int RPI = 64 / CPR;  // rows the wave moves per iteration
-    int *stage = reinterpret_cast<int *>(lds_raw) + wave * 32 * EPI_STRIDE;
-    const int cg = lane % CPR, rsub = lane / CPR;
-    const int n = n0 + wave_n * WN + cg * 4;
-    const bool n_ok = n < p.N;
-    v4f div = {1.f, 1.f, 1.f, 1.f}, bias = {0.f, 0.f, 0.f, 0.f};
-    if (n_ok && e.chan_div) div = *reinterpret_cast<const v4f *>(e.chan_div + n);
-    if (n_ok && e.bias) bias = *reinterpret_cast<const v4f *>(e.bias + n);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
-      const int64_t mbase = m0 + wave_m * WM + i * 32;
-#pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it) {
-        const int row = it * RPI + rsub;
-        const int64_t m = mbase + row;
-        const v4i a = *reinterpret_cast<const v4i *>(stage + row * EPI_STRIDE + cg * 4);
-        if (!n_ok || m >= p.M) continue;
-        const int64_t idx = m * p.N + n;
-        if (e.acc_out) *reinterpret_cast<v4i *>(e.acc_out + idx) = a;
-        v4f res = {0.f, 0.f, 0.f, 0.f};
-        if (e.resid) res = *reinterpret_cast<const v4f *>(e.resid + idx);
-        float v[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float x = __builtin_ldexpf((float)a[t], e.exp2);
-          if (e.chan_div) x = x / div[t];
-          if (e.bias) x = x + bias[t];
-          if (e.resid) x = x + res[t];
-          if (e.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
-          if (e.act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
-          v[t] = x;
-        }
-        if (e.y) {
-          if (e.y_f16) {
-            __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
-                            __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
-            *reinterpret_cast<v2i *>(reinterpret_cast<__half *>(e.y) + idx) = *reinterpret_cast<v2i *>(h);
-          } else {
-            v4f o = {v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<v4f *>(reinterpret_cast<float *>(e.y) + idx) = o;
-          }
-        }
-        if (e.q) {
-          if (e.q_bw == 8) {
-            unsigned pk = 0;
-#pragma unroll
-            for (int t = 0; t < 4; ++t) pk |= (unsigned)(quant1<8>(v[t], e.q_scale, e.q_neg_pos) & 0xff) << (8 * t);
-            *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = pk;
-          } else {
-            v2i pk;
-            unsigned h[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) h[t] = (unsigned)quant1<16>(v[t], e.q_scale, e.q_neg_pos) & 0xffffu;
-            pk[0] = (int)(h[0] | (h[1] << 16));
-            pk[1] = (int)(h[2] | (h[3] << 16));
-            *reinterpret_cast<v2i *>(reinterpret_cast<int16_t *>(e.q) + idx) = pk;
-          }
-        }
-      }
-    }
-  }
-}
-
-static bool vec_epilogue_ok(int N, const EpiDev &e) {
-  return N % 4 == 0 && aligned16(e.chan_div) && aligned16(e.bias) && aligned16(e.resid) && aligned16(e.y) &&
-         aligned16(e.acc_out) && aligned16(e.q);
+  int *stage = reinterpret_cast<int *>(lds_raw) + wave * 32 * EPI_STRIDE;
+  igemm_epilogue<TM, TN, EPI>(acc, stage, m0 + wave_m * WM, n0 + wave_n * WN, lane, p, e);
 }
 
 template <int BM, int BN, int LOAD>
@@ -344,10 +259,14 @@ static int launch_igemm(const void *a, const void *b, IgemmParams p, const EpiDe
   const int64_t nb = tiles_m * p.tiles_n;
   if (nb > 0x7fffffff) return CATCHQ_ERR_SHAPE;
   p.nblocks = (int)nb;
-  if (vec_epilogue_ok(p.N, e))
-    igemm_i8_kernel<BM, BN, LOAD, true><<<(int)nb, 256, 0, s>>>((const int8_t *)a, (const int8_t *)b, p, e);
+  const int epi = pick_epilogue(p.N, e);
+  if (epi == EPI_SCALAR)
+    igemm_i8_kernel<BM, BN, LOAD, EPI_SCALAR><<<(int)nb, 256, 0, s>>>((const int8_t *)a, (const int8_t *)b, p, e);
+  else if (LOAD == LOAD_C4 && epi == EPI_Q8_RELU)  // the network stem: conv + ReLU feeding the next conv
+    igemm_i8_kernel<BM, BN, LOAD, (LOAD == LOAD_C4 ? EPI_Q8_RELU : EPI_VECTOR)><<<(int)nb, 256, 0, s>>>(
+        (const int8_t *)a, (const int8_t *)b, p, e);
   else
-    igemm_i8_kernel<BM, BN, LOAD, false><<<(int)nb, 256, 0, s>>>((const int8_t *)a, (const int8_t *)b, p, e);
+    igemm_i8_kernel<BM, BN, LOAD, EPI_VECTOR><<<(int)nb, 256, 0, s>>>((const int8_t *)a, (const int8_t *)b, p, e);
   return launch_status();
 }
 
@@ -366,12 +285,25 @@ static int pick_tile(const void *a, const void *b, const IgemmParams &p, const E
   return launch_igemm<64, 64, LOAD>(a, b, p, e, s);
 }
 
+// CATCHQ_NO_DMA=1 keeps every shape on the register-staged kernel (for A/B timing)
+static bool dma_enabled() {
+  static const bool on = [] {
+    const char *v = getenv("CATCHQ_NO_DMA");
+    return !(v && v[0] == '1');
+  }();
+  return on;
+}
+
 int gemm_nt_mfma_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e,
                     hipStream_t s) {
   IgemmParams p = {};
   p.M = M;
   p.N = (int)N;
   p.K = (int)K;
+  if (dma_enabled()) {
+    const int st = igemm_dma_launch(LOAD_GEMM, a, b, p, e, M * K, N * K, s);
+    if (st >= 0) return st;
+  }
   return pick_tile<LOAD_GEMM>(a, b, p, e, s);
 }
 
@@ -388,6 +320,10 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     return pick_tile<LOAD_C4>(x, w, p, e, s);
   }
   p.K = kh * kw * Ci;
+  if (dma_enabled()) {
+    const int st = igemm_dma_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci, (int64_t)Co * p.K, s);
+    if (st >= 0) return st;
+  }
   return pick_tile<LOAD_CONV>(x, w, p, e, s);
 }
 

@@ -15,6 +15,7 @@
 #include <c10/core/DeviceGuard.h>
 #include <torch/library.h>
 
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -183,6 +184,53 @@ Tensor as_f32_vec(const c10::optional<Tensor> &t, int64_t n, const char *name) {
   return t->to(at::kFloat).contiguous();
 }
 
+uint32_t version_of(const Tensor &t);
+
+// Correctly rounded reciprocals of a per-channel divisor vector, kept per divisor tensor (one
+// device-to-host copy the first time a tensor is seen).  Undefined when some divisor has an
+// all-ones significand: the kernels then divide (see catchq_epilogue_t::chan_rcp).
+struct RcpEntry {
+  c10::weak_intrusive_ptr<c10::TensorImpl> impl;
+  uint32_t version;
+  const void *ptr;
+  Tensor rcp;
+};
+std::mutex g_rcp_mutex;
+std::unordered_map<const c10::TensorImpl *, RcpEntry> g_rcp_cache;
+
+Tensor reciprocals_for(const Tensor &div) {
+  const c10::TensorImpl *key = div.unsafeGetTensorImpl();
+  {
+    std::lock_guard<std::mutex> lock(g_rcp_mutex);
+    auto it = g_rcp_cache.find(key);
+    if (it != g_rcp_cache.end()) {
+      const RcpEntry &r = it->second;
+      if (!r.impl.expired() && r.impl._unsafe_get_target() == key && r.version == version_of(div) &&
+          r.ptr == div.data_ptr())
+        return r.rcp;
+      g_rcp_cache.erase(it);
+    }
+  }
+  Tensor host = div.to(at::kCPU).contiguous();
+  const float *d = host.data_ptr<float>();
+  const int64_t n = host.numel();
+  std::vector<float> r(n);
+  bool usable = n > 0;
+  for (int64_t i = 0; i < n; ++i) {
+    uint32_t bits;
+    std::memcpy(&bits, &d[i], 4);
+    if ((bits & 0x7fffffu) == 0x7fffffu || !(d[i] > 0.0f) || !std::isfinite(d[i])) usable = false;
+    r[i] = 1.0f / d[i];  // IEEE division: correctly rounded
+  }
+  Tensor rcp;
+  if (usable) rcp = at::from_blob(r.data(), {n}, at::TensorOptions().dtype(at::kFloat)).to(div.device());
+  std::lock_guard<std::mutex> lock(g_rcp_mutex);
+  if (g_rcp_cache.size() > 4096) g_rcp_cache.clear();
+  g_rcp_cache.insert_or_assign(key, RcpEntry{c10::weak_intrusive_ptr<c10::TensorImpl>(div.getIntrusivePtr()),
+                                             version_of(div), div.data_ptr(), rcp});
+  return rcp;
+}
+
 // fills a catchq_epilogue_t; `keep` holds the temporaries alive until the launch is enqueued
 EpiOut prepare_epilogue(const EpiArgs &a, at::IntArrayRef out_shape, int64_t co, const at::TensorOptions &opts,
                         catchq_epilogue_t *e, std::vector<Tensor> *keep) {
@@ -191,7 +239,12 @@ EpiOut prepare_epilogue(const EpiArgs &a, at::IntArrayRef out_shape, int64_t co,
   TORCH_CHECK(a.exp2 >= -126 && a.exp2 <= 126, "position sum out of range");
   e->exp2 = (int)a.exp2;
   Tensor cd = as_f32_vec(a.chan_div, co, "chan_div"), bs = as_f32_vec(a.bias, co, "bias");
-  if (cd.defined()) { e->chan_div = cd.data_ptr<float>(); keep->push_back(cd); }
+  if (cd.defined()) {
+    e->chan_div = cd.data_ptr<float>();
+    keep->push_back(cd);
+    Tensor rcp = reciprocals_for(cd);
+    if (rcp.defined()) { e->chan_rcp = rcp.data_ptr<float>(); keep->push_back(rcp); }
+  }
   if (bs.defined()) { e->bias = bs.data_ptr<float>(); keep->push_back(bs); }
   if (a.resid.has_value() && a.resid->defined()) {
     TORCH_CHECK(a.resid->sizes() == out_shape && a.resid->scalar_type() == at::kFloat && a.resid->is_contiguous(),
@@ -448,8 +501,12 @@ std::shared_ptr<Prepared> prepared_for(const Tensor &weight, const Tensor &q_sca
 }
 
 void clear_cache_op() {
-  std::lock_guard<std::mutex> lock(g_cache_mutex);
-  g_cache.clear();
+  {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    g_cache.clear();
+  }
+  std::lock_guard<std::mutex> lock(g_rcp_mutex);
+  g_rcp_cache.clear();
 }
 
 Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, at::IntArrayRef padding,

@@ -114,10 +114,17 @@ int catchq_dequantize(const void *q, int bits, void *y, int y_dtype, int64_t n, 
  *   v = act(v)
  * then any of: y[r][c] = v (fp32, or fp16 by one RNE conversion); acc_out[r][c] = acc;
  * q[r][c] = sat(rne(v * q_scale * 2^-q_position)) for the next layer (q_bitwidth 8/16).
- * All fp32, no fused multiply-add, true division. */
+ * All fp32, no fused multiply-add between the steps, true division.
+ * chan_rcp (optional, only with chan_div) lets the kernels evaluate the division as
+ *   q = v*r; e = fma(-q, d, v); v/d = fma(e, r, q)      (r = chan_rcp[c], d = chan_div[c])
+ * which is the correctly rounded quotient, bit for bit the same as v / d, when r is the correctly
+ * rounded reciprocal of d, d's significand is not all ones and nothing under/overflows
+ * (Markstein's theorem).  The caller guarantees the first two; the kernels use the form only for
+ * -64 <= exp2 <= 64 and divide otherwise. */
 typedef struct catchq_epilogue {
   int exp2;
   const float *chan_div; /* device [co] or NULL */
+  const float *chan_rcp; /* device [co] or NULL: 1/chan_div[c] rounded to nearest (see below) */
   const float *bias;     /* device [co] or NULL */
   const float *resid;    /* device [rows, co] fp32 or NULL */
   int act;               /* CATCHQ_ACT_* */

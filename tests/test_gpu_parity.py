@@ -161,11 +161,40 @@ def test_gemm_i8_acc_and_epilogue(m, n, k):
     out = cabi.gemm_nt(ad, bd, exp2=-9, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=1)
     assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
     assert same_bits(orc.epilogue(acc, -9, div, bias, None, 1), out["y"].cpu().numpy())
+    # the same through the reciprocal form of the division
+    out = cabi.gemm_nt(ad, bd, exp2=-9, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=1,
+                       chan_rcp=cabi.dev(np.float32(1) / div))
+    assert same_bits(orc.epilogue(acc, -9, div, bias, None, 1), out["y"].cpu().numpy())
     out = cabi.gemm_nt(ad, bd, exp2=-9, bias=cabi.dev(bias), act=0, y_dtype=torch.float16, want_acc=False,
                        q_bw=8, q_pos=-2)
     y = orc.epilogue(acc, -9, None, bias, None, 0)
     assert same_bits(y.astype(np.float16), out["y"].cpu().numpy())
     assert same_bits(orc.quantize(y, 8, -2), out["q"].cpu().numpy())
+
+
+def test_division_by_reciprocal_is_exact():
+    """v/d evaluated as q=v*r, e=fma(-q,d,v), fma(e,r,q) with r = RN(1/d) must equal IEEE division bit
+    for bit: adversarial divisor significands x a wide set of dividends x several exponents."""
+    r = rng(77)
+    n = 256
+    mant = np.concatenate([[0, 1, 2, 3, 0x7ffffe, 0x7ffffd, 0x400000, 0x400001, 0x3fffff, 0x2aaaaa, 0x555555, 0x6db6db,
+                            0x7ff000, 0x000fff], r.integers(0, 0x7fffff, n - 14)]).astype(np.uint32)
+    expo = r.integers(125, 130, n).astype(np.uint32)  # divisors in [0.25, 8)
+    div = ((expo << 23) | mant).view(np.float32)
+    rcp = (np.float32(1) / div).astype(np.float32)
+    for k, m in ((16, 4096), (64, 2048), (1024, 512)):
+        a, b = _ints(r, (m, k), 8), _ints(r, (n, k), 8)
+        if k == 16:
+            a[:, 4:] = 0  # small sums: every short bit pattern shows up
+        acc, _ = orc.gemm_nt(a, b)
+        for exp2 in (-13, 0, 7, -64, 64):
+            note("div by rcp", k, m, exp2)
+            out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=exp2, chan_div=cabi.dev(div), chan_rcp=cabi.dev(rcp),
+                               want_acc=False)
+            assert same_bits(orc.epilogue(acc, exp2, div), out["y"].cpu().numpy())
+    # outside the exponent window the kernels divide even when reciprocals are supplied
+    out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=-90, chan_div=cabi.dev(div), chan_rcp=cabi.dev(rcp * 0))
+    assert same_bits(orc.epilogue(acc, -90, div), out["y"].cpu().numpy())
 
 
 @pytest.mark.parametrize("bits", [(16, 8), (16, 16)])
@@ -248,7 +277,7 @@ def test_conv_i8_acc_and_epilogue(case):
     resid = r.standard_normal(acc.shape).astype(np.float32)
     xd, wd = cabi.dev(x), cabi.dev(wt)
     out = cabi.conv2d_nhwc(xd, wd, pad, stride, dil, g, exp2=-10, chan_div=cabi.dev(div), bias=cabi.dev(bias),
-                           resid=cabi.dev(resid), act=1, q_bw=8, q_pos=-3)
+                           resid=cabi.dev(resid), act=1, q_bw=8, q_pos=-3, chan_rcp=cabi.dev(np.float32(1) / div))
     assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
     y = orc.epilogue(acc, -10, div, bias, resid, 1)
     assert same_bits(y, out["y"].cpu().numpy())
