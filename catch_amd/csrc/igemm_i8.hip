@@ -320,7 +320,7 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     return pick_tile<LOAD_C4>(x, w, p, e, s);
   }
   p.K = kh * kw * Ci;
-  if (dma_enabled()) {
+  if (dma_enabled() && kh * kw <= 32) {  // the DMA loader keeps one validity bit per filter tap
     const int st = igemm_dma_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci, (int64_t)Co * p.K, s);
     if (st >= 0) return st;
   }
