@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0
+# HBM bytes moved by the igemm launches of one ResNet-50 bs64 step, from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy in the same runs):
+# 2.262e9 read + 2.196e9 written.  Valid for the default workload only.
+MEASURED_TRAFFIC_BYTES = {("resnet50", 64): 4.459e9}
 
 
 def parse():
@@ -38,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 1 GiB device copy (reference dispatch for scaling rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
@@ -106,6 +113,12 @@ def main():
     import catch_amd  # noqa: F401  (fails loudly if the HIP extension is missing)
     from catch_amd import nets, pipeline
 
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     batch = args.batch or {"resnet50": 64, "resnet18": 64, "mobilenet_v2": 128}[args.workload]
     layers = nets.NETS[args.workload]()
     net = nets.FloatNet(layers, seed=0).eval()
@@ -146,7 +159,8 @@ def main():
         print("sum of conv/fc launches: %.1f us; graph step: %.1f us" % (t_all * 1e6, ms_per_step * 1e3), file=sys.stderr)
     roofline = {"bound": "hbm", "kernel": "igemm_i8_kernel (all %d launches of one step)" % len(conv_rows),
                 "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, batch)),
                 "avg_launch_us": round(t_conv / max(len(conv_rows), 1) * 1e6, 2),
                 "algorithmic_bytes_per_step": b_conv, "int8_tops": round(o_conv / t_conv / 1e12, 1),
                 "mfma_frac": round(o_conv / t_conv / 1e12 / INT8_PEAK_TOPS, 4)}
