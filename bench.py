@@ -83,10 +83,10 @@ def layer_profile(fused, x, iters=20):
 
             def run(l=l, lq=lq, qx=qx, qd=qd, want_y=want_y, resid=resid):
                 return ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
-                                   [l.stride, l.stride], [1, 1], l.groups, {"none": 0, "relu": 1, "relu6": 2}[l.act],
+                                   [l.stride, l.stride], [1, 1], lq.groups, {"none": 0, "relu": 1, "relu6": 2}[l.act],
                                    want_y, False, False, qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
             route = ops.conv2d_route(8, 8, list(qx.shape), list(lq.qw.shape[:3]) + [lq.qw.shape[3]],
-                                     [l.pad, l.pad], [l.stride, l.stride], [1, 1], l.groups)
+                                     [l.pad, l.pad], [l.stride, l.stride], [1, 1], lq.groups)
         else:
             def run(lq=lq, qx=qx):
                 return ops.qlinear(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, False, 0, 0, 1.0)

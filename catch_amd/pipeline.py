@@ -37,10 +37,20 @@ def pos_from_scale(bw, scale):
 
 class _LayerQ(object):
     """decoded q-params and the quantized weight of one conv / fc layer"""
-    __slots__ = ("bw_x", "bw_w", "pos_x", "pos_w", "qw", "chan_div", "bias", "exp2", "cpad")
+    __slots__ = ("bw_x", "bw_w", "pos_x", "pos_w", "qw", "chan_div", "bias", "exp2", "cpad", "groups")
 
 
-def _decode(layer, sd, device):
+def _pad16(c):
+    """device-side channel count of a tensor with c channels: the matrix-core route wants multiples
+    of 16 (a 16-byte K chunk must not straddle filter taps); 1..3 channel inputs take 4"""
+    if c <= 4:
+        return 4 if c < 4 else c
+    return (c + 15) // 16 * 16
+
+
+def _decode(layer, sd, device, ci_dev, co_dev):
+    """ci_dev / co_dev: channel counts of the layer's input / output tensors as laid out on the
+    device (>= the real counts; extra channels are zeros: zero weights, zero bias, divisor 1)."""
     q = _LayerQ()
     k = _key(layer.name)
     w = sd[k + "weight"].to(device=device, dtype=torch.float32)
@@ -67,14 +77,28 @@ def _decode(layer, sd, device):
         q.pos_x, q.pos_w = int(mode[0]), int(mode[1])
         qw = torch.ops.torch_mlu.quantize(w, q.bw_w, q.pos_w)
     q.exp2 = q.pos_x + q.pos_w
-    q.cpad = 0
+    q.cpad = ci_dev
+    pad = torch.nn.functional.pad
+    co = qw.shape[0]
     if layer.kind == "conv":
         qw = qw.permute(0, 2, 3, 1)  # [Co,kh,kw,Ci/g] view of the same memory
-        if layer.groups == 1 and layer.ci < 4:  # few-channel network input: pad channels to 4 (zeros)
-            q.cpad = 4
-            qw = torch.nn.functional.pad(qw, (0, 4 - layer.ci))
-        qw = qw.contiguous()
-    q.qw = qw
+        depthwise = layer.groups > 1 and layer.groups == layer.ci == layer.co
+        if layer.groups == 1 and ci_dev != layer.ci:
+            qw = pad(qw, (0, ci_dev - layer.ci))
+        if layer.groups > 1 and not depthwise and (ci_dev != layer.ci or co_dev != co):
+            raise ValueError("grouped convolution %s needs unpadded channels" % layer.name)
+        q.groups = co_dev if depthwise else layer.groups
+    else:
+        if ci_dev != layer.ci:
+            qw = pad(qw, (0, ci_dev - layer.ci))
+        q.groups = 1
+    if co_dev != co:  # zero filters for the padding channels
+        qw = pad(qw, (0, 0) * (qw.dim() - 1) + (0, co_dev - co))
+        if q.bias is not None:
+            q.bias = pad(q.bias, (0, co_dev - co))
+        if q.chan_div is not None:
+            q.chan_div = pad(q.chan_div, (0, co_dev - co), value=1.0)
+    q.qw = qw.contiguous()
     return q
 
 
@@ -84,7 +108,22 @@ class FusedNet(object):
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
         self.out_half = out_half
-        self.q = {l.name: _decode(l, state_dict, self.device) for l in self.layers if l.kind in ("conv", "fc")}
+        # channel counts: real (chan) and as laid out on the device (cdev)
+        self.chan, self.cdev = {"input": self.layers[0].ci}, {"input": _pad16(self.layers[0].ci)}
+        for l in self.layers:
+            if l.kind == "conv":
+                self.chan[l.name], self.cdev[l.name] = l.co, _pad16(l.co)
+            elif l.kind == "fc":
+                self.chan[l.name] = self.cdev[l.name] = l.co
+            elif l.kind == "concat":
+                for s_ in l.src:
+                    if self.chan[s_] != self.cdev[s_]:
+                        raise ValueError("concat %s: source %s has padded channels" % (l.name, s_))
+                self.chan[l.name] = self.cdev[l.name] = sum(self.chan[s_] for s_ in l.src)
+            else:
+                self.chan[l.name], self.cdev[l.name] = self.chan[l.src], self.cdev[l.src]
+        self.q = {l.name: _decode(l, state_dict, self.device, self.cdev[l.src], self.cdev[l.name])
+                  for l in self.layers if l.kind in ("conv", "fc")}
         self._plan_demands()
         self._graph = None
 
@@ -126,9 +165,7 @@ class FusedNet(object):
         env = {}
         tracing = trace is not None
         for d in self.q_demand["input"]:
-            first = self.layers[0]
-            cpad = self.q[first.name].cpad if first.kind == "conv" else 0
-            env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], cpad)
+            env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"])
         for l in self.layers:
             name = l.name
             if l.kind == "conv":
@@ -138,7 +175,7 @@ class FusedNet(object):
                 qd = self.q_demand[name][0] if self.q_demand[name] else None
                 want_y = self.f_demand[name] or tracing or qd is None
                 y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
-                                        [l.stride, l.stride], [1, 1], l.groups, _ACT_CODE[l.act], want_y,
+                                        [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
                                         self.out_half and name in self.outputs, tracing,
                                         qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
                 if want_y:
@@ -177,7 +214,9 @@ class FusedNet(object):
         outs = []
         for o in self.outputs:
             y = env[(o, "f")]
-            outs.append(y.permute(0, 3, 1, 2) if y.dim() == 4 else y)  # logical NCHW over NHWC memory
+            if y.dim() == 4:  # logical NCHW over NHWC memory, padding channels dropped
+                y = y.permute(0, 3, 1, 2)[:, :self.chan[o]]
+            outs.append(y)
         return outs[0] if len(outs) == 1 else tuple(outs)
 
     __call__ = forward

@@ -39,14 +39,15 @@ def check_against_oracle(layers, sd, x, fused):
             continue
         r, g = rec[l.name], trace[l.name]
         assert r["overflow"] == 0, l.name
-        qx = g["qx"].cpu().numpy()
-        if qx.ndim == 4 and qx.shape[-1] != r["qx"].shape[-1]:  # channel-padded network input
-            assert not qx[..., r["qx"].shape[-1]:].any()
-            qx = qx[..., :r["qx"].shape[-1]]
-        assert np.array_equal(r["qx"].reshape(qx.shape), qx), "quantized input of " + l.name
-        assert np.array_equal(r["acc"].astype(np.int32), g["acc"].cpu().numpy().reshape(r["acc"].shape)), \
-            "accumulators of " + l.name
-        assert np.array_equal(r["y"].reshape(-1), g["y"].float().cpu().numpy().reshape(-1)), "output of " + l.name
+        def real(t, want):  # drop the zero channels the device layout pads with
+            t = t.cpu().numpy()
+            if t.shape[-1] != want.shape[-1]:
+                assert not t[..., want.shape[-1]:].any(), "padding channels of %s are not zero" % l.name
+                t = t[..., :want.shape[-1]]
+            return t.reshape(want.shape)
+        assert np.array_equal(r["qx"], real(g["qx"], r["qx"])), "quantized input of " + l.name
+        assert np.array_equal(r["acc"].astype(np.int32), real(g["acc"], r["acc"])), "accumulators of " + l.name
+        assert np.array_equal(r["y"], real(g["y"].float(), r["y"])), "output of " + l.name
     outs = out if isinstance(out, tuple) else (out,)
     for name, o in zip(fused.outputs, outs):
         want = t[name]
@@ -91,6 +92,19 @@ def test_resnet50_small_batch_and_graph_replay():
         assert torch.equal(out, logits), "replay %d" % i
         _ = fused.forward(torch.randn(2, 3, 112, 112, device="cuda"))
         torch.cuda.synchronize()
+
+
+def test_mobilenet_v2_small():
+    """MobileNetV2: depthwise stencil kernel, ReLU6, linear bottlenecks with residual adds, channel
+    counts (24, 144) that the device layout pads to multiples of 16."""
+    note("mobilenet_v2 bs2 96x96")
+    layers = nets.mobilenet_v2()
+    net = nets.FloatNet(layers, seed=5, weight_std=0.2).eval()
+    x = torch.randn(2, 3, 96, 96, generator=torch.Generator().manual_seed(6))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd)
+    assert fused.cdev["b1.proj"] == 32 and fused.chan["b1.proj"] == 24
+    check_against_oracle(layers, sd, x, fused)
 
 
 def test_dropin_modules_match_fused_pipeline():
