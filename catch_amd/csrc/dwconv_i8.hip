@@ -1,8 +1,14 @@
 // Depthwise int8 convolution (groups == Ci == Co) on NHWC tensors: a stencil, not a contraction,
-// so no matrix cores.  A block owns a strip of output pixels of one image row and all channels of a
+// so no matrix cores.  Two kernels:
+//  * dw3x3_kernel: 3x3, dilation 1, stride 1 or 2 (every depthwise layer of the MobileNet family).
+//    A lane owns 4 channels x (2 rows x 4 columns) of output pixels, slides the input window through
+//    registers and finishes with the vector epilogue of the GEMM kernels; adjacent lanes hold adjacent
+//    channel quads, so loads and stores of a wave are contiguous runs of the NHWC row.
+//  * dwconv_i8_kernel: any filter up to 5x5, any stride/dilation.  A block owns a strip of output pixels of one image row and all channels of a
 // 64-channel slab; the input rows the strip needs are staged in LDS once and every tap is read
 // from there, the filter taps of the slab sit in LDS transposed to [tap][channel].
 #include "catchq_common.h"
+#include "igemm_common.h"
 
 namespace catchq {
 
@@ -87,6 +93,127 @@ __global__ __launch_bounds__(256) void dwconv_i8_kernel(const int8_t *__restrict
   }
 }
 
+struct Dw3Params {
+  int N, H, W, C, ph, pw, Ho, Wo;
+  int CQ;     // channel quads
+  int WG;     // column groups per output row
+  int items;  // WG * CQ
+};
+
+constexpr int DW3_PW = 4, DW3_PH = 2;
+
+template <int S, int EPI>
+__global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x, const int8_t *__restrict__ w,
+                                                   Dw3Params p, EpiDev e) {
+  typedef typename EpiOf<EPI>::type Sp;
+  constexpr int PW = DW3_PW, PH = DW3_PH;
+  constexpr int NC = (PW - 1) * S + 3;  // input columns of the window
+  constexpr int NR = (PH - 1) * S + 3;  // input rows of the window
+  const int item = blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.items) return;
+  const int wg = item / p.CQ, cq = item - wg * p.CQ;
+  const int ho0 = blockIdx.y * PH, img = blockIdx.z;
+  const int c = cq * 4;
+
+  // 36 filter bytes of the four channels ([channel][tap]) -> sign-extended taps
+  int wraw[9];
+#pragma unroll
+  for (int i = 0; i < 9; ++i) wraw[i] = *reinterpret_cast<const int *>(w + (int64_t)c * 9 + 4 * i);
+  int wu[9][4];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int b = j * 9 + t;
+      wu[t][j] = (int)(int8_t)(wraw[b >> 2] >> (8 * (b & 3)));
+    }
+
+  int acc[PH][PW][4];
+#pragma unroll
+  for (int a = 0; a < PH; ++a)
+#pragma unroll
+    for (int b = 0; b < PW; ++b)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[a][b][j] = 0;
+
+  const int hi0 = ho0 * S - p.ph, wi0 = wg * PW * S - p.pw;
+  const int8_t *xi = x + (int64_t)img * p.H * p.W * p.C + c;
+#pragma unroll
+  for (int ri = 0; ri < NR; ++ri) {
+    const int hi = hi0 + ri;
+    const bool row_ok = (unsigned)hi < (unsigned)p.H;
+    int xr[NC];
+#pragma unroll
+    for (int col = 0; col < NC; ++col) {
+      const int wi = wi0 + col;
+      xr[col] = 0;
+      if (row_ok && (unsigned)wi < (unsigned)p.W)
+        xr[col] = *reinterpret_cast<const int *>(xi + ((int64_t)hi * p.W + wi) * p.C);
+    }
+#pragma unroll
+    for (int col = 0; col < NC; ++col) {
+      int xs[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xs[j] = (int)(int8_t)(xr[col] >> (8 * j));
+#pragma unroll
+      for (int py = 0; py < PH; ++py) {
+        const int r = ri - py * S;
+        if (r < 0 || r > 2) continue;
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+          const int d = col - q;
+          if (d < 0 || d % S != 0 || d / S >= PW) continue;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[py][d / S][j] += xs[j] * wu[r * 3 + q][j];
+        }
+      }
+    }
+  }
+
+  const EpiLane L = epi_lane_setup<Sp>(c, true, e);
+#pragma unroll
+  for (int py = 0; py < PH; ++py) {
+    const int ho = ho0 + py;
+    if (ho >= p.Ho) continue;
+#pragma unroll
+    for (int px = 0; px < PW; ++px) {
+      const int wo = wg * PW + px;
+      if (wo >= p.Wo) continue;
+      const int64_t idx = (((int64_t)img * p.Ho + ho) * p.Wo + wo) * p.C + c;
+      v4f res = {0.f, 0.f, 0.f, 0.f};
+      if (L.use_res) res = *reinterpret_cast<const v4f *>(e.resid + idx);
+      const v4i a = {acc[py][px][0], acc[py][px][1], acc[py][px][2], acc[py][px][3]};
+      epi_vec4<Sp>(a, res, L, idx, e);
+    }
+  }
+}
+
+template <int S, int EPI>
+static void dw3x3_launch(const void *x, const void *w, const Dw3Params &p, dim3 grid, const EpiDev &e, hipStream_t s) {
+  dw3x3_kernel<S, EPI><<<grid, 256, 0, s>>>((const int8_t *)x, (const int8_t *)w, p, e);
+}
+
+// 0 when launched, -1 when the shape is not this kernel's
+static int dw3x3(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
+                 int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
+  if (kh != 3 || kw != 3 || dh != 1 || dw != 1 || sh != sw || (sh != 1 && sh != 2)) return -1;
+  const int epi = pick_epilogue(C, e);
+  if (epi == EPI_SCALAR) return -1;
+  Dw3Params p = {N, H, W, C, ph, pw, Ho, Wo, C / 4, (Wo + DW3_PW - 1) / DW3_PW, 0};
+  const int64_t items = (int64_t)p.WG * p.CQ;
+  const int rows = (Ho + DW3_PH - 1) / DW3_PH;
+  if (items > 0x7fffff00 || rows > 65535 || N > 65535) return -1;
+  p.items = (int)items;
+  const dim3 grid((unsigned)((items + 255) / 256), (unsigned)rows, (unsigned)N);
+  const bool s2 = sh == 2;
+  switch (epi) {
+    case EPI_Q8_RELU6: s2 ? dw3x3_launch<2, EPI_Q8_RELU6>(x, w, p, grid, e, s) : dw3x3_launch<1, EPI_Q8_RELU6>(x, w, p, grid, e, s); break;
+    case EPI_Q8_RELU: s2 ? dw3x3_launch<2, EPI_Q8_RELU>(x, w, p, grid, e, s) : dw3x3_launch<1, EPI_Q8_RELU>(x, w, p, grid, e, s); break;
+    default: s2 ? dw3x3_launch<2, EPI_VECTOR>(x, w, p, grid, e, s) : dw3x3_launch<1, EPI_VECTOR>(x, w, p, grid, e, s); break;
+  }
+  return 0;
+}
+
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw) {
   if (C % 4 != 0 || kh * kw > DW_MAXTAPS) return false;
   const int in_w = (DW_TW - 1) * sw + (kw - 1) * dw + 1;
@@ -95,6 +222,7 @@ bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw) {
 
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
+  if (dw3x3(x, w, N, H, W, C, kh, kw, ph, pw, sh, sw, dh, dw, Ho, Wo, e, s) == 0) return launch_status();
   DwParams p = {N, H, W, C, kh, kw, ph, pw, sh, sw, dh, dw, Ho, Wo, 0, 0};
   p.strips = (Wo + DW_TW - 1) / DW_TW;
   p.slabs = (C + DW_CS - 1) / DW_CS;

@@ -95,6 +95,88 @@ inline int pick_epilogue(int N, const EpiDev &e) {
   return EPI_VECTOR;
 }
 
+// per-channel constants of one lane's four consecutive channels
+struct EpiLane {
+  v4f div, rcp, bias;
+  bool use_rcp, use_div, use_bias, use_res, unit_q;
+  int act;
+};
+
+template <class S>
+__device__ __forceinline__ EpiLane epi_lane_setup(int n, bool n_ok, const EpiDev &e) {
+  EpiLane L;
+  L.use_rcp = S::rcp(e); L.use_div = S::truediv(e); L.use_bias = S::bias(e); L.use_res = S::resid(e);
+  L.act = S::act(e);
+  L.unit_q = S::kGeneric ? (e.q_scale == 1.0f) : true;
+  // Reciprocal form with the power of two folded in:
+  //   v = (f*2^e)/d  ==  q = f*(r*2^e); err = fma(-q, d*2^-e, f); fma(err, r*2^e, q)
+  // (scaling by 2^e is exact, so every intermediate is the scaled image of the unfolded one)
+  L.div = v4f{1.f, 1.f, 1.f, 1.f}; L.rcp = v4f{1.f, 1.f, 1.f, 1.f}; L.bias = v4f{0.f, 0.f, 0.f, 0.f};
+  if (n_ok && (L.use_rcp || L.use_div)) L.div = *reinterpret_cast<const v4f *>(e.chan_div + n);
+  if (n_ok && L.use_rcp) {
+    L.rcp = *reinterpret_cast<const v4f *>(e.chan_rcp + n);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      L.rcp[t] = __builtin_ldexpf(L.rcp[t], e.exp2);
+      L.div[t] = __builtin_ldexpf(L.div[t], -e.exp2);
+    }
+  }
+  if (n_ok && L.use_bias) L.bias = *reinterpret_cast<const v4f *>(e.bias + n);
+  return L;
+}
+
+// four integer sums of one pixel (channels n..n+3, linear index idx) -> all requested outputs
+template <class S>
+__device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLane &L, int64_t idx, const EpiDev &e) {
+  if (S::acc(e)) *reinterpret_cast<v4i *>(e.acc_out + idx) = a;
+  float v[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    float x = (float)a[t];
+    if (L.use_rcp) x = div_by_rcp(x, L.div[t], L.rcp[t]);
+    else {
+      x = __builtin_ldexpf(x, e.exp2);
+      if (L.use_div) x = x / L.div[t];
+    }
+    if (L.use_bias) x = x + L.bias[t];
+    if (L.use_res) x = x + res[t];
+    if (L.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
+    if (L.act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
+    v[t] = x;
+  }
+  if (S::y16(e)) {
+    __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
+                    __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
+    *reinterpret_cast<v2i *>(reinterpret_cast<__half *>(e.y) + idx) = *reinterpret_cast<v2i *>(h);
+  } else if (S::y32(e)) {
+    v4f o = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<v4f *>(reinterpret_cast<float *>(e.y) + idx) = o;
+  }
+  if (S::q8(e)) {
+    int b[4];
+    if (L.unit_q) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) b[t] = quant1_unit<8>(v[t], e.q_neg_pos);
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) b[t] = quant1<8>(v[t], e.q_scale, e.q_neg_pos);
+    }
+    // four clamped values -> four bytes: two byte permutes and a merge
+    const unsigned lo = __builtin_amdgcn_perm((unsigned)b[1], (unsigned)b[0], 0x0c0c0400u);
+    const unsigned hi = __builtin_amdgcn_perm((unsigned)b[3], (unsigned)b[2], 0x04000c0cu);
+    *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = lo | hi;
+  } else if (S::q16(e)) {
+    v2i pk;
+    unsigned h[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      h[t] = (unsigned)(L.unit_q ? quant1_unit<16>(v[t], e.q_neg_pos) : quant1<16>(v[t], e.q_scale, e.q_neg_pos)) & 0xffffu;
+    pk[0] = (int)(h[0] | (h[1] << 16));
+    pk[1] = (int)(h[2] | (h[3] << 16));
+    *reinterpret_cast<v2i *>(reinterpret_cast<int16_t *>(e.q) + idx) = pk;
+  }
+}
+
 // Epilogue of one wave.  acc[i][j] are 32x32 MFMA tiles: lane holds column (lane&31) and rows
 // 8*(r/4) + 4*(lane>>5) + (r&3).  (m_w, n_w) = global row / column of the wave tile's origin.
 // Vector variants: the wave transposes 32 rows at a time through its private LDS area `stage` so
@@ -130,23 +212,8 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
     const int cg = lane % CPR, rsub = lane / CPR;
     const int n = n_w + cg * 4;
     const bool n_ok = n < p.N;
-    const bool use_rcp = S::rcp(e), use_div = S::truediv(e), use_bias = S::bias(e), use_res = S::resid(e);
-    const int act = S::act(e);
-    // per-channel constants of this lane.  Reciprocal form with the power of two folded in:
-    //   v = (f*2^e)/d  ==  q = f*(r*2^e); err = fma(-q, d*2^-e, f); fma(err, r*2^e, q)
-    // (scaling by 2^e is exact, so every intermediate is the scaled image of the unfolded one)
-    v4f div = {1.f, 1.f, 1.f, 1.f}, rcp = {1.f, 1.f, 1.f, 1.f}, bias = {0.f, 0.f, 0.f, 0.f};
-    if (n_ok && (use_rcp || use_div)) div = *reinterpret_cast<const v4f *>(e.chan_div + n);
-    if (n_ok && use_rcp) {
-      rcp = *reinterpret_cast<const v4f *>(e.chan_rcp + n);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        rcp[t] = __builtin_ldexpf(rcp[t], e.exp2);
-        div[t] = __builtin_ldexpf(div[t], -e.exp2);
-      }
-    }
-    if (n_ok && use_bias) bias = *reinterpret_cast<const v4f *>(e.bias + n);
-    const bool unit_q = S::kGeneric ? (e.q_scale == 1.0f) : true;
+    const EpiLane L = epi_lane_setup<S>(n, n_ok, e);
+    const bool use_res = L.use_res;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       // residual rows of this 32-row block: all loads in flight before the staging below
@@ -173,53 +240,7 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
         const v4i a = *reinterpret_cast<const v4i *>(stage + row * EPI_STRIDE + cg * 4);
         if (!n_ok || m >= p.M) continue;
         const int64_t idx = m * p.N + n;
-        if (S::acc(e)) *reinterpret_cast<v4i *>(e.acc_out + idx) = a;
-        float v[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float x = (float)a[t];
-          if (use_rcp) x = div_by_rcp(x, div[t], rcp[t]);
-          else {
-            x = __builtin_ldexpf(x, e.exp2);
-            if (use_div) x = x / div[t];
-          }
-          if (use_bias) x = x + bias[t];
-          if (use_res) x = x + resv[it][t];
-          if (act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
-          if (act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
-          v[t] = x;
-        }
-        if (S::y16(e)) {
-          __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
-                          __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
-          *reinterpret_cast<v2i *>(reinterpret_cast<__half *>(e.y) + idx) = *reinterpret_cast<v2i *>(h);
-        } else if (S::y32(e)) {
-          v4f o = {v[0], v[1], v[2], v[3]};
-          *reinterpret_cast<v4f *>(reinterpret_cast<float *>(e.y) + idx) = o;
-        }
-        if (S::q8(e)) {
-          int b[4];
-          if (unit_q) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) b[t] = quant1_unit<8>(v[t], e.q_neg_pos);
-          } else {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) b[t] = quant1<8>(v[t], e.q_scale, e.q_neg_pos);
-          }
-          // four clamped values -> four bytes: two byte permutes and a merge
-          const unsigned lo = __builtin_amdgcn_perm((unsigned)b[1], (unsigned)b[0], 0x0c0c0400u);
-          const unsigned hi = __builtin_amdgcn_perm((unsigned)b[3], (unsigned)b[2], 0x04000c0cu);
-          *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = lo | hi;
-        } else if (S::q16(e)) {
-          v2i pk;
-          unsigned h[4];
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-            h[t] = (unsigned)(unit_q ? quant1_unit<16>(v[t], e.q_neg_pos) : quant1<16>(v[t], e.q_scale, e.q_neg_pos)) & 0xffffu;
-          pk[0] = (int)(h[0] | (h[1] << 16));
-          pk[1] = (int)(h[2] | (h[3] << 16));
-          *reinterpret_cast<v2i *>(reinterpret_cast<int16_t *>(e.q) + idx) = pk;
-        }
+        epi_vec4<S>(a, use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, idx, e);
       }
     }
   }

@@ -260,6 +260,10 @@ CONV_CASES = [
     (1, 8, 10, 10, 8, 3, 3, (1, 1), (2, 2), (1, 1), 8),        # depthwise, few channels
     (1, 36, 40, 40, 36, 5, 5, (2, 2), (1, 1), (1, 1), 36),     # depthwise 5x5, several strips
     (1, 6, 7, 7, 6, 3, 3, (1, 1), (1, 1), (1, 1), 6),          # depthwise C%4 != 0 -> direct
+    (1, 16, 9, 7, 16, 3, 3, (0, 0), (1, 1), (1, 1), 16),       # depthwise, no padding, ragged 2x4 windows
+    (2, 24, 11, 13, 24, 3, 3, (1, 1), (2, 2), (1, 1), 24),     # depthwise s2, odd extents
+    (1, 320, 7, 7, 320, 3, 3, (1, 1), (1, 1), (1, 1), 320),    # depthwise, many channels, tiny image
+    (1, 16, 9, 9, 16, 3, 3, (2, 2), (1, 1), (2, 2), 16),       # depthwise dilated -> strip kernel
 ]
 
 
