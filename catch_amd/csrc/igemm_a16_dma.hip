@@ -1,0 +1,318 @@
+// int16 activations x int8 weights on the int8 matrix cores, LDS-DMA pipelined.
+//
+// An int16 value splits exactly into two int8 digits and a constant:
+//     x = 256*hi + lo_s + 128,    hi = x >> 8  (signed high byte),   lo_s = (x & 255) - 128,
+// so   sum_k x_k*w_k = 256 * sum hi_k*w_k  +  sum lo_s_k*w_k  +  128 * sum_k w_k.
+// The two digit sums are int8 x int8 MFMA accumulations, the last term is a per-output-channel
+// constant that a wave collects from the weight fragments it loads anyway (v_dot4 with all-ones).
+// A zero written by the hardware for an out-of-image tap or a row beyond M decodes to
+// (hi, lo_s) = (0, -128), i.e. to x = 0 after the constant is added, so the convolution's zero
+// padding needs no special case; the same identity makes whatever the weight operand holds beyond
+// K irrelevant.  All three terms are accumulated modulo 2^32, so the result is exact whenever the
+// true sum fits an int32 (the precondition of the int16 x int8 contraction).
+//
+// The split happens in registers, between the LDS fetch and the MFMA: activations stay plain
+// int16 NHWC in memory.  A-tile rows are 128 bytes (64 int16 of K) = eight 16-byte chunks, the
+// chunk index XOR-ed with row&7; weight rows keep the 64-byte layout of the int8 kernel.
+#include "igemm_i8_dma.inc"
+
+namespace catchq {
+
+// 16 consecutive int16 (two 16-byte chunks) -> their high bytes and their biased low bytes
+__device__ __forceinline__ void split_i16(const v4i c0, const v4i c1, v4i &hi, v4i &lo) {
+  hi[0] = (int)__builtin_amdgcn_perm((unsigned)c0[1], (unsigned)c0[0], 0x07050301u);
+  hi[1] = (int)__builtin_amdgcn_perm((unsigned)c0[3], (unsigned)c0[2], 0x07050301u);
+  hi[2] = (int)__builtin_amdgcn_perm((unsigned)c1[1], (unsigned)c1[0], 0x07050301u);
+  hi[3] = (int)__builtin_amdgcn_perm((unsigned)c1[3], (unsigned)c1[2], 0x07050301u);
+  lo[0] = (int)(__builtin_amdgcn_perm((unsigned)c0[1], (unsigned)c0[0], 0x06040200u) ^ 0x80808080u);
+  lo[1] = (int)(__builtin_amdgcn_perm((unsigned)c0[3], (unsigned)c0[2], 0x06040200u) ^ 0x80808080u);
+  lo[2] = (int)(__builtin_amdgcn_perm((unsigned)c1[1], (unsigned)c1[0], 0x06040200u) ^ 0x80808080u);
+  lo[3] = (int)(__builtin_amdgcn_perm((unsigned)c1[3], (unsigned)c1[2], 0x06040200u) ^ 0x80808080u);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int LOAD, int EPI>
+__global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(const int16_t *__restrict__ A,
+                                                                            const int8_t *__restrict__ B,
+                                                                            IgemmParams p, EpiDev e,
+                                                                            unsigned a_bytes, unsigned b_bytes) {
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_STAGE = BM * BK * 2, B_STAGE = BN * BK;
+  constexpr int STAGE_BYTES = A_STAGE + B_STAGE;
+  constexpr int PIPE_BYTES = STAGES * STAGE_BYTES;
+  constexpr int NIA = BM / 8, NIB = BN / 16;  // DMA instructions (1 KiB each) per stage: A, B
+  constexpr int NI = (NIA + NIB) / NW;        // per wave
+  static_assert((NIA + NIB) % NW == 0, "tile rows must split evenly over the waves");
+  static_assert(STAGES >= 3, "the ring needs at least three stages");
+  constexpr int EPI_STRIDE = WN + 8;
+  extern __shared__ __attribute__((aligned(16))) int8_t lds_dyn[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+
+  const int logical = xcd_remap(blockIdx.x, p.nblocks);
+  const int tile_n = logical % p.tiles_n;
+  const int tile_m = logical / p.tiles_n;
+  const int64_t m0 = (int64_t)tile_m * BM;
+  const int n0 = tile_n * BN;
+
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A, 0, (int)a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)B, 0, (int)b_bytes, 0x00020000);
+  constexpr unsigned OOB = 0x80000000u;
+
+  // ---- loader state -----------------------------------------------------------------------------
+  // A instruction: 8 tile rows x 8 chunks (lane -> row lane/8, physical chunk lane%8);
+  // B instruction: 16 tile rows x 4 chunks (lane -> row lane/4, physical chunk lane%4).
+  unsigned rowbase[NI];  // byte offset of the row's K origin
+  unsigned vmask[NI];    // A: bit t = filter tap t inside the image; B / plain GEMM: bit 0 = row exists
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int slot = wave * NI + j;
+    if (slot < NIA) {
+      const int64_t m = m0 + slot * 8 + (lane >> 3);
+      const bool ok = m < p.M;
+      const int64_t mm = ok ? m : 0;
+      if constexpr (LOAD == LOAD_CONV) {
+        const int wo = (int)(mm % p.Wo);
+        const int64_t t = mm / p.Wo;
+        const int ho = (int)(t % p.Ho);
+        const int64_t img = t / p.Ho;
+        const int hi0 = ho * p.sh - p.ph, wi0 = wo * p.sw - p.pw;
+        rowbase[j] = 2u * ((unsigned)(img * p.H * p.W * p.Ci) + (unsigned)((hi0 * p.W + wi0) * p.Ci));  // mod 2^32
+        unsigned mask = 0;
+        for (int r = 0; r < p.kh; ++r)
+          for (int q = 0; q < p.kw; ++q)
+            if ((unsigned)(hi0 + r * p.dh) < (unsigned)p.H && (unsigned)(wi0 + q * p.dw) < (unsigned)p.W)
+              mask |= 1u << (r * p.kw + q);
+        vmask[j] = ok ? mask : 0u;
+      } else {
+        rowbase[j] = (unsigned)(mm * p.K * 2);
+        vmask[j] = ok ? 1u : 0u;
+      }
+    } else {
+      const int n = n0 + (slot - NIA) * 16 + (lane >> 2);
+      const bool ok = n < p.N;
+      rowbase[j] = (unsigned)((int64_t)(ok ? n : 0) * p.K);
+      vmask[j] = ok ? 1u : 0u;
+    }
+  }
+  // this lane's position along K, in elements: as a loader of A (8-element chunks) and of B (16)
+  int ka_lin = ((lane & 7) ^ (lane >> 3)) * 8;
+  int kb_lin = ((lane & 3) ^ ((lane >> 4) & 3)) * 16;
+  int kr = 0, kq = 0, kci = ka_lin, tap = 0;
+  unsigned tapbase = 0;  // (kr*dh*W + kq*dw)*Ci elements
+  auto normalise_tap = [&]() {
+    while (kci >= p.Ci) {
+      kci -= p.Ci;
+      ++tap;
+      if (++kq == p.kw) { kq = 0; ++kr; }
+      tapbase = (unsigned)((kr * p.dh * p.W + kq * p.dw) * p.Ci);
+    }
+  };
+  if constexpr (LOAD == LOAD_CONV) normalise_tap();
+
+  auto issue_stage = [&](int stage_off) {
+    const bool ka_ok = ka_lin < p.K, kb_ok = kb_lin < p.K;
+    const unsigned a_koff = 2u * ((LOAD == LOAD_CONV) ? tapbase + (unsigned)kci : (unsigned)ka_lin);
+    const unsigned a_bit = (LOAD == LOAD_CONV) ? (1u << tap) : 1u;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int slot = wave * NI + j;
+      const bool is_a = slot < NIA;  // wave-uniform
+      lds_ptr_t dst = (lds_ptr_t)(lds_dyn + stage_off + slot * 1024);  // B slots follow the A slots
+      if (is_a) {
+        const unsigned voff = (ka_ok && (vmask[j] & a_bit)) ? rowbase[j] + a_koff : OOB;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, (int)voff, 0, 0, 0);
+      } else {
+        const unsigned voff = (kb_ok && vmask[j]) ? rowbase[j] + (unsigned)kb_lin : OOB;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, (int)voff, 0, 0, 0);
+      }
+    }
+    ka_lin += BK;
+    kb_lin += BK;
+    if constexpr (LOAD == LOAD_CONV) {
+      kci += BK;
+      normalise_tap();
+    }
+  };
+
+  v16i acc_hi[TM][TN], acc_lo[TM][TN];
+  int wsum[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) wsum[j] = 0;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { acc_hi[i][j][r] = 0; acc_lo[i][j][r] = 0; }
+
+  // ---- operand fetch addresses (LDS byte offsets) ------------------------------------------------
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)lds_dyn;
+  // A: elements [ks*32 + fhalf*16, +16) of the step = logical chunks ks*4 + fhalf*2 and the next one
+  const unsigned a_c0 = (unsigned)(((fhalf * 2) ^ (frow & 7)) * 16);
+  const unsigned a_row = lds_base + (unsigned)((wave_m * WM + frow) * (BK * 2));
+  // B: as in the int8 kernel
+  const int swb = (frow >> 2) & 3;
+  const unsigned b_k0 = (unsigned)((fhalf ^ swb) * 16), b_k1 = (unsigned)(((fhalf ^ swb) ^ 2) * 16);
+  const unsigned b_row = lds_base + (unsigned)(A_STAGE + (wave_n * WN + frow) * BK);
+
+  auto half_step = [&](unsigned a_base, unsigned a_chunk, unsigned b_addr) {
+    v4i fa[TM][2], fb[TN];
+    const unsigned a_first = a_base + a_chunk, a_second = a_base + (a_chunk ^ 16u);
+    // tile i of this wave sits 32 rows further: 4096 bytes for A, 2048 for B
+    fa[0][0] = ds_read_b128<0>(a_first);
+    fa[0][1] = ds_read_b128<0>(a_second);
+    if constexpr (TM > 1) {
+      fa[1][0] = ds_read_b128<4096>(a_first);
+      fa[1][1] = ds_read_b128<4096>(a_second);
+    }
+    fb[0] = ds_read_b128<0>(b_addr);
+    if constexpr (TN > 1) fb[1] = ds_read_b128<2048>(b_addr);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) { lgkm_wait<0>(fa[i][0]); lgkm_wait<0>(fa[i][1]); }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) lgkm_wait<0>(fb[j]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) wsum[j] = __builtin_amdgcn_sdot4(fb[j][d], 0x01010101, wsum[j], false);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      v4i hi, lo;
+      split_i16(fa[i][0], fa[i][1], hi, lo);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc_hi[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(hi, fb[j], acc_hi[i][j], 0, 0, 0);
+        acc_lo[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, fb[j], acc_lo[i][j], 0, 0, 0);
+      }
+    }
+  };
+  static_assert(TM <= 2 && TN <= 2, "wave tile larger than 64x64");
+
+  auto compute = [&](unsigned stage_off) {
+    half_step(a_row + stage_off, a_c0, b_row + stage_off + b_k0);
+    half_step(a_row + stage_off, a_c0 ^ 64u, b_row + stage_off + b_k1);
+  };
+
+  // ---- pipeline (same schedule as the int8 kernel) ---------------------------------------------------
+  const int nsteps = (p.K + BK - 1) / BK;
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue_stage(s * STAGE_BYTES);
+  int rd_off = 0, wr_off = (STAGES - 1) * STAGE_BYTES;
+  for (int step = 0; step < nsteps; ++step) {
+    CATCHQ_VMCNT(NI * (STAGES - 2));
+    __builtin_amdgcn_s_barrier();
+    issue_stage(wr_off);
+    compute((unsigned)rd_off);
+    rd_off = (rd_off + STAGE_BYTES == PIPE_BYTES) ? 0 : rd_off + STAGE_BYTES;
+    wr_off = (wr_off + STAGE_BYTES == PIPE_BYTES) ? 0 : wr_off + STAGE_BYTES;
+  }
+  CATCHQ_VMCNT(0);
+  __syncthreads();
+
+  // the two K halves of a column's weight sum sit in lanes l and l^32; the accumulator layout has
+  // column = lane & 31, the same as the weight fragment's row
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const unsigned ws = (unsigned)(wsum[j] + __shfl_xor(wsum[j], 32, 64)) << 7;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc_lo[i][j][r] = (int)(((unsigned)acc_hi[i][j][r] << 8) + (unsigned)acc_lo[i][j][r] + ws);
+  }
+  int *stage = reinterpret_cast<int *>(lds_dyn) + wave * 32 * EPI_STRIDE;
+  igemm_epilogue<TM, TN, EPI>(acc_lo, stage, m0 + wave_m * WM, n0 + wave_n * WN, lane, p, e);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int LOAD, int EPI>
+static int launch_a16_epi(const void *a, const void *b, const IgemmParams &p, const EpiDev &e, int64_t a_bytes,
+                          int64_t b_bytes, hipStream_t s) {
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int PIPE_BYTES = STAGES * (2 * BM + BN) * BK;
+  constexpr int EPI_BYTES = NW * 32 * (BN / WAVES_N + 8) * 4;
+  constexpr int LDS_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
+  static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
+  auto kern = igemm_a16_dma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI>;
+  if (LDS_BYTES > 64 * 1024) {
+    static bool raised[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CATCHQ_ERR_LAUNCH;
+    if (!raised[dev]) {
+      if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+        return CATCHQ_ERR_LAUNCH;
+      raised[dev] = true;
+    }
+  }
+  kern<<<p.nblocks, 64 * NW, LDS_BYTES, s>>>((const int16_t *)a, (const int8_t *)b, p, e, (unsigned)a_bytes,
+                                             (unsigned)b_bytes);
+  return launch_status();
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int LOAD>
+static int launch_a16(const void *a, const void *b, IgemmParams p, const EpiDev &e, int64_t a_bytes, int64_t b_bytes,
+                      hipStream_t s) {
+  const int64_t tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  const int64_t nb = tiles_m * p.tiles_n;
+  if (nb > 0x7fffffff) return CATCHQ_ERR_SHAPE;
+  p.nblocks = (int)nb;
+  if (pick_epilogue(p.N, e) == EPI_SCALAR)
+    return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_SCALAR>(a, b, p, e, a_bytes, b_bytes, s);
+  return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_VECTOR>(a, b, p, e, a_bytes, b_bytes, s);
+}
+
+template <int LOAD>
+static int pick_a16_tile(const void *a, const void *b, const IgemmParams &p, const EpiDev &e, int64_t a_bytes,
+                         int64_t b_bytes, hipStream_t s) {
+  auto blocks = [&](int bm, int bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+  constexpr int64_t kCUs = 256;
+  int tile = forced_tile();
+  if (!tile) {
+    if (p.N >= 256 && p.K >= 256 && blocks(128, 256) >= kCUs * 3 / 2) tile = 128256;
+    else if (p.N <= 64 || p.K < 256) tile = 64064;
+    else if (blocks(128, 128) >= kCUs * 3 / 2) tile = 128128;
+    else if (blocks(64, 128) >= kCUs * 3 / 2) tile = 64128;
+    else tile = 64064;
+  }
+  switch (tile) {
+    case 128256: return launch_a16<128, 256, 2, 4, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+    case 128128: return launch_a16<128, 128, 2, 2, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+    case 64128: return launch_a16<64, 128, 2, 2, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+    default: return launch_a16<64, 64, 2, 2, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+  }
+}
+
+// int16 x int8 contractions on the matrix cores; -1 when the shape is not eligible
+int igemm_a16_launch(int load, const void *a, const void *b, IgemmParams p, const EpiDev &e, int64_t a_bytes,
+                     int64_t b_bytes, hipStream_t s) {
+  if (a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || a_bytes <= 0 || b_bytes <= 0) return -1;
+  if (load == LOAD_GEMM) return pick_a16_tile<LOAD_GEMM>(a, b, p, e, a_bytes, b_bytes, s);
+  if (load == LOAD_CONV) return pick_a16_tile<LOAD_CONV>(a, b, p, e, a_bytes, b_bytes, s);
+  return -1;
+}
+
+int gemm_nt_mfma_a16(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s) {
+  IgemmParams p = {};
+  p.M = M;
+  p.N = (int)N;
+  p.K = (int)K;
+  return igemm_a16_launch(LOAD_GEMM, a, b, p, e, M * K * 2, N * K, s);
+}
+
+int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
+                    int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
+  IgemmParams p = {};
+  p.M = (int64_t)N * Ho * Wo;
+  p.N = Co;
+  p.H = H; p.W = W; p.Ci = Ci; p.Ho = Ho; p.Wo = Wo;
+  p.kh = kh; p.kw = kw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+  p.K = kh * kw * Ci;
+  return igemm_a16_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci * 2, (int64_t)Co * p.K, s);
+}
+
+}  // namespace catchq

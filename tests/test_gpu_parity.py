@@ -198,9 +198,10 @@ def test_division_by_reciprocal_is_exact():
 
 
 @pytest.mark.parametrize("bits", [(16, 8), (16, 16)])
-@pytest.mark.parametrize("m,n,k", [(20, 125, 100), (64, 64, 128), (3, 5, 600)])
+@pytest.mark.parametrize("m,n,k", [(20, 125, 100), (64, 64, 128), (3, 5, 600), (200, 96, 72), (130, 260, 520),
+                                   (1, 4, 8), (77, 64, 1024)])
 def test_gemm_wide(bits, m, n, k):
-    note("gemm_wide", bits, m, n, k)
+    note("gemm_wide", bits, m, n, k, cabi.lib().catchq_gemm_route(bits[0], bits[1], m, n, k))
     r = rng(k + bits[1])
     a, b = _ints(r, (m, k), bits[0]), _ints(r, (n, k), bits[1])
     bias = r.standard_normal(n).astype(np.float32)
@@ -210,6 +211,28 @@ def test_gemm_wide(bits, m, n, k):
         assert ovf == 0
         assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
     assert same_bits(orc.epilogue(acc, -20, None, bias), out["y"].cpu().numpy())
+
+
+@pytest.mark.parametrize("m,n,k", [(16384, 768, 256), (8192, 768, 320), (4096, 768, 256), (4096, 3072, 768)])
+def test_gemm_a16_tiles(m, n, k):
+    """int16 x int8 on the matrix cores, one shape per tile configuration, with the extreme digits
+    (-32768, 32767, -1, 0, 255, 256) planted; sampled rows against the oracle, all rows by linearity."""
+    note("gemm_a16", m, n, k, cabi.lib().catchq_gemm_route(16, 8, m, n, k))
+    r = rng(m + k)
+    a, b = (_ints(r, (m, k), 16) // 8).astype(np.int16), _ints(r, (n, k), 8)
+    a[5, :6] = (-32768, 32767, -1, 0, 255, 256)
+    a[m - 1, -6:] = (32767, -32768, 128, -128, 127, -129)
+    out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), y_dtype=None)
+    acc = out["acc"].cpu().numpy()
+    rows = np.concatenate([r.integers(0, m, 96), [0, 5, m - 1]])
+    want, ovf = orc.gemm_nt(a[rows], b)
+    assert ovf == 0 and np.array_equal(want.astype(np.int32), acc[rows])
+    # (a_hi*256 + a_lo) B^T = 256 * a_hi B^T + a_lo B^T, both halves through the int8 kernel
+    a_hi, a_lo = (a >> 8).astype(np.int8), ((a & 255) - 128).astype(np.int8)
+    hi = cabi.gemm_nt(cabi.dev(a_hi), cabi.dev(b), y_dtype=None)["acc"]
+    lo = cabi.gemm_nt(cabi.dev(a_lo), cabi.dev(b), y_dtype=None)["acc"]
+    bsum = torch.from_numpy(b.astype(np.int32).sum(1)).cuda()
+    assert torch.equal(hi * 256 + lo + 128 * bsum[None, :], out["acc"])
 
 
 def test_gemm_full_size_properties():
@@ -291,10 +314,14 @@ def test_conv_i8_acc_and_epilogue(case):
 
 
 @pytest.mark.parametrize("bits", [(16, 8), (16, 16)])
-@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[4], CONV_CASES[12]])
+@pytest.mark.parametrize("case", [CONV_CASES[i] for i in (0, 1, 4, 5, 6, 7, 8, 9, 10, 11, 12, 16, 17)] + [
+    (2, 8, 13, 13, 32, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # 8 channels: K = 72, ragged last K step
+    (1, 24, 9, 9, 255, 1, 1, (0, 0), (1, 1), (1, 1), 1),        # detection head: 255 outputs
+    (2, 256, 12, 12, 320, 3, 3, (1, 1), (1, 1), (1, 1), 1),     # wider tile
+])
 def test_conv_wide(bits, case):
     n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
-    note("conv_wide", bits, case)
+    note("conv_wide", bits, case, cabi.conv_route(bits[0], bits[1], (n, h, w, ci), (co, kh, kw, ci // g), pad, stride, dil, g))
     r = rng(sum(case[:7]) + bits[1])
     x, wt = _ints(r, (n, h, w, ci), bits[0]), _ints(r, (co, kh, kw, ci // g), bits[1])
     acc, ovf = orc.conv2d_nhwc(x, wt, pad, stride, dil, g)

@@ -107,9 +107,14 @@ def test_routes(lib):
     assert route(32, 32, 3, 32) == "depthwise"
     assert route(4, 16, 3, 2) == "direct"
     assert route(64, 64, 3, 1, (16, 16)) == "direct"
+    assert route(64, 64, 3, 1, (16, 8)) == "mfma_a16"
+    assert route(8, 32, 3, 1, (16, 8)) == "mfma_a16"
+    assert route(4, 32, 3, 1, (16, 8)) == "direct"
     assert route(64, 64, 30, 1) == "invalid"  # kernel larger than the image
     assert lib.catchq_gemm_route(8, 8, 4096, 3072, 768) == b"mfma"
     assert lib.catchq_gemm_route(8, 8, 10, 25, 10) == b"direct"
+    assert lib.catchq_gemm_route(16, 8, 4096, 3072, 768) == b"mfma_a16"
+    assert lib.catchq_gemm_route(16, 16, 4096, 3072, 768) == b"direct"
 
 
 # ------------------------------------------------------------------ the Python tool (A1/A2/A15)
