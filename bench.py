@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "resnet18", "mobilenet_v2"])
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "resnet18", "mobilenet_v2", "darknet53_yolov3"])
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--calib-images", type=int, default=8)
     ap.add_argument("--cpu-images", type=int, default=2)
@@ -78,14 +78,17 @@ def layer_profile(fused, x, iters=20):
         qx = trace[l.name]["qx"]
         qd = fused.q_demand[l.name][0] if fused.q_demand[l.name] else None
         want_y = fused.f_demand[l.name] or qd is None
+        y_half = fused.out_half and l.name in fused.outputs
         if l.kind == "conv":
             resid = torch.zeros_like(trace[l.name]["y"]) if l.add else None
 
             def run(l=l, lq=lq, qx=qx, qd=qd, want_y=want_y, resid=resid):
                 return ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
-                                   [l.stride, l.stride], [1, 1], lq.groups, {"none": 0, "relu": 1, "relu6": 2}[l.act],
-                                   want_y, False, False, qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
-            route = ops.conv2d_route(8, 8, list(qx.shape), list(lq.qw.shape[:3]) + [lq.qw.shape[3]],
+                                   [l.stride, l.stride], [1, 1], lq.groups,
+                                   {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}[l.act],
+                                   want_y, y_half, False, qd[0] if qd else 0, qd[1] if qd else 0, 1.0, 0.1,
+                                   bool(l.add_after))
+            route = ops.conv2d_route(lq.bw_x, lq.bw_w, list(qx.shape), list(lq.qw.shape[:3]) + [lq.qw.shape[3]],
                                      [l.pad, l.pad], [l.stride, l.stride], [1, 1], lq.groups)
         else:
             def run(lq=lq, qx=qx):
@@ -96,7 +99,7 @@ def layer_profile(fused, x, iters=20):
         n_out = y.numel()
         macs = n_out * (lq.qw.numel() // lq.qw.shape[0])
         bytes_alg = qx.numel() * qx.element_size() + lq.qw.numel() * lq.qw.element_size()
-        bytes_alg += (4 * n_out if want_y else 0) + (n_out * (qd[0] // 8) if qd else 0) + (4 * n_out if resid is not None else 0)
+        bytes_alg += ((2 if y_half else 4) * n_out if want_y else 0) + (n_out * (qd[0] // 8) if qd else 0) + (4 * n_out if resid is not None else 0)
         t = event_time(run, iters)
         rows.append(dict(name=l.name, route=route, t=t, ops=2 * macs, bytes=bytes_alg))
     return rows
@@ -119,14 +122,25 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    batch = args.batch or {"resnet50": 64, "resnet18": 64, "mobilenet_v2": 128}[args.workload]
+    batch = args.batch or {"resnet50": 64, "resnet18": 64, "mobilenet_v2": 128, "darknet53_yolov3": 16}[args.workload]
     layers = nets.NETS[args.workload]()
-    net = nets.FloatNet(layers, seed=0).eval()
-    x = torch.randn(batch, 3, 224, 224, generator=torch.Generator().manual_seed(1))
+    detector = args.workload == "darknet53_yolov3"
+    side = 416 if detector else 224
+    gen = torch.Generator().manual_seed(1)
     t0 = time.time()
-    sd = pipeline.calibrate(net, x[:args.calib_images], "int8", True)
+    if detector:
+        # int16 activations x int8 weights, q-params in the [bitwidths],[positions] encoding, fp16 outputs
+        net = nets.FloatNet(layers, seed=0, weight_std="he").eval()
+        x = torch.rand(batch, 3, side, side, generator=gen)
+        sd = pipeline.to_position_encoding(pipeline.calibrate(net, x[:min(args.calib_images, 2)], "int16", False), 16, 8)
+        what = "int16 activations x int8 weights (per-tensor positions), batch %d, 3x416x416 U(0,1), fp16 outputs" % batch
+    else:
+        net = nets.FloatNet(layers, seed=0).eval()
+        x = torch.randn(batch, 3, side, side, generator=gen)
+        sd = pipeline.calibrate(net, x[:args.calib_images], "int8", True)
+        what = "int8 (per-channel W, per-tensor act), batch %d, 3x224x224 N(0,1)" % batch
     t_cal = time.time() - t0
-    fused = pipeline.FusedNet(layers, sd)
+    fused = pipeline.FusedNet(layers, sd, out_half=detector)
     xg = x.cuda()
     static_in, replay = fused.capture(xg)
     static_in.copy_(xg)
@@ -141,12 +155,13 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = s.elapsed_time(e) / args.steps
     value = batch / (ms_per_step * 1e-3)
-    logits = out.float().cpu()
-    assert torch.isfinite(logits).all()
+    outs = out if isinstance(out, tuple) else (out,)
+    for o in outs:
+        assert torch.isfinite(o.float()).all()
 
     # ---- per-kernel roofline of the dominant family: the implicit-GEMM convolutions ------------
     rows = layer_profile(fused, xg)
-    conv_rows = [r for r in rows if r["route"] == "mfma"]
+    conv_rows = [r for r in rows if r["route"].startswith("mfma")]
     t_conv = sum(r["t"] for r in conv_rows)
     b_conv = sum(r["bytes"] for r in conv_rows)
     o_conv = sum(r["ops"] for r in conv_rows)
@@ -157,7 +172,8 @@ def main():
                                                                 r["bytes"] / r["t"] / 1e9, r["ops"] / r["t"] / 1e12),
                   file=sys.stderr)
         print("sum of conv/fc launches: %.1f us; graph step: %.1f us" % (t_all * 1e6, ms_per_step * 1e3), file=sys.stderr)
-    roofline = {"bound": "hbm", "kernel": "igemm_i8_kernel (all %d launches of one step)" % len(conv_rows),
+    roofline = {"bound": "hbm", "kernel": "%s (all %d launches of one step)" % (
+                    "igemm_a16_dma_kernel" if detector else "igemm_i8_dma_kernel", len(conv_rows)),
                 "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, batch)),
@@ -169,17 +185,17 @@ def main():
               else "int8 %s images/sec" % args.workload,
               "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-              "dtype": "int8", "data": "synthetic",
-              "config": {"workload": "%s int8 (per-channel W, per-tensor act), batch %d, 3x224x224 N(0,1), fused "
-                                     "requant pipeline replayed from a HIP graph" % (args.workload, batch),
+              "dtype": "int16xint8" if detector else "int8", "data": "synthetic",
+              "config": {"workload": "%s %s, fused requant pipeline replayed from a HIP graph" % (args.workload, what),
                          "global_batch": batch, "calibration_images": args.calib_images,
-                         "gop_per_step": round(2 * nets.conv_macs(layers, batch, 224, 224) / 1e9, 1)},
+                         "gop_per_step": round(2 * nets.conv_macs(layers, batch, side, side) / 1e9, 1)},
               "roofline": roofline}
 
     if not args.no_extras:
         result["extras"] = extras()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(layers, sd, x[:args.cpu_images], out[:args.cpu_images].float().cpu())
+        result["cpu_baseline"] = cpu_baseline(layers, sd, x[:args.cpu_images], outs[0][:args.cpu_images].float().cpu(),
+                                              fused.outputs[0])
     result["calibration_s"] = round(t_cal, 2)
     print(json.dumps(result))
 
@@ -207,7 +223,7 @@ def extras():
     return out
 
 
-def cpu_baseline(layers, sd, x_sample, gpu_logits):
+def cpu_baseline(layers, sd, x_sample, gpu_logits, out_name):
     """the oracle's unfused execution of the same network on a few images of the same batch"""
     import numpy as np
     import oracle as orc
@@ -216,7 +232,9 @@ def cpu_baseline(layers, sd, x_sample, gpu_logits):
     t0 = time.time()
     t, _ = netref.run(layers, sdn, x_sample.numpy())
     dt = time.time() - t0
-    want = t[layers[-1].name].reshape(gpu_logits.shape)
+    if gpu_logits.dim() == 4:  # logical NCHW -> the oracle's NHWC
+        gpu_logits = gpu_logits.permute(0, 2, 3, 1).contiguous()
+    want = t[out_name].reshape(gpu_logits.shape)
     span = float(want.max() - want.min())
     err = float(np.abs(want - gpu_logits.numpy()).max())
     return {"value": round(x_sample.shape[0] / dt, 3), "unit": "images/s", "cores": orc.num_threads(), "kind": "port",

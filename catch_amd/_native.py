@@ -20,7 +20,8 @@ class Epilogue(ctypes.Structure):
     _fields_ = [("exp2", ctypes.c_int), ("chan_div", ctypes.c_void_p), ("chan_rcp", ctypes.c_void_p), ("bias", ctypes.c_void_p),
                 ("resid", ctypes.c_void_p), ("act", ctypes.c_int), ("y", ctypes.c_void_p),
                 ("y_dtype", ctypes.c_int), ("acc_out", ctypes.c_void_p), ("q", ctypes.c_void_p),
-                ("q_bitwidth", ctypes.c_int), ("q_position", ctypes.c_int), ("q_scale", ctypes.c_float)]
+                ("q_bitwidth", ctypes.c_int), ("q_position", ctypes.c_int), ("q_scale", ctypes.c_float),
+                ("act_slope", ctypes.c_float), ("resid_after_act", ctypes.c_int)]
 
 
 class ConvDesc(ctypes.Structure):

@@ -91,6 +91,8 @@ struct EpiDev {
   int q_bw;
   int q_neg_pos;
   float q_scale;
+  float act_slope;
+  int resid_after;
 };
 
 inline EpiDev make_epi(const catchq_epilogue_t *e) {
@@ -108,6 +110,8 @@ inline EpiDev make_epi(const catchq_epilogue_t *e) {
   d.q_bw = e->q_bitwidth;
   d.q_neg_pos = -e->q_position;
   d.q_scale = e->q_scale;
+  d.act_slope = e->act_slope;
+  d.resid_after = (e->resid && e->resid_after_act) ? 1 : 0;
   return d;
 }
 
@@ -116,7 +120,7 @@ inline int check_epi(const catchq_epilogue_t *e) {
   if (!e->y && !e->acc_out && !e->q) return CATCHQ_ERR_ARG;
   if (e->y && e->y_dtype != CATCHQ_F32 && e->y_dtype != CATCHQ_F16) return CATCHQ_ERR_DTYPE;
   if (e->q && e->q_bitwidth != 8 && e->q_bitwidth != 16) return CATCHQ_ERR_BITWIDTH;
-  if (e->act < CATCHQ_ACT_NONE || e->act > CATCHQ_ACT_RELU6) return CATCHQ_ERR_ARG;
+  if (e->act < CATCHQ_ACT_NONE || e->act > CATCHQ_ACT_LEAKY) return CATCHQ_ERR_ARG;
   if (e->exp2 < -126 || e->exp2 > 126) return CATCHQ_ERR_ARG;
   if (e->q && (e->q_position < -126 || e->q_position > 126)) return CATCHQ_ERR_ARG;
   return CATCHQ_OK;
@@ -127,9 +131,11 @@ __device__ __forceinline__ float epi_value(float facc, int64_t idx, int c, const
   float v = __builtin_ldexpf(facc, e.exp2);
   if (e.chan_div) v = v / e.chan_div[c];
   if (e.bias) v = v + e.bias[c];
-  if (e.resid) v = v + e.resid[idx];
-  if (e.act >= CATCHQ_ACT_RELU) v = (v > 0.0f) ? v : 0.0f;
+  if (e.resid && !e.resid_after) v = v + e.resid[idx];
+  if (e.act == CATCHQ_ACT_LEAKY) v = (v > 0.0f) ? v : v * e.act_slope;
+  else if (e.act >= CATCHQ_ACT_RELU) v = (v > 0.0f) ? v : 0.0f;
   if (e.act == CATCHQ_ACT_RELU6) v = (v < 6.0f) ? v : 6.0f;
+  if (e.resid && e.resid_after) v = v + e.resid[idx];
   return v;
 }
 

@@ -39,7 +39,7 @@ inline bool vec_epilogue_ok(int N, const EpiDev &e) {
 // What an epilogue instance knows at compile time.  A field of -1 is decided at run time from the
 // EpiDev (the generic instance); fixed fields let the compiler drop every untaken branch, which
 // matters because the epilogue is VALU-bound (about a dozen fp32 operations per output element).
-//   DIV  0 none, 1 reciprocal form, 2 true division      BIAS, RESID  0/1
+//   DIV  0 none, 1 reciprocal form, 2 true division      BIAS 0/1     RESID 0 none, 1 before, 2 after the activation
 //   ACT  CATCHQ_ACT_*       YM  0 none, 1 fp32, 2 fp16     QM  0 none, 8, 16     ACC 0/1
 template <int DIV, int BIAS, int RESID, int ACT, int YM, int QM, int ACC>
 struct EpiSpec {
@@ -49,7 +49,8 @@ struct EpiSpec {
     return DIV < 0 ? (e.chan_div != nullptr && e.chan_rcp == nullptr) : DIV == 2;
   }
   static __device__ __forceinline__ bool bias(const EpiDev &e) { return BIAS < 0 ? e.bias != nullptr : BIAS == 1; }
-  static __device__ __forceinline__ bool resid(const EpiDev &e) { return RESID < 0 ? e.resid != nullptr : RESID == 1; }
+  static __device__ __forceinline__ bool resid(const EpiDev &e) { return RESID < 0 ? e.resid != nullptr : RESID >= 1; }
+  static __device__ __forceinline__ bool resid_after(const EpiDev &e) { return RESID < 0 ? e.resid_after != 0 : RESID == 2; }
   static __device__ __forceinline__ int act(const EpiDev &e) { return ACT < 0 ? e.act : ACT; }
   static __device__ __forceinline__ bool y32(const EpiDev &e) { return YM < 0 ? (e.y && !e.y_f16) : YM == 1; }
   static __device__ __forceinline__ bool y16(const EpiDev &e) { return YM < 0 ? (e.y && e.y_f16) : YM == 2; }
@@ -85,7 +86,8 @@ inline int pick_epilogue(int N, const EpiDev &e) {
   const bool rcp = e.chan_rcp != nullptr, bias = e.bias != nullptr, resid = e.resid != nullptr;
   const int ym = !e.y ? 0 : (e.y_f16 ? 2 : 1);
   const int qm = !e.q ? 0 : e.q_bw;
-  if (!rcp || !bias || e.acc_out || (qm && e.q_scale != 1.0f)) return EPI_VECTOR;
+  if (!rcp || !bias || e.acc_out || (qm && e.q_scale != 1.0f) || e.resid_after || e.act == CATCHQ_ACT_LEAKY)
+    return EPI_VECTOR;
   if (!resid && e.act == CATCHQ_ACT_RELU && ym == 0 && qm == 8) return EPI_Q8_RELU;
   if (resid && e.act == CATCHQ_ACT_RELU && ym == 1 && qm == 8) return EPI_RES_Y_Q8;
   if (!resid && e.act == CATCHQ_ACT_NONE && ym == 1 && qm == 0) return EPI_Y32;
@@ -98,7 +100,7 @@ inline int pick_epilogue(int N, const EpiDev &e) {
 // per-channel constants of one lane's four consecutive channels
 struct EpiLane {
   v4f div, rcp, bias;
-  bool use_rcp, use_div, use_bias, use_res, unit_q;
+  bool use_rcp, use_div, use_bias, use_res, res_after, unit_q;
   int act;
 };
 
@@ -106,6 +108,7 @@ template <class S>
 __device__ __forceinline__ EpiLane epi_lane_setup(int n, bool n_ok, const EpiDev &e) {
   EpiLane L;
   L.use_rcp = S::rcp(e); L.use_div = S::truediv(e); L.use_bias = S::bias(e); L.use_res = S::resid(e);
+  L.res_after = S::resid_after(e);
   L.act = S::act(e);
   L.unit_q = S::kGeneric ? (e.q_scale == 1.0f) : true;
   // Reciprocal form with the power of two folded in:
@@ -139,9 +142,11 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
       if (L.use_div) x = x / L.div[t];
     }
     if (L.use_bias) x = x + L.bias[t];
-    if (L.use_res) x = x + res[t];
-    if (L.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
+    if (L.use_res && !L.res_after) x = x + res[t];
+    if (L.act == CATCHQ_ACT_LEAKY) x = (x > 0.0f) ? x : x * e.act_slope;
+    else if (L.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
     if (L.act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
+    if (L.use_res && L.res_after) x = x + res[t];
     v[t] = x;
   }
   if (S::y16(e)) {

@@ -172,6 +172,8 @@ struct EpiArgs {
   bool want_y = true, y_half = false, want_acc = false;
   int64_t q_bitwidth = 0, q_position = 0;
   double q_scale = 1.0;
+  double act_slope = 0.0;
+  bool resid_after_act = false;
 };
 
 struct EpiOut {
@@ -252,6 +254,8 @@ EpiOut prepare_epilogue(const EpiArgs &a, at::IntArrayRef out_shape, int64_t co,
     e->resid = a.resid->data_ptr<float>();
   }
   e->act = (int)a.act;
+  e->act_slope = (float)a.act_slope;
+  e->resid_after_act = a.resid_after_act ? 1 : 0;
   if (a.want_y) {
     o.y = at::empty(out_shape, opts.dtype(a.y_half ? at::kHalf : at::kFloat));
     e->y = o.y.data_ptr();
@@ -314,8 +318,10 @@ EpiOut qlinear_impl(const Tensor &qx, const Tensor &qw, const EpiArgs &a) {
 
 EpiArgs make_args(int64_t exp2, const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias,
                   const c10::optional<Tensor> &resid, int64_t act, bool want_y, bool y_half, bool want_acc,
-                  int64_t q_bitwidth, int64_t q_position, double q_scale) {
+                  int64_t q_bitwidth, int64_t q_position, double q_scale, double act_slope = 0.0,
+                  bool resid_after_act = false) {
   EpiArgs a;
+  a.act_slope = act_slope; a.resid_after_act = resid_after_act;
   a.exp2 = exp2; a.chan_div = chan_div; a.bias = bias; a.resid = resid; a.act = act;
   a.want_y = want_y; a.y_half = y_half; a.want_acc = want_acc;
   a.q_bitwidth = q_bitwidth; a.q_position = q_position; a.q_scale = q_scale;
@@ -330,11 +336,12 @@ std::tuple<Tensor, Tensor, Tensor> qconv2d_op(const Tensor &qx, const Tensor &qw
                                               const c10::optional<Tensor> &resid, at::IntArrayRef padding,
                                               at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups,
                                               int64_t act, bool want_y, bool y_half, bool want_acc,
-                                              int64_t q_bitwidth, int64_t q_position, double q_scale) {
+                                              int64_t q_bitwidth, int64_t q_position, double q_scale,
+                                              double act_slope, bool resid_after_act) {
   c10::DeviceGuard guard(qx.device());
   return tup(qconv2d_impl(qx, qw, padding, stride, dilation, groups,
                           make_args(exp2, chan_div, bias, resid, act, want_y, y_half, want_acc, q_bitwidth,
-                                    q_position, q_scale)));
+                                    q_position, q_scale, act_slope, resid_after_act)));
 }
 
 std::tuple<Tensor, Tensor, Tensor> qlinear_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
@@ -607,8 +614,8 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("mm_q(Tensor a, int pos_a, Tensor b, int pos_b) -> Tensor");
   m.def("qconv2d(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, Tensor? resid, "
         "int[] padding, int[] stride, int[] dilation, int groups, int act=0, bool want_y=True, "
-        "bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0) "
-        "-> (Tensor, Tensor, Tensor)");
+        "bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
+        "float act_slope=0.0, bool resid_after_act=False) -> (Tensor, Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
         "bool want_y=True, bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, "
         "float q_scale=1.0) -> (Tensor, Tensor, Tensor)");

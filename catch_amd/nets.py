@@ -19,14 +19,19 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-Layer = namedtuple("Layer", "kind name src ci co k stride pad groups act add")
-Layer.__new__.__defaults__ = (None,) * 11
+Layer = namedtuple("Layer", "kind name src ci co k stride pad groups act add add_after")
+Layer.__new__.__defaults__ = (None,) * 12
+
+LEAKY_SLOPE = 0.1
 
 BN_EPS = 1e-5
 
 
-def conv(name, src, ci, co, k, stride=1, pad=None, groups=1, act="relu", add=None):
-    return Layer("conv", name, src, ci, co, k, stride, (k // 2) if pad is None else pad, groups, act, add)
+def conv(name, src, ci, co, k, stride=1, pad=None, groups=1, act="relu", add=None, add_after=False):
+    """add: tensor added to the convolution's output, before the activation (ResNet) or, with
+    add_after, after it (Darknet's shortcut layers)."""
+    return Layer("conv", name, src, ci, co, k, stride, (k // 2) if pad is None else pad, groups, act, add,
+                 bool(add_after))
 
 
 def maxpool(name, src, k, stride, pad):
@@ -107,7 +112,7 @@ def darknet53_yolov3(num_outputs=255):
     def cbl(src, ci, co, k, stride=1, act="leaky", add=None):
         cnt[0] += 1
         name = "c%d" % cnt[0]
-        L.append(conv(name, src, ci, co, k, stride, k // 2, act=act, add=add))
+        L.append(conv(name, src, ci, co, k, stride, k // 2, act=act, add=add, add_after=True))
         return name
 
     x = cbl("input", 3, 32, 3)
@@ -117,7 +122,7 @@ def darknet53_yolov3(num_outputs=255):
         x = cbl(x, cin, co, 3, 2)
         for _ in range(n):
             y = cbl(x, co, co // 2, 1)
-            x = cbl(y, co // 2, co, 3, add=x)  # residual add after the activation of the 3x3
+            x = cbl(y, co // 2, co, 3, add=x)  # shortcut: input + leaky(conv), linear afterwards
         cin = co
         routes[stage] = x
 
@@ -190,12 +195,14 @@ def conv_macs(layers, n, h, w):
 
 
 # ----------------------------------------------------------------------------------------------
-_ACT = {"none": lambda x: x, "relu": F.relu, "relu6": F.relu6, "leaky": lambda x: F.leaky_relu(x, 0.1)}
+_ACT = {"none": lambda x: x, "relu": F.relu, "relu6": F.relu6, "leaky": lambda x: F.leaky_relu(x, LEAKY_SLOPE)}
 
 
 class FloatNet(nn.Module):
     """The float model of a layer list: plain nn.Conv2d / nn.Linear children (so that
-    ``quantize_dynamic_mlu`` can swap them) wired according to the description."""
+    ``quantize_dynamic_mlu`` can swap them) wired according to the description.  weight_std: one
+    standard deviation for every layer, or "he" for sqrt(2 / fan_in) per layer, a quarter of that on
+    convolutions whose output is added to a shortcut (keeps activations of deep stacks at unit scale)."""
 
     def __init__(self, layers, seed=0, weight_std=0.05):
         super().__init__()
@@ -208,14 +215,18 @@ class FloatNet(nn.Module):
             if l.kind == "conv":
                 m = nn.Conv2d(l.ci, l.co, l.k, l.stride, l.pad, 1, l.groups, bias=True)
                 with torch.no_grad():
-                    m.weight.copy_(torch.randn(m.weight.shape, generator=g) * weight_std * fold)
+                    std = weight_std
+                    if weight_std == "he":  # the last convolution of a residual branch starts small
+                        std = math.sqrt(2.0 / (l.ci // l.groups * l.k * l.k)) * (0.25 if l.add else 1.0)
+                    m.weight.copy_(torch.randn(m.weight.shape, generator=g) * std * fold)
                     m.bias.zero_()
                 mods[l.name.replace(".", "_")] = m
             elif l.kind == "fc":
                 m = nn.Linear(l.ci, l.co, bias=True)
                 with torch.no_grad():
-                    m.weight.copy_(torch.randn(m.weight.shape, generator=g) * weight_std)
-                    m.bias.copy_(torch.randn(m.bias.shape, generator=g) * weight_std)
+                    std = math.sqrt(1.0 / l.ci) if weight_std == "he" else weight_std
+                    m.weight.copy_(torch.randn(m.weight.shape, generator=g) * std)
+                    m.bias.copy_(torch.randn(m.bias.shape, generator=g) * std)
                 mods[l.name.replace(".", "_")] = m
         self.mods = nn.ModuleDict(mods)
 
@@ -227,9 +238,11 @@ class FloatNet(nn.Module):
         for l in self.layers:
             if l.kind == "conv":
                 y = self.module_of(l.name)(t[l.src])
-                if l.add:
+                if l.add and not l.add_after:
                     y = y + t[l.add]
                 y = _ACT[l.act](y)
+                if l.add and l.add_after:
+                    y = y + t[l.add]
             elif l.kind == "maxpool":
                 y = F.max_pool2d(t[l.src], l.k, l.stride, l.pad)
             elif l.kind == "gap":

@@ -19,9 +19,9 @@ import numpy as np
 import torch
 
 from . import _native
-from .nets import outputs_of
+from .nets import LEAKY_SLOPE, outputs_of
 
-_ACT_CODE = {"none": 0, "relu": 1, "relu6": 2}
+_ACT_CODE = {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}
 _PASS = ("maxpool", "upsample", "concat")
 
 
@@ -40,12 +40,24 @@ class _LayerQ(object):
     __slots__ = ("bw_x", "bw_w", "pos_x", "pos_w", "qw", "chan_div", "bias", "exp2", "cpad", "groups")
 
 
-def _pad16(c):
-    """device-side channel count of a tensor with c channels: the matrix-core route wants multiples
-    of 16 (a 16-byte K chunk must not straddle filter taps); 1..3 channel inputs take 4"""
+def _pad16(c, bw=8):
+    """device-side channel count of a tensor with c channels: the matrix-core routes want a 16-byte
+    K chunk not to straddle filter taps, i.e. multiples of 16 channels for int8 activations (1..3
+    channel inputs take 4: one pixel per dword) and of 8 for int16 activations"""
+    if bw == 16:
+        return (c + 7) // 8 * 8
     if c <= 4:
         return 4 if c < 4 else c
     return (c + 15) // 16 * 16
+
+
+def _act_bits(layer, sd):
+    """bit width of the layer's quantized input, from the checkpoint's q-param encoding"""
+    k = _key(layer.name)
+    mode = sd[k + "quantized_mode"].detach().cpu().reshape(-1)
+    if mode.numel() == 1:
+        return 8 if int(mode[0]) in (1, 3) else 16
+    return int(sd[k + "scale"].detach().float().cpu()[0].item())
 
 
 def _decode(layer, sd, device, ci_dev, co_dev):
@@ -109,10 +121,11 @@ class FusedNet(object):
         self.outputs = outputs_of(self.layers)
         self.out_half = out_half
         # channel counts: real (chan) and as laid out on the device (cdev)
-        self.chan, self.cdev = {"input": self.layers[0].ci}, {"input": _pad16(self.layers[0].ci)}
+        bw = _act_bits(self.layers[0], state_dict)
+        self.chan, self.cdev = {"input": self.layers[0].ci}, {"input": _pad16(self.layers[0].ci, bw)}
         for l in self.layers:
             if l.kind == "conv":
-                self.chan[l.name], self.cdev[l.name] = l.co, _pad16(l.co)
+                self.chan[l.name], self.cdev[l.name] = l.co, _pad16(l.co, bw)
             elif l.kind == "fc":
                 self.chan[l.name] = self.cdev[l.name] = l.co
             elif l.kind == "concat":
@@ -177,7 +190,8 @@ class FusedNet(object):
                 y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
                                         [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
                                         self.out_half and name in self.outputs, tracing,
-                                        qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
+                                        qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
+                                        bool(l.add_after))
                 if want_y:
                     env[(name, "f")] = y
                 if qd:
@@ -271,4 +285,27 @@ def calibrate(float_net, x_cpu, dtype="int8", per_channel=True):
                 out[k] = torch.cat((sd[k], sd[p + "scale_weight_per_channel"])).float()
                 m = int(sd[p + "quantized_mode"].item())
                 out[p + "quantized_mode"] = torch.tensor([m + 2 if m in (1, 2) else m], dtype=torch.int32)
+    return out
+
+
+def to_position_encoding(sd, bw_x=16, bw_w=8):
+    """Rewrite a per-tensor checkpoint into the reference's second q-param encoding:
+    ``scale = [bitwidth_input, bitwidth_weight]``, ``quantized_mode = [position_input,
+    position_weight]`` (quantify_conv_forward.cpp:79-88), pure power-of-two quantization.  The
+    activation range is recovered from the calibrated scale (scale = qmax / absmax), the weight
+    range is the tensor's own max-abs."""
+    out = dict(sd)
+    for k in list(sd.keys()):
+        if not k.endswith(".quantized_mode"):
+            continue
+        p = k[:-len("quantized_mode")]
+        m = int(sd[k].reshape(-1)[0].item())
+        qmax_cal = 127.0 if m in (1, 3) else 32767.0
+        absmax_x = qmax_cal / float(sd[p + "scale"].reshape(-1)[0].item())
+        absmax_w = float(sd[p + "weight"].abs().max().item())
+        qx, qw = float(2 ** (bw_x - 1) - 1), float(2 ** (bw_w - 1) - 1)
+        pos_x = pos_from_scale(bw_x, qx / absmax_x)
+        pos_w = pos_from_scale(bw_w, qw / absmax_w if absmax_w > 0 else 1.0)
+        out[p + "scale"] = torch.tensor([float(bw_x), float(bw_w)])
+        out[k] = torch.tensor([pos_x, pos_w], dtype=torch.int32)
     return out

@@ -40,7 +40,7 @@ enum {
 };
 
 enum { CATCHQ_F32 = 0, CATCHQ_F16 = 1 };
-enum { CATCHQ_ACT_NONE = 0, CATCHQ_ACT_RELU = 1, CATCHQ_ACT_RELU6 = 2 };
+enum { CATCHQ_ACT_NONE = 0, CATCHQ_ACT_RELU = 1, CATCHQ_ACT_RELU6 = 2, CATCHQ_ACT_LEAKY = 3 };
 /* cnnlQuantizeMode_t values used by the reference (operators/cnnl/internal/quantize_param.cpp:70-78) */
 enum { CATCHQ_QUANTIZE_POSITION = 0, CATCHQ_QUANTIZE_POSITION_SCALE = 1, CATCHQ_QUANTIZE_POSITION_SCALE_OFFSET = 2 };
 
@@ -111,7 +111,8 @@ int catchq_dequantize(const void *q, int bits, void *y, int y_dtype, int64_t n, 
  *   v = v / chan_div[c]   if chan_div       "output / new_scale" (quantify_conv_forward.cpp:127; linear.cpp:56)
  *   v = v + bias[c]       if bias           (quantify_conv_forward.cpp:129; linear.cpp:57-59)
  *   v = v + resid[r][c]   if resid          residual branch of the caller's graph (fp32)
- *   v = act(v)
+ *   v = act(v)                              ReLU, ReLU6, or leaky ReLU: v > 0 ? v : v * act_slope
+ *   (with resid_after_act != 0 the residual is added after the activation instead of before it)
  * then any of: y[r][c] = v (fp32, or fp16 by one RNE conversion); acc_out[r][c] = acc;
  * q[r][c] = sat(rne(v * q_scale * 2^-q_position)) for the next layer (q_bitwidth 8/16).
  * All fp32, no fused multiply-add between the steps, true division.
@@ -135,6 +136,8 @@ typedef struct catchq_epilogue {
   int q_bitwidth;
   int q_position;
   float q_scale;
+  float act_slope;       /* CATCHQ_ACT_LEAKY: factor for v <= 0 */
+  int resid_after_act;   /* 0: act(v + resid), otherwise act(v) + resid */
 } catchq_epilogue_t;
 
 /* cnnl_mm(self, self_position, other, other_position, false, true) -> cnnlMatMul

@@ -199,8 +199,29 @@ def conv2d_nhwc(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1):
     return acc, ovf
 
 
-def epilogue(acc, exp2, chan_div=None, bias=None, resid=None, act=0, out_dtype=np.float32):
-    """acc [..., Co] integer sums -> fp32/fp16 [..., Co]"""
+def leaky_relu(y, slope):
+    """x > 0 ? x : x * slope in fp32 (one rounding), the elementwise op of torch.nn.LeakyReLU"""
+    y = np.asarray(y, np.float32)
+    return np.where(y > 0, y, y * np.float32(slope)).astype(np.float32)
+
+
+def epilogue(acc, exp2, chan_div=None, bias=None, resid=None, act=0, out_dtype=np.float32, act_slope=0.0,
+             resid_after_act=False):
+    """acc [..., Co] integer sums -> fp32/fp16 [..., Co].  act 3 = leaky ReLU with act_slope;
+    resid_after_act: act(v) + resid instead of act(v + resid).  Those two variants are composed
+    here from the plain dequant+bias step and separate fp32 elementwise steps, the way a model
+    built from the reference's ops runs them (activation and add are ops of their own there)."""
+    if act == 3 or (resid_after_act and resid is not None):
+        y = epilogue(acc, exp2, chan_div, bias, None if resid_after_act else resid, 0)
+        if act == 3:
+            y = leaky_relu(y, act_slope)
+        elif act >= 1:
+            y = np.where(y > 0, y, np.float32(0)).astype(np.float32)
+            if act == 2:
+                y = np.where(y < 6, y, np.float32(6)).astype(np.float32)
+        if resid_after_act and resid is not None:
+            y = (y + np.asarray(resid, np.float32).reshape(y.shape)).astype(np.float32)
+        return y.astype(np.float16) if out_dtype == np.float16 else y
     acc = _c(acc, np.int64)
     co = acc.shape[-1]
     rows = acc.size // max(co, 1)

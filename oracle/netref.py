@@ -13,7 +13,8 @@ from . import (conv2d_nhwc, epilogue, gemm_nt, global_avgpool_nhwc, maxpool_nhwc
                quantize_per_channel)
 from .ops import decode_qparams
 
-_ACT = {"none": 0, "relu": 1, "relu6": 2}
+_ACT = {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}
+LEAKY_SLOPE = 0.1
 
 
 def _key(name):
@@ -44,7 +45,8 @@ def run(layers, sd, x_nchw):
             else:
                 acc, ovf = gemm_nt(qx, qw)
                 resid = None
-            y = epilogue(acc, d["pos_x"] + d["pos_w"], d["new_scale"], b, resid, _ACT[l.act])
+            y = epilogue(acc, d["pos_x"] + d["pos_w"], d["new_scale"], b, resid, _ACT[l.act], act_slope=LEAKY_SLOPE,
+                         resid_after_act=bool(l.add_after))
             rec[l.name] = dict(qx=qx, acc=acc, y=y, overflow=ovf, pos_x=d["pos_x"], pos_w=d["pos_w"])
             t[l.name] = y
         elif l.kind == "maxpool":

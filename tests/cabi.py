@@ -82,8 +82,9 @@ def dequantize(q, pos, scale=1.0, half=False):
 
 
 def _epilogue(shape, device, exp2, chan_div, bias, resid, act, y_dtype, want_acc, q_bw, q_pos, q_scale,
-              chan_rcp=None):
+              chan_rcp=None, act_slope=0.0, resid_after_act=False):
     e = Epilogue()
+    e.act_slope, e.resid_after_act = act_slope, int(resid_after_act)
     out = {}
     e.exp2 = exp2
     e.chan_div, e.chan_rcp, e.bias, e.resid = ptr(chan_div), ptr(chan_rcp), ptr(bias), ptr(resid)
@@ -120,12 +121,12 @@ def conv_desc(x_shape, w_shape, padding, stride, dilation, groups):
 
 def conv2d_nhwc(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1, exp2=0, chan_div=None, bias=None,
                 resid=None, act=0, y_dtype=torch.float32, want_acc=True, q_bw=0, q_pos=0, q_scale=1.0,
-                chan_rcp=None):
+                chan_rcp=None, act_slope=0.0, resid_after_act=False):
     d = conv_desc(x.shape, w.shape, padding, stride, dilation, groups)
     ho = lib().catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h)
     wo = lib().catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w)
     e, out = _epilogue((d.n, ho, wo, d.co), x.device, exp2, chan_div, bias, resid, act, y_dtype, want_acc, q_bw,
-                       q_pos, q_scale, chan_rcp)
+                       q_pos, q_scale, chan_rcp, act_slope, resid_after_act)
     check(lib().catchq_conv2d_nhwc(ptr(x), x.element_size() * 8, ptr(w), w.element_size() * 8, ctypes.byref(d),
                                    ctypes.byref(e), stream()))
     return out

@@ -313,6 +313,27 @@ def test_conv_i8_acc_and_epilogue(case):
     assert same_bits(orc.epilogue(acc, -10, None, None, None, 2, np.float16), out["y"].cpu().numpy())
 
 
+@pytest.mark.parametrize("case", [CONV_CASES[4], CONV_CASES[17], CONV_CASES[18], CONV_CASES[3]])
+@pytest.mark.parametrize("after", [False, True])
+def test_conv_leaky_relu_and_residual_order(case, after):
+    """leaky ReLU (v > 0 ? v : v*slope) and the residual added before / after the activation, on the
+    vector epilogue (matrix cores, depthwise) and the scalar one (direct kernel, Co % 4 != 0)."""
+    n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
+    note("conv_leaky", case, after)
+    r = rng(sum(case[:7]) + 99)
+    x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, kh, kw, ci // g), 8)
+    acc, _ = orc.conv2d_nhwc(x, wt, pad, stride, dil, g)
+    bias = r.standard_normal(co).astype(np.float32)
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    for act in (3, 1):
+        out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), pad, stride, dil, g, exp2=-11, bias=cabi.dev(bias),
+                               resid=cabi.dev(resid), act=act, q_bw=16, q_pos=-9, want_acc=False, act_slope=0.1,
+                               resid_after_act=after)
+        y = orc.epilogue(acc, -11, None, bias, resid, act, act_slope=0.1, resid_after_act=after)
+        assert same_bits(y, out["y"].cpu().numpy())
+        assert same_bits(orc.quantize(y, 16, -9), out["q"].cpu().numpy())
+
+
 @pytest.mark.parametrize("bits", [(16, 8), (16, 16)])
 @pytest.mark.parametrize("case", [CONV_CASES[i] for i in (0, 1, 4, 5, 6, 7, 8, 9, 10, 11, 12, 16, 17)] + [
     (2, 8, 13, 13, 32, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # 8 channels: K = 72, ragged last K step

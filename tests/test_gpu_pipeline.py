@@ -107,6 +107,22 @@ def test_mobilenet_v2_small():
     check_against_oracle(layers, sd, x, fused)
 
 
+def test_darknet53_yolov3_int16_activations():
+    """Darknet-53 + three YOLOv3 heads with int16 activations x int8 weights in the reference's
+    [bitwidths],[positions] q-param encoding: leaky ReLU, shortcut adds after the activation,
+    upsample + concat on the integers, 255-channel heads (padded to 256 on the device)."""
+    note("darknet53_yolov3 bs1 64x64 int16 x int8")
+    layers = nets.darknet53_yolov3()
+    net = nets.FloatNet(layers, seed=7, weight_std="he").eval()
+    x = torch.rand(1, 3, 64, 64, generator=torch.Generator().manual_seed(8))
+    sd = pipeline.to_position_encoding(pipeline.calibrate(net, x, "int16", False), 16, 8)
+    fused = pipeline.FusedNet(layers, sd, out_half=False)
+    assert fused.cdev["input"] == 8 and fused.cdev["yolo13"] == 256
+    assert fused.q["c2"].bw_x == 16 and fused.q["c2"].bw_w == 8
+    outs = check_against_oracle(layers, sd, x, fused)
+    assert [tuple(o.shape) for o in outs] == [(1, 255, 2, 2), (1, 255, 4, 4), (1, 255, 8, 8)]
+
+
 def test_dropin_modules_match_fused_pipeline():
     """quantize_dynamic_mlu flow (torch_mlu::conv2d/linear + ATen relu/add/pool in float) gives
     the same logits as the fused plan, up to the global-average-pool summation order."""
