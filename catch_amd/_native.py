@@ -21,7 +21,8 @@ class Epilogue(ctypes.Structure):
                 ("resid", ctypes.c_void_p), ("act", ctypes.c_int), ("y", ctypes.c_void_p),
                 ("y_dtype", ctypes.c_int), ("acc_out", ctypes.c_void_p), ("q", ctypes.c_void_p),
                 ("q_bitwidth", ctypes.c_int), ("q_position", ctypes.c_int), ("q_scale", ctypes.c_float),
-                ("act_slope", ctypes.c_float), ("resid_after_act", ctypes.c_int)]
+                ("act_slope", ctypes.c_float), ("resid_after_act", ctypes.c_int),
+                ("exp2_dev", ctypes.c_void_p * 2)]
 
 
 class ConvDesc(ctypes.Structure):
@@ -50,6 +51,8 @@ SIGNATURES = {
     "catchq_conv2d_nhwc": (_I, [_P, _I, _P, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Epilogue), _P]),
     "catchq_maxpool_nhwc": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "catchq_global_avgpool_nhwc": (_I, [_P, _P, _I, _I, _I, _P]),
+    "catchq_quantize_conv2d_workspace_size": (_I, [ctypes.POINTER(ConvDesc), _I, _I, ctypes.POINTER(_SZ)]),
+    "catchq_quantize_conv2d_nhwc": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, ctypes.POINTER(ConvDesc), _P, _P, _I, _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
 }

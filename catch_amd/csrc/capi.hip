@@ -139,3 +139,46 @@ CATCHQ_API int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int 
     }
   }
 }
+
+static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+CATCHQ_API int catchq_quantize_conv2d_workspace_size(const catchq_conv_desc_t *desc, int x_bits, int w_bits,
+                                                     size_t *bytes) {
+  int ho, wo;
+  int st = check_conv(desc, &ho, &wo);
+  if (st != CATCHQ_OK) return st;
+  if (!bytes) return CATCHQ_ERR_ARG;
+  if ((x_bits != 8 && x_bits != 16) || (w_bits != 8 && w_bits != 16)) return CATCHQ_ERR_BITWIDTH;
+  const size_t xe = (size_t)desc->n * desc->h * desc->w * desc->ci;
+  const size_t we = (size_t)desc->co * desc->kh * desc->kw * (desc->ci / desc->groups);
+  *bytes = round256(xe * (x_bits / 8)) + round256(we * (w_bits / 8));
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_quantize_conv2d_nhwc(const void *x, int x_dtype, const int32_t *x_position_dev, int x_bits,
+                                           const void *w, int w_dtype, const int32_t *w_position_dev, int w_bits,
+                                           const catchq_conv_desc_t *desc, const float *bias, void *y, int y_dtype,
+                                           void *workspace, size_t workspace_bytes, catchq_stream_t stream) {
+  size_t need = 0;
+  int st = catchq_quantize_conv2d_workspace_size(desc, x_bits, w_bits, &need);
+  if (st != CATCHQ_OK) return st;
+  if (desc->n == 0) return CATCHQ_OK;
+  if (!x || !w || !y || !x_position_dev || !w_position_dev || !workspace) return CATCHQ_ERR_ARG;
+  if (workspace_bytes < need || !aligned16(workspace)) return CATCHQ_ERR_ARG;
+  const int64_t xe = (int64_t)desc->n * desc->h * desc->w * desc->ci;
+  const int64_t we = (int64_t)desc->co * desc->kh * desc->kw * (desc->ci / desc->groups);
+  void *qx = workspace;
+  void *qw = (char *)workspace + round256((size_t)xe * (x_bits / 8));
+  st = catchq_quantize_devpos(x, x_dtype, qx, x_bits, xe, x_position_dev, nullptr, stream);
+  if (st != CATCHQ_OK) return st;
+  st = catchq_quantize_devpos(w, w_dtype, qw, w_bits, we, w_position_dev, nullptr, stream);
+  if (st != CATCHQ_OK) return st;
+  catchq_epilogue_t e;
+  memset(&e, 0, sizeof(e));
+  e.exp2_dev[0] = x_position_dev;
+  e.exp2_dev[1] = w_position_dev;
+  e.bias = bias;
+  e.y = y;
+  e.y_dtype = y_dtype;
+  return catchq_conv2d_nhwc(qx, x_bits, qw, w_bits, desc, &e, stream);
+}

@@ -93,13 +93,15 @@ struct EpiDev {
   float q_scale;
   float act_slope;
   int resid_after;
+  const int *exp2_a, *exp2_b;  // device-resident positions added to exp2 (resolve_exp2)
 };
 
 inline EpiDev make_epi(const catchq_epilogue_t *e) {
   EpiDev d;
   d.exp2 = e->exp2;
   d.chan_div = e->chan_div;
-  d.chan_rcp = (e->chan_div && e->chan_rcp && e->exp2 >= -64 && e->exp2 <= 64) ? e->chan_rcp : nullptr;
+  const bool dev_exp = e->exp2_dev[0] || e->exp2_dev[1];
+  d.chan_rcp = (e->chan_div && e->chan_rcp && !dev_exp && e->exp2 >= -64 && e->exp2 <= 64) ? e->chan_rcp : nullptr;
   d.bias = e->bias;
   d.resid = e->resid;
   d.act = e->act;
@@ -112,6 +114,8 @@ inline EpiDev make_epi(const catchq_epilogue_t *e) {
   d.q_scale = e->q_scale;
   d.act_slope = e->act_slope;
   d.resid_after = (e->resid && e->resid_after_act) ? 1 : 0;
+  d.exp2_a = e->exp2_dev[0];
+  d.exp2_b = e->exp2_dev[1];
   return d;
 }
 
@@ -124,6 +128,17 @@ inline int check_epi(const catchq_epilogue_t *e) {
   if (e->exp2 < -126 || e->exp2 > 126) return CATCHQ_ERR_ARG;
   if (e->q && (e->q_position < -126 || e->q_position > 126)) return CATCHQ_ERR_ARG;
   return CATCHQ_OK;
+}
+
+// first statement of every kernel that takes an EpiDev: fold the device-resident positions into exp2
+// (uniform scalar loads; the sum is clamped to what ldexpf handles without surprises)
+__device__ __forceinline__ void resolve_exp2(EpiDev &e) {
+  if (e.exp2_a || e.exp2_b) {
+    int v = e.exp2;
+    if (e.exp2_a) v += *e.exp2_a;
+    if (e.exp2_b) v += *e.exp2_b;
+    e.exp2 = v < -252 ? -252 : (v > 252 ? 252 : v);
+  }
 }
 
 // value after dequant / bias / residual / activation; facc = float(acc) (one RNE conversion)

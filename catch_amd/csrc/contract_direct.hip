@@ -30,6 +30,7 @@ template <int AB, int BB>
 __global__ __launch_bounds__(256) void gemm_nt_direct_kernel(const typename IntOf<AB>::type *__restrict__ a,
                                                             const typename IntOf<BB>::type *__restrict__ b,
                                                             int64_t M, int64_t N, int64_t K, EpiDev e) {
+  resolve_exp2(e);
   typedef typename AccOf<AB, BB>::type TAcc;
   const int64_t total = M * N;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -50,6 +51,7 @@ template <int AB, int BB>
 __global__ __launch_bounds__(256) void conv2d_direct_kernel(const typename IntOf<AB>::type *__restrict__ x,
                                                            const typename IntOf<BB>::type *__restrict__ w,
                                                            ConvDev d, EpiDev e) {
+  resolve_exp2(e);
   typedef typename AccOf<AB, BB>::type TAcc;
   const int cig = d.Ci / d.groups, cog = d.Co / d.groups;
   const int64_t total = (int64_t)d.N * d.Ho * d.Wo * d.Co;

@@ -26,6 +26,7 @@ constexpr int DW_LDS_BYTES = 32 * 1024;
 // threads: 256 = 16 channel-quads (x4 channels) x 16 pixels
 __global__ __launch_bounds__(256) void dwconv_i8_kernel(const int8_t *__restrict__ x,
                                                        const int8_t *__restrict__ w, DwParams p, EpiDev e) {
+  resolve_exp2(e);
   __shared__ __attribute__((aligned(16))) int8_t tile[DW_LDS_BYTES];
   __shared__ __attribute__((aligned(16))) int8_t wt[DW_MAXTAPS * DW_CS];
 
@@ -105,6 +106,7 @@ constexpr int DW3_PW = 4, DW3_PH = 2;
 template <int S, int EPI>
 __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x, const int8_t *__restrict__ w,
                                                    Dw3Params p, EpiDev e) {
+  resolve_exp2(e);
   typedef typename EpiOf<EPI>::type Sp;
   constexpr int PW = DW3_PW, PH = DW3_PH;
   constexpr int NC = (PW - 1) * S + 3;  // input columns of the window

@@ -35,6 +35,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
                                                                             const int8_t *__restrict__ B,
                                                                             IgemmParams p, EpiDev e,
                                                                             unsigned a_bytes, unsigned b_bytes) {
+  resolve_exp2(e);
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;

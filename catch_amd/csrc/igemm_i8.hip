@@ -33,6 +33,7 @@ template <int BM, int BN, int LOAD, int EPI>
 __global__ __launch_bounds__(256) void igemm_i8_kernel(const int8_t *__restrict__ A,
                                                       const int8_t *__restrict__ B, IgemmParams p,
                                                       EpiDev e) {
+  resolve_exp2(e);
   constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int LA = BM / 64, LB = BN / 64;  // 16-byte chunks each thread loads per K step

@@ -538,6 +538,48 @@ Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   return o.y.permute({0, 3, 1, 2});  // logical NCHW over channels-last memory, like the reference
 }
 
+// cnnl_quantize_convolution_internal(input, input_position, weight, weight_position, bias, padding, stride,
+// dilation, groups, bitwidth)      operators/cnnl/internal/quantize_convolution.cpp:57-235
+// float tensors in, positions as int32 device tensors, nothing copied to the host
+Tensor quantize_conv2d_op(const Tensor &input, const Tensor &input_position, const Tensor &weight,
+                          const Tensor &weight_position, const Tensor &bias, at::IntArrayRef padding,
+                          at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups, int64_t input_bitwidth,
+                          int64_t weight_bitwidth) {
+  TORCH_CHECK(input.dim() == 4 && weight.dim() == 4, "conv2d only support 4 dims.");
+  TORCH_CHECK(padding.size() == 2 && stride.size() == 2 && dilation.size() == 2, "padding/stride/dilation: two values each");
+  const int x_dt = fp_dtype(input, "quantify only support input float/half");
+  const int w_dt = fp_dtype(weight, "quantify only support input float/half");
+  TORCH_CHECK((input_bitwidth == 8 || input_bitwidth == 16) && (weight_bitwidth == 8 || weight_bitwidth == 16),
+              "bitwidth not support");
+  TORCH_CHECK(input_position.scalar_type() == at::kInt && weight_position.scalar_type() == at::kInt &&
+                  input_position.numel() == 1 && weight_position.numel() == 1 &&
+                  input_position.device() == input.device() && weight_position.device() == input.device(),
+              "positions must be int32 tensors of one element on the input's device");
+  if (has_bias(bias)) TORCH_CHECK(bias.dim() == 1 && bias.size(0) == weight.size(0), "currently only support 1-dim bias");
+  c10::DeviceGuard guard(input.device());
+  Tensor x = input.contiguous(at::MemoryFormat::ChannelsLast);   // memory [N][H][W][C]
+  Tensor w = weight.contiguous(at::MemoryFormat::ChannelsLast);  // memory [Co][kh][kw][Ci/g]
+  catchq_conv_desc_t d = {(int)x.size(0), (int)x.size(2), (int)x.size(3), (int)x.size(1), (int)w.size(0),
+                          (int)w.size(2), (int)w.size(3), (int)padding[0], (int)padding[1], (int)stride[0],
+                          (int)stride[1], (int)dilation[0], (int)dilation[1], (int)groups};
+  TORCH_CHECK(groups > 0 && x.size(1) == w.size(1) * groups, "channel mismatch: input ", input.sizes(), ", weight ",
+              weight.sizes(), ", groups ", groups);
+  size_t ws_bytes = 0;
+  check_status(catchq_quantize_conv2d_workspace_size(&d, (int)input_bitwidth, (int)weight_bitwidth, &ws_bytes),
+               "torch_mlu::quantize_conv2d");
+  const int ho = catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h);
+  const int wo = catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w);
+  Tensor workspace = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kChar));
+  Tensor y = at::empty({d.n, ho, wo, d.co}, x.options());
+  Tensor bs = has_bias(bias) ? bias.to(at::kFloat).contiguous() : Tensor();
+  check_status(catchq_quantize_conv2d_nhwc(x.data_ptr(), x_dt, input_position.data_ptr<int32_t>(), (int)input_bitwidth,
+                                           w.data_ptr(), w_dt, weight_position.data_ptr<int32_t>(),
+                                           (int)weight_bitwidth, &d, bs.defined() ? bs.data_ptr<float>() : nullptr,
+                                           y.data_ptr(), x_dt, workspace.data_ptr(), ws_bytes, current_stream()),
+               "torch_mlu::quantize_conv2d");
+  return y.permute({0, 3, 1, 2});
+}
+
 Tensor linear_op(const Tensor &input, const Tensor &weight, const Tensor &bias, const Tensor &q_scale,
                  const Tensor &q_mode) {
   TORCH_CHECK(weight.dim() == 2, "we only support the  dim of weight is 2");
@@ -619,6 +661,8 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
         "bool want_y=True, bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, "
         "float q_scale=1.0) -> (Tensor, Tensor, Tensor)");
+  m.def("quantize_conv2d(Tensor input, Tensor input_position, Tensor weight, Tensor weight_position, Tensor bias, "
+        "int[] padding, int[] stride, int[] dilation, int groups, int input_bitwidth=8, int weight_bitwidth=8) -> Tensor");
   m.def("maxpool_nhwc(Tensor x, int k, int stride, int pad) -> Tensor");
   m.def("global_avgpool_nhwc(Tensor x) -> Tensor");
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
@@ -636,6 +680,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("quantize_per_channel", &quantize_per_channel_op);
   m.impl("dequantize", &dequantize_op);
   m.impl("mm_q", &mm_q_op);
+  m.impl("quantize_conv2d", &quantize_conv2d_op);
   m.impl("qconv2d", &qconv2d_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);

@@ -138,6 +138,8 @@ typedef struct catchq_epilogue {
   float q_scale;
   float act_slope;       /* CATCHQ_ACT_LEAKY: factor for v <= 0 */
   int resid_after_act;   /* 0: act(v + resid), otherwise act(v) + resid */
+  const int32_t *exp2_dev[2]; /* device-resident positions added to exp2 when non-NULL (no host sync);
+                                 the reciprocal form of the division is not used with them */
 } catchq_epilogue_t;
 
 /* cnnl_mm(self, self_position, other, other_position, false, true) -> cnnlMatMul
@@ -166,6 +168,19 @@ int catchq_conv_out_size(int in, int k, int pad, int stride, int dil);
  * direct kernel; the arithmetic is the same in all of them. */
 int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int w_bits, const catchq_conv_desc_t *desc,
                        const catchq_epilogue_t *epilogue, catchq_stream_t stream);
+
+/* cnnl_quantize_convolution_internal -> cnnlQuantizeConvolutionForward
+ *                                                          operators/cnnl/internal/quantize_convolution.cpp:57-235
+ * Convolution of floating tensors quantized on the fly with positions that live in device memory (int32[1]
+ * each; scale 1, no offset, as the reference passes them): x [n,h,w,ci] and w [co,kh,kw,ci/groups] fp32/fp16,
+ * q = sat(rne(v * 2^-position)) at x_bits / w_bits, integer convolution, y = acc * 2^(pos_x + pos_w) + bias
+ * as fp32/fp16 NHWC.  No host synchronisation.  The caller supplies the workspace (the quantized copies of
+ * both operands), as with the reference's cnnlGetConvolutionForwardWorkspaceSize (:160-169). */
+int catchq_quantize_conv2d_workspace_size(const catchq_conv_desc_t *desc, int x_bits, int w_bits, size_t *bytes);
+int catchq_quantize_conv2d_nhwc(const void *x, int x_dtype, const int32_t *x_position_dev, int x_bits,
+                                const void *w, int w_dtype, const int32_t *w_position_dev, int w_bits,
+                                const catchq_conv_desc_t *desc, const float *bias, void *y, int y_dtype,
+                                void *workspace, size_t workspace_bytes, catchq_stream_t stream);
 
 /* ------------------------------------------------------------------ neighbours of the convolutions */
 

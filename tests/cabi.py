@@ -132,6 +132,22 @@ def conv2d_nhwc(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1, 
     return out
 
 
+def quantize_conv2d(x, pos_x, w, pos_w, x_bits=8, w_bits=8, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1,
+                    bias=None):
+    """x [N,H,W,Ci], w [Co,kh,kw,Ci/g] floating, pos_x / pos_w int32 device tensors of one element"""
+    d = conv_desc(x.shape, w.shape, padding, stride, dilation, groups)
+    ho = lib().catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h)
+    wo = lib().catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w)
+    need = ctypes.c_size_t()
+    check(lib().catchq_quantize_conv2d_workspace_size(ctypes.byref(d), x_bits, w_bits, ctypes.byref(need)))
+    ws = torch.empty(need.value, dtype=torch.int8, device=x.device)
+    y = torch.empty((d.n, ho, wo, d.co), dtype=x.dtype, device=x.device)
+    dt = lambda t: F16 if t.dtype == torch.float16 else F32
+    check(lib().catchq_quantize_conv2d_nhwc(ptr(x), dt(x), ptr(pos_x), x_bits, ptr(w), dt(w), ptr(pos_w), w_bits,
+                                            ctypes.byref(d), ptr(bias), ptr(y), dt(x), ptr(ws), need.value, stream()))
+    return y
+
+
 def conv_route(x_bits, w_bits, x_shape, w_shape, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1):
     d = conv_desc(x_shape, w_shape, padding, stride, dilation, groups)
     return lib().catchq_conv2d_route(x_bits, w_bits, ctypes.byref(d)).decode()

@@ -234,3 +234,22 @@ def test_helper_ops():
     b = torch.randint(-128, 128, (11, 32), dtype=torch.int8).cuda()
     acc, _ = orc.gemm_nt(a.cpu().numpy(), b.cpu().numpy())
     assert same_bits(orc.epilogue(acc, -7), torch.ops.torch_mlu.mm_q(a, -3, b, -4).cpu().numpy())
+
+
+def test_quantize_conv2d_op_matches_conv2d_op():
+    """torch_mlu::quantize_conv2d (positions as device tensors) against torch_mlu::conv2d with the same
+    positions given through the [bitwidths],[positions] q-param encoding."""
+    note("quantize_conv2d op")
+    torch.manual_seed(11)
+    x = torch.randn(2, 16, 9, 9, device="cuda")
+    w = torch.randn(24, 16, 3, 3, device="cuda") * 0.2
+    b = torch.randn(24, device="cuda")
+    px = torch.tensor([-5], dtype=torch.int32, device="cuda")
+    pw = torch.tensor([-8], dtype=torch.int32, device="cuda")
+    got = torch.ops.torch_mlu.quantize_conv2d(x, px, w, pw, b, [1, 1], [1, 1], [1, 1], 1, 8, 8)
+    want = torch.ops.torch_mlu.conv2d(x, w, b, [1, 1], [1, 1], [1, 1], 1, torch.tensor([8., 8.]),
+                                      torch.tensor([-5, -8], dtype=torch.int32))
+    assert got.shape == want.shape == (2, 24, 9, 9)
+    assert torch.equal(got, want)
+    with pytest.raises(Exception):
+        torch.ops.torch_mlu.quantize_conv2d(x, px.cpu(), w, pw, b, [1, 1], [1, 1], [1, 1], 1, 8, 8)

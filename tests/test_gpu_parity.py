@@ -354,6 +354,33 @@ def test_conv_wide(bits, case):
     assert same_bits(orc.epilogue(acc, -22, None, bias), out["y"].cpu().numpy())
 
 
+@pytest.mark.parametrize("bits", [(8, 8), (16, 8), (16, 16)])
+@pytest.mark.parametrize("case", [CONV_CASES[i] for i in (0, 1, 3, 4, 7, 12, 18)])
+def test_quantize_conv2d_device_positions(bits, case):
+    """float operands quantized on the fly with positions read from device memory
+    (cnnlQuantizeConvolutionForward's contract): equal to quantize -> integer conv -> dequant + bias."""
+    n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
+    note("quantize_conv2d", bits, case)
+    r = rng(sum(case[:7]) + bits[0])
+    x = (r.standard_normal((n, h, w, ci)) * 3).astype(np.float32)
+    wt = (r.standard_normal((co, kh, kw, ci // g)) * 0.3).astype(np.float32)
+    bias = r.standard_normal(co).astype(np.float32)
+    pos_x, pos_w = (-4, -8) if bits[0] == 8 else (-11, -8 if bits[1] == 8 else -15)
+    qx, qw = orc.quantize(x, bits[0], pos_x), orc.quantize(wt, bits[1], pos_w)
+    acc, _ = orc.conv2d_nhwc(qx, qw, pad, stride, dil, g)
+    want = orc.epilogue(acc, pos_x + pos_w, None, bias)
+    px = torch.tensor([pos_x], dtype=torch.int32, device="cuda")
+    pw = torch.tensor([pos_w], dtype=torch.int32, device="cuda")
+    got = cabi.quantize_conv2d(cabi.dev(x), px, cabi.dev(wt), pw, bits[0], bits[1], pad, stride, dil, g, cabi.dev(bias))
+    assert same_bits(want, got.cpu().numpy())
+    # half tensors in, half out (one rounding at the end)
+    xh, wh = x.astype(np.float16), wt.astype(np.float16)
+    acc, _ = orc.conv2d_nhwc(orc.quantize(xh, bits[0], pos_x), orc.quantize(wh, bits[1], pos_w), pad, stride, dil, g)
+    want = orc.epilogue(acc, pos_x + pos_w, None, bias, None, 0, np.float16)
+    got = cabi.quantize_conv2d(cabi.dev(xh), px, cabi.dev(wh), pw, bits[0], bits[1], pad, stride, dil, g, cabi.dev(bias))
+    assert same_bits(want, got.cpu().numpy())
+
+
 def test_error_statuses():
     note("error statuses")
     x = torch.zeros(16, device="cuda")
