@@ -1,0 +1,76 @@
+"""Lowering of traced drop-in models (torch_mlu::conv2d / linear nodes + float neighbours) to the
+fused integer plan: the lowered network must reproduce, bit for bit, the plan built directly from
+the architecture description and the same checkpoint."""
+import sys
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    import catch_amd  # noqa: F401
+    from catch_amd import jit, nets, pipeline
+    from catch_amd.core.mlu_quantize import quantize_dynamic_mlu
+
+torch.set_grad_enabled(False)
+
+
+def note(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def dropin_model(layers, x, seed, weight_std, per_channel=True):
+    net = nets.FloatNet(layers, seed=seed, weight_std=weight_std).eval()
+    spec = {"use_avg": False, "data_scale": 1.0, "per_channel": per_channel, "firstconv": False, "iteration": 1}
+    calib = quantize_dynamic_mlu(net, spec, dtype="int8", gen_quant=True)
+    calib(x)
+    qnet = quantize_dynamic_mlu(net)
+    qnet.load_state_dict(calib.state_dict())
+    return net, qnet.to("cuda").eval()
+
+
+@pytest.mark.parametrize("arch,size,std", [("resnet18", 64, 0.05), ("mobilenet_v2", 64, 0.2),
+                                           ("darknet53_yolov3", 64, "he")])
+def test_lowered_trace_equals_direct_plan(arch, size, std):
+    note("jit lowering", arch)
+    layers = nets.NETS[arch]()
+    x = torch.rand(2, 3, size, size, generator=torch.Generator().manual_seed(3))
+    net, qnet = dropin_model(layers, x, 9, std)
+    fused, lowered_layers = jit.lower(qnet, x.cuda())
+    assert [l.kind for l in lowered_layers] == [l.kind for l in layers]
+    for a, b in zip(lowered_layers, layers):
+        assert (a.act, bool(a.add), bool(a.add and a.add_after), a.k, a.stride, a.pad, a.groups) == \
+               (b.act, bool(b.add), bool(b.add and b.add_after), b.k, b.stride, b.pad, b.groups), (a, b)
+    direct = pipeline.FusedNet(layers, pipeline.calibrate(net, x, "int8", True))
+    got, want = fused.forward(x.cuda()), direct.forward(x.cuda())
+    got = got if isinstance(got, tuple) else (got,)
+    want = want if isinstance(want, tuple) else (want,)
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        assert torch.equal(g, w)
+    # and the traced module itself (float tensors between the ops) agrees within the stated tolerance
+    ref = qnet(x.cuda())
+    ref = ref if isinstance(ref, tuple) else (ref,)
+    for g, r in zip(got, ref):
+        span = (r.max() - r.min()).item()
+        assert (g - r).abs().max().item() <= 1e-3 * span + 1e-6
+
+
+def test_lowering_rejects_unknown_nodes():
+    note("jit lowering rejects")
+
+    class Odd(torch.nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, x):
+            return torch.sigmoid(self.inner(x))
+
+    layers = nets.resnet(18)
+    x = torch.rand(1, 3, 64, 64, generator=torch.Generator().manual_seed(4))
+    _, qnet = dropin_model(layers, x, 2, 0.05)
+    with pytest.raises(jit.LoweringError):
+        jit.lower(Odd(qnet), x.cuda())
