@@ -13,7 +13,10 @@
 //
 // The split happens in registers, between the LDS fetch and the MFMA: activations stay plain
 // int16 NHWC in memory.  A-tile rows are 128 bytes (64 int16 of K) = eight 16-byte chunks, the
-// chunk index XOR-ed with (row>>1)&7; weight rows keep the 64-byte layout of the int8 kernel.
+// chunk index XOR-ed with row&7; weight rows keep the 64-byte layout of the int8 kernel.  (row&7
+// leaves a two-way bank conflict on the A fetches; the conflict-free (row>>1)&7 needs a second K
+// position per lane in the loader and measured 8 % slower end to end: the loop is bound by the
+// address arithmetic and issue of the loads, not by the LDS reads.)
 #include "igemm_i8_dma.inc"
 
 namespace catchq {
@@ -99,61 +102,43 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
       vmask[j] = ok ? 1u : 0u;
     }
   }
-  // this lane's position along K, in elements: as a loader of B (16-element chunks) and of A
-  // (8-element chunks).  The A swizzle (row>>1)&7 involves the parity of the 8-row block an
-  // instruction fills, so there is one A position for even blocks and one (32 elements away) for odd.
+  // this lane's position along K, in elements: as a loader of A (8-element chunks) and of B (16)
+  int ka_lin = ((lane & 7) ^ (lane >> 3)) * 8;
   int kb_lin = ((lane & 3) ^ ((lane >> 4) & 3)) * 16;
-  int ka_lin[2], kr[2], kq[2], kci[2], tap[2];
-  unsigned tapbase[2];  // (kr*dh*W + kq*dw)*Ci elements
-  auto normalise_tap = [&](int h) {
-    while (kci[h] >= p.Ci) {
-      kci[h] -= p.Ci;
-      ++tap[h];
-      if (++kq[h] == p.kw) { kq[h] = 0; ++kr[h]; }
-      tapbase[h] = (unsigned)((kr[h] * p.dh * p.W + kq[h] * p.dw) * p.Ci);
+  int kr = 0, kq = 0, kci = ka_lin, tap = 0;
+  unsigned tapbase = 0;  // (kr*dh*W + kq*dw)*Ci elements
+  auto normalise_tap = [&]() {
+    while (kci >= p.Ci) {
+      kci -= p.Ci;
+      ++tap;
+      if (++kq == p.kw) { kq = 0; ++kr; }
+      tapbase = (unsigned)((kr * p.dh * p.W + kq * p.dw) * p.Ci);
     }
   };
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    ka_lin[h] = kci[h] = (((lane & 7) ^ (lane >> 4)) ^ (h * 4)) * 8;
-    kr[h] = kq[h] = tap[h] = 0;
-    tapbase[h] = 0;
-    if constexpr (LOAD == LOAD_CONV) normalise_tap(h);
-  }
+  if constexpr (LOAD == LOAD_CONV) normalise_tap();
 
   auto issue_stage = [&](int stage_off) {
-    const bool kb_ok = kb_lin < p.K;
-    bool ka_ok[2];
-    unsigned a_koff[2], a_bit[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      ka_ok[h] = ka_lin[h] < p.K;
-      a_koff[h] = 2u * ((LOAD == LOAD_CONV) ? tapbase[h] + (unsigned)kci[h] : (unsigned)ka_lin[h]);
-      a_bit[h] = (LOAD == LOAD_CONV) ? (1u << tap[h]) : 1u;
-    }
+    const bool ka_ok = ka_lin < p.K, kb_ok = kb_lin < p.K;
+    const unsigned a_koff = 2u * ((LOAD == LOAD_CONV) ? tapbase + (unsigned)kci : (unsigned)ka_lin);
+    const unsigned a_bit = (LOAD == LOAD_CONV) ? (1u << tap) : 1u;
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       const int slot = wave * NI + j;
       const bool is_a = slot < NIA;  // wave-uniform
       lds_ptr_t dst = (lds_ptr_t)(lds_dyn + stage_off + slot * 1024);  // B slots follow the A slots
       if (is_a) {
-        const bool odd = slot & 1;  // wave-uniform
-        const bool ok = (odd ? ka_ok[1] : ka_ok[0]) && (vmask[j] & (odd ? a_bit[1] : a_bit[0]));
-        const unsigned voff = select_u32(ok, rowbase[j] + (odd ? a_koff[1] : a_koff[0]), OOB);
+        const unsigned voff = select_u32(ka_ok && (vmask[j] & a_bit), rowbase[j] + a_koff, OOB);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, (int)voff, 0, 0, 0);
       } else {
         const unsigned voff = select_u32(kb_ok && vmask[j], rowbase[j] + (unsigned)kb_lin, OOB);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, (int)voff, 0, 0, 0);
       }
     }
+    ka_lin += BK;
     kb_lin += BK;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      ka_lin[h] += BK;
-      if constexpr (LOAD == LOAD_CONV) {
-        kci[h] += BK;
-        normalise_tap(h);
-      }
+    if constexpr (LOAD == LOAD_CONV) {
+      kci += BK;
+      normalise_tap();
     }
   };
 
@@ -172,7 +157,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
   const int frow = lane & 31, fhalf = lane >> 5;
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)lds_dyn;
   // A: elements [ks*32 + fhalf*16, +16) of the step = logical chunks ks*4 + fhalf*2 and the next one
-  const unsigned a_c0 = (unsigned)(((fhalf * 2) ^ ((frow >> 1) & 7)) * 16);
+  const unsigned a_c0 = (unsigned)(((fhalf * 2) ^ (frow & 7)) * 16);
   const unsigned a_row = lds_base + (unsigned)((wave_m * WM + frow) * (BK * 2));
   // B: as in the int8 kernel
   const int swb = (frow >> 2) & 3;
