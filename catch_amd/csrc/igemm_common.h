@@ -44,6 +44,8 @@ inline bool vec_epilogue_ok(int N, const EpiDev &e) {
 template <int DIV, int BIAS, int RESID, int ACT, int YM, int QM, int ACC>
 struct EpiSpec {
   static constexpr bool kGeneric = DIV < 0;
+  static constexpr int kAct = ACT;
+  static constexpr int kQ = QM;
   static __device__ __forceinline__ bool rcp(const EpiDev &e) { return DIV < 0 ? e.chan_rcp != nullptr : DIV == 1; }
   static __device__ __forceinline__ bool truediv(const EpiDev &e) {
     return DIV < 0 ? (e.chan_div != nullptr && e.chan_rcp == nullptr) : DIV == 2;
@@ -157,7 +159,22 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     v4f o = {v[0], v[1], v[2], v[3]};
     *reinterpret_cast<v4f *>(reinterpret_cast<float *>(e.y) + idx) = o;
   }
-  if (S::q8(e)) {
+  if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
+    // values are >= 0 and never NaN here, the requantization scale is 1:
+    //   sat(rne(x * 2^-pos)) = low byte of the float  fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23)
+    // (the product is exact, so the fma rounds once, to an integer, ties to even; clamping before
+    // the rounding equals clamping after it because the bound is an integer multiple of 2^pos)
+    const float hi = __builtin_ldexpf(127.0f, -e.q_neg_pos), sc = __builtin_ldexpf(1.0f, e.q_neg_pos);
+    unsigned b[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float x = (v[t] < hi) ? v[t] : hi;
+      b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
+    }
+    const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+    const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+    *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = lo | hi2;
+  } else if (S::q8(e)) {
     int b[4];
     if (L.unit_q) {
 #pragma unroll
@@ -238,14 +255,17 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
         for (int r = 0; r < 16; ++r)
           stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
       const int64_t mbase = m_w + i * 32;
+      // all reads first: one LDS latency per 32 rows instead of one per iteration
+      v4i av[32 / RPI];
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it)
+        av[it] = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
-        const int row = it * RPI + rsub;
-        const int64_t m = mbase + row;
-        const v4i a = *reinterpret_cast<const v4i *>(stage + row * EPI_STRIDE + cg * 4);
+        const int64_t m = mbase + it * RPI + rsub;
         if (!n_ok || m >= p.M) continue;
         const int64_t idx = m * p.N + n;
-        epi_vec4<S>(a, use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, idx, e);
+        epi_vec4<S>(av[it], use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, idx, e);
       }
     }
   }

@@ -295,8 +295,14 @@ static bool dma_enabled() {
   return on;
 }
 
+int gemm_nt_stream_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
+
 int gemm_nt_mfma_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e,
                     hipStream_t s) {
+  if (dma_enabled()) {  // short K, narrow N, many rows: the streaming kernel
+    const int st = gemm_nt_stream_i8(a, b, M, N, K, e, s);
+    if (st >= 0) return st;
+  }
   IgemmParams p = {};
   p.M = M;
   p.N = (int)N;
@@ -321,6 +327,11 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     return pick_tile<LOAD_C4>(x, w, p, e, s);
   }
   p.K = kh * kw * Ci;
+  if (dma_enabled() && kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
+    // a pointwise convolution is a plain GEMM over the pixels
+    const int st = gemm_nt_stream_i8(x, w, p.M, Co, Ci, e, s);
+    if (st >= 0) return st;
+  }
   if (dma_enabled() && kh * kw <= 32) {  // the DMA loader keeps one validity bit per filter tap
     const int st = igemm_dma_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci, (int64_t)Co * p.K, s);
     if (st >= 0) return st;

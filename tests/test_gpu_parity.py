@@ -145,7 +145,10 @@ def _ints(r, shape, bits):
 
 
 GEMM_SHAPES = [(1, 1, 16), (5, 7, 16), (128, 128, 64), (130, 70, 80), (257, 129, 1040), (64, 1000, 2048),
-               (300, 64, 48), (1, 10, 10), (20, 125, 100), (33, 17, 7)]
+               (300, 64, 48), (1, 10, 10), (20, 125, 100), (33, 17, 7),
+               # many rows, short K, narrow N: the streaming kernel, one shape per (K steps, N fragments) class
+               (5000, 96, 16), (4100, 16, 32), (8200, 144, 32), (4099, 24, 96), (6000, 64, 64), (4097, 160, 32),
+               (4500, 100, 48), (9000, 128, 16), (4096, 36, 80), (5555, 64, 96)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
@@ -287,6 +290,8 @@ CONV_CASES = [
     (2, 24, 11, 13, 24, 3, 3, (1, 1), (2, 2), (1, 1), 24),     # depthwise s2, odd extents
     (1, 320, 7, 7, 320, 3, 3, (1, 1), (1, 1), (1, 1), 320),    # depthwise, many channels, tiny image
     (1, 16, 9, 9, 16, 3, 3, (2, 2), (1, 1), (2, 2), 16),       # depthwise dilated -> strip kernel
+    (2, 32, 50, 50, 16, 1, 1, (0, 0), (1, 1), (1, 1), 1),      # pointwise, 5000 pixels: streaming kernel
+    (1, 16, 70, 71, 96, 1, 1, (0, 0), (1, 1), (1, 1), 1),      # pointwise expand, K = 16
 ]
 
 
