@@ -75,7 +75,7 @@ def layer_profile(fused, x, iters=20):
         if l.kind not in ("conv", "fc"):
             continue
         lq = fused.q[l.name]
-        qx = trace[l.name]["qx"]
+        qx = trace[l.name].get("qx_dev", trace[l.name]["qx"])  # the tensor the kernel reads
         qd = fused.q_demand[l.name][0] if fused.q_demand[l.name] else None
         want_y = fused.f_demand[l.name] or qd is None
         y_half = fused.out_half and l.name in fused.outputs
@@ -83,13 +83,13 @@ def layer_profile(fused, x, iters=20):
             resid = torch.zeros_like(trace[l.name]["y"]) if l.add else None
 
             def run(l=l, lq=lq, qx=qx, qd=qd, want_y=want_y, resid=resid):
-                return ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
+                return ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, fused.padding(l),
                                    [l.stride, l.stride], [1, 1], lq.groups,
                                    {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}[l.act],
                                    want_y, y_half, False, qd[0] if qd else 0, qd[1] if qd else 0, 1.0, 0.1,
                                    bool(l.add_after))
             route = ops.conv2d_route(lq.bw_x, lq.bw_w, list(qx.shape), list(lq.qw.shape[:3]) + [lq.qw.shape[3]],
-                                     [l.pad, l.pad], [l.stride, l.stride], [1, 1], lq.groups)
+                                     fused.padding(l), [l.stride, l.stride], [1, 1], lq.groups)
         else:
             def run(lq=lq, qx=qx):
                 return ops.qlinear(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, False, 0, 0, 1.0)

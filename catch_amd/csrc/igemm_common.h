@@ -11,6 +11,10 @@ struct IgemmParams {
   int N, K;
   int H, W, Ci, Ho, Wo, kh, kw, ph, pw, sh, sw, dh, dw;
   int kwq;  // LOAD_C4: chunks (groups of 4 taps) per filter row
+  // LDS-DMA im2col loader: element strides of the activation tensor (image, image row, output-column
+  // step unit).  A plain NHWC tensor has H*W*Ci, W*Ci, Ci; the pixel-window form of a few-channel
+  // input (a filter row = one contiguous run of kw*C elements) uses other values.
+  unsigned img_stride, row_stride, pix_stride;
   int tiles_n;
   int nblocks;
 };
@@ -199,16 +203,65 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
   }
 }
 
-// Epilogue of one wave.  acc[i][j] are 32x32 MFMA tiles: lane holds column (lane&31) and rows
-// 8*(r/4) + 4*(lane>>5) + (r&3).  (m_w, n_w) = global row / column of the wave tile's origin.
-// Vector variants: the wave transposes 32 rows at a time through its private LDS area `stage` so
-// that a lane owns four consecutive channels of one pixel.
+// this lane's four channels within a wave tile of TN*32 columns starting at n_w
+template <int TN>
+__device__ __forceinline__ int epi_lane_channel(int n_w, int lane) { return n_w + (lane % (TN * 8)) * 4; }
+
+// Vector epilogue of one wave with the lane's per-channel constants supplied by the caller (kernels
+// that run many row groups against the same columns set them up once).
+template <int TM, int TN, int EPI>
+__device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
+                                                   const IgemmParams &p, const EpiDev &e, const EpiLane &L) {
+  typedef typename EpiOf<EPI>::type S;
+  constexpr int WN = TN * 32;
+  constexpr int EPI_STRIDE = WN + 8;  // +8 ints: the two half-waves write different banks
+  const int frow = lane & 31, fhalf = lane >> 5;
+  constexpr int CPR = WN / 4;    // 4-channel groups per staged row
+  constexpr int RPI = 64 / CPR;  // rows the wave moves per iteration
+  const int cg = lane % CPR, rsub = lane / CPR;
+  const int n = n_w + cg * 4;
+  const bool n_ok = n < p.N;
+  const bool use_res = L.use_res;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    // residual rows of this 32-row block: all loads in flight before the staging below
+    v4f resv[32 / RPI];
+    if (use_res) {
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int64_t m = m_w + i * 32 + it * RPI + rsub;
+        resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
+        if (n_ok && m < p.M) resv[it] = *reinterpret_cast<const v4f *>(e.resid + m * p.N + n);
+      }
+    }
+    // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
+    const int64_t mbase = m_w + i * 32;
+    // all reads first: one LDS latency per 32 rows instead of one per iteration
+    v4i av[32 / RPI];
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it)
+      av[it] = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int64_t m = mbase + it * RPI + rsub;
+      if (!n_ok || m >= p.M) continue;
+      const int64_t idx = m * p.N + n;
+      epi_vec4<S>(av[it], use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, idx, e);
+    }
+  }
+}
+
+// Epilogue of one wave.  acc[i][j] is the 32x32 accumulator of rows m_w + i*32 .., columns
+// n_w + j*32 ..; stage is this wave's private LDS area of 32 * (TN*32 + 8) ints.
 template <int TM, int TN, int EPI>
 __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
                                                const IgemmParams &p, const EpiDev &e) {
   typedef typename EpiOf<EPI>::type S;
-  constexpr int WN = TN * 32;
-  constexpr int EPI_STRIDE = WN + 8;  // +8 ints: the two half-waves write different banks
   const int frow = lane & 31, fhalf = lane >> 5;
   if constexpr (EPI == EPI_SCALAR) {
 #pragma unroll
@@ -229,45 +282,9 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
       }
     }
   } else {
-    constexpr int CPR = WN / 4;    // 4-channel groups per staged row
-    constexpr int RPI = 64 / CPR;  // rows the wave moves per iteration
-    const int cg = lane % CPR, rsub = lane / CPR;
-    const int n = n_w + cg * 4;
-    const bool n_ok = n < p.N;
-    const EpiLane L = epi_lane_setup<S>(n, n_ok, e);
-    const bool use_res = L.use_res;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      // residual rows of this 32-row block: all loads in flight before the staging below
-      v4f resv[32 / RPI];
-      if (use_res) {
-#pragma unroll
-        for (int it = 0; it < 32 / RPI; ++it) {
-          const int64_t m = m_w + i * 32 + it * RPI + rsub;
-          resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
-          if (n_ok && m < p.M) resv[it] = *reinterpret_cast<const v4f *>(e.resid + m * p.N + n);
-        }
-      }
-      // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
-      const int64_t mbase = m_w + i * 32;
-      // all reads first: one LDS latency per 32 rows instead of one per iteration
-      v4i av[32 / RPI];
-#pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it)
-        av[it] = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
-#pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it) {
-        const int64_t m = mbase + it * RPI + rsub;
-        if (!n_ok || m >= p.M) continue;
-        const int64_t idx = m * p.N + n;
-        epi_vec4<S>(av[it], use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, idx, e);
-      }
-    }
+    const int n = epi_lane_channel<TN>(n_w, lane);
+    const EpiLane L = epi_lane_setup<S>(n, n < p.N, e);
+    igemm_epilogue_vec<TM, TN, EPI>(acc, stage, m_w, n_w, lane, p, e, L);
   }
 }
 

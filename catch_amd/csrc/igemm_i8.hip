@@ -296,6 +296,8 @@ static bool dma_enabled() {
 }
 
 int gemm_nt_stream_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
+int conv2d_stem_i8(const void *x, const void *w, int N, int H, int W, int Co, int kh, int kw, int sh, int sw, int dh,
+                   int Ho, int Wo, const EpiDev &e, hipStream_t s);
 
 int gemm_nt_mfma_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e,
                     hipStream_t s) {
@@ -321,6 +323,24 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
   p.N = Co;
   p.H = H; p.W = W; p.Ci = Ci; p.Ho = Ho; p.Wo = Wo;
   p.kh = kh; p.kw = kw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+  if (Ci == 4 && ph == 0 && pw == 0 && dw == 1 && dma_enabled()) {  // framed few-channel image: streaming kernel
+    const int st = conv2d_stem_i8(x, w, N, H, W, Co, kh, kw, sh, sw, dh, Ho, Wo, e, s);
+    if (st >= 0) return st;
+  }
+  if (Ci == 4 && pw == 0 && dw == 1 && kw % 4 == 0 && kh <= 32 && dma_enabled()) {
+    // Few-channel input already padded horizontally, filter rows padded to whole 16-byte chunks:
+    // a filter row is one contiguous run of kw*4 bytes of an image row, starting sw*4 bytes further
+    // for every output column.  To the loader that is a convolution with kh x 1 taps of kw*4
+    // "channels" over an image whose "pixels" are sw*4 bytes apart and whose width is Wo.
+    IgemmParams q = p;
+    q.K = kh * kw * 4;
+    q.Ci = kw * 4;
+    q.kw = 1; q.sw = 1; q.pw = 0; q.dw = 1;
+    q.W = Wo;
+    q.img_stride = (unsigned)(H * W * 4); q.row_stride = (unsigned)(W * 4); q.pix_stride = (unsigned)(sw * 4);
+    const int st = igemm_dma_launch(LOAD_CONV, x, w, q, e, (int64_t)N * H * W * 4, (int64_t)Co * q.K, s);
+    if (st >= 0) return st;
+  }
   if (Ci == 4) {
     p.kwq = (kw + 3) / 4;
     p.K = kh * p.kwq * 16;
@@ -332,6 +352,7 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     const int st = gemm_nt_stream_i8(x, w, p.M, Co, Ci, e, s);
     if (st >= 0) return st;
   }
+  p.img_stride = (unsigned)(H * W * Ci); p.row_stride = (unsigned)(W * Ci); p.pix_stride = (unsigned)Ci;
   if (dma_enabled() && kh * kw <= 32) {  // the DMA loader keeps one validity bit per filter tap
     const int st = igemm_dma_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci, (int64_t)Co * p.K, s);
     if (st >= 0) return st;

@@ -150,6 +150,36 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw_nhwc_kernel(const TIn 
   }
 }
 
+// The same into a frame: output [n, oh, ow, CPAD] holds the image at (top, left) and zeros around it
+// (a convolution's zero padding materialised once, so its loads need no border handling).
+template <typename TIn, int BW, int CPAD>
+__global__ __launch_bounds__(kThreads) void quantize_nchw_nhwc_frame_kernel(const TIn *__restrict__ x,
+                                                                           typename QRange<BW>::type *__restrict__ q,
+                                                                           int n, int c, int h, int w, int oh, int ow,
+                                                                           int top, int left, int pos, float scale) {
+  typedef typename QRange<BW>::type TQ;
+  const int64_t total = (int64_t)n * oh * ow, hw = (int64_t)h * w;
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < total; p += stride) {
+    const int ox = (int)(p % ow);
+    const int64_t t = p / ow;
+    const int oy = (int)(t % oh);
+    const int64_t img = t / oh;
+    const int iy = oy - top, ix = ox - left;
+    const bool inside = (unsigned)iy < (unsigned)h && (unsigned)ix < (unsigned)w;
+    TQ out[CPAD];
+#pragma unroll
+    for (int ch = 0; ch < CPAD; ++ch) {
+      out[ch] = 0;
+      if (inside && ch < c) out[ch] = (TQ)quant1<BW>(ld_f(x, (img * c + ch) * hw + (int64_t)iy * w + ix), scale, -pos);
+    }
+    constexpr int BYTES = CPAD * sizeof(TQ);
+    if constexpr (BYTES == 4) *reinterpret_cast<int *>(q + p * CPAD) = *reinterpret_cast<int *>(out);
+    else if constexpr (BYTES == 8) *reinterpret_cast<v2i *>(q + p * CPAD) = *reinterpret_cast<v2i *>(out);
+    else *reinterpret_cast<v4i *>(q + p * CPAD) = *reinterpret_cast<v4i *>(out);
+  }
+}
+
 // General (any C) transpose-quantize through LDS: tile of 64 pixels x 64 channels.
 template <typename TIn, int BW>
 __global__ __launch_bounds__(kThreads) void quantize_nchw_nhwc_tile_kernel(const TIn *__restrict__ x,
@@ -336,6 +366,35 @@ CATCHQ_API int catchq_quantize_nchw_to_nhwc(const void *x, int x_dtype, void *q,
                          : launch_nchw_nhwc<float, 16>(x, q, n, c, h, w, cpad, position, scale, s);
   return bitwidth == 8 ? launch_nchw_nhwc<__half, 8>(x, q, n, c, h, w, cpad, position, scale, s)
                        : launch_nchw_nhwc<__half, 16>(x, q, n, c, h, w, cpad, position, scale, s);
+}
+
+template <typename TIn, int BW, int CPAD>
+static int launch_frame(const void *x, void *q, int n, int c, int h, int w, int oh, int ow, int top, int left, int pos,
+                        float scale, hipStream_t s) {
+  typedef typename QRange<BW>::type TQ;
+  quantize_nchw_nhwc_frame_kernel<TIn, BW, CPAD><<<grid_for((int64_t)n * oh * ow, kThreads), kThreads, 0, s>>>(
+      (const TIn *)x, (TQ *)q, n, c, h, w, oh, ow, top, left, pos, scale);
+  return launch_status();
+}
+
+CATCHQ_API int catchq_quantize_nchw_to_nhwc_frame(const void *x, int x_dtype, void *q, int bitwidth, int n, int c,
+                                                  int h, int w, int cpad, int out_h, int out_w, int top, int left,
+                                                  int position, float scale, catchq_stream_t stream) {
+  if (n < 0 || c < 0 || h < 0 || w < 0 || cpad < c || top < 0 || left < 0 || out_h < h + top || out_w < w + left)
+    return CATCHQ_ERR_SHAPE;
+  if (x_dtype != CATCHQ_F32 && x_dtype != CATCHQ_F16) return CATCHQ_ERR_DTYPE;
+  if (bitwidth != 8 && bitwidth != 16) return CATCHQ_ERR_BITWIDTH;
+  if (position < -126 || position > 126) return CATCHQ_ERR_ARG;
+  if (!((bitwidth == 8 && cpad == 4) || cpad == 8)) return CATCHQ_ERR_SHAPE;  // one 4/8/16-byte vector per pixel
+  if ((int64_t)n * out_h * out_w == 0) return CATCHQ_OK;
+  if (!x || !q || !aligned16(q)) return CATCHQ_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const bool f32 = x_dtype == CATCHQ_F32;
+#define CATCHQ_FRAME(T, BW, CP) launch_frame<T, BW, CP>(x, q, n, c, h, w, out_h, out_w, top, left, position, scale, s)
+  if (bitwidth == 8 && cpad == 4) return f32 ? CATCHQ_FRAME(float, 8, 4) : CATCHQ_FRAME(__half, 8, 4);
+  if (bitwidth == 8) return f32 ? CATCHQ_FRAME(float, 8, 8) : CATCHQ_FRAME(__half, 8, 8);
+  return f32 ? CATCHQ_FRAME(float, 16, 8) : CATCHQ_FRAME(__half, 16, 8);
+#undef CATCHQ_FRAME
 }
 
 static int absmax_blocks(int64_t n) { return grid_for(n / 4, kThreads * 4); }

@@ -387,6 +387,22 @@ Tensor quantize_nhwc_op(const Tensor &x, int64_t bitwidth, int64_t position, int
   return quantize_to_nhwc(x, (int)bitwidth, (int)position, cpad);
 }
 
+// [N,C,H,W] floating -> [N, out_h, out_w, cpad] integers, the image at (top, left), zeros around it
+Tensor quantize_nhwc_frame_op(const Tensor &x, int64_t bitwidth, int64_t position, int64_t cpad, int64_t out_h,
+                              int64_t out_w, int64_t top, int64_t left) {
+  c10::DeviceGuard guard(x.device());
+  const int dt = fp_dtype(x, "quantify only support input float/half");
+  TORCH_CHECK(x.dim() == 4, "a 4-d activation tensor is expected");
+  Tensor xc = x.contiguous();
+  Tensor q = at::empty({x.size(0), out_h, out_w, cpad}, x.options().dtype(int_type(bitwidth)));
+  check_status(catchq_quantize_nchw_to_nhwc_frame(xc.data_ptr(), dt, q.data_ptr(), (int)bitwidth, (int)x.size(0),
+                                                  (int)x.size(1), (int)x.size(2), (int)x.size(3), (int)cpad,
+                                                  (int)out_h, (int)out_w, (int)top, (int)left, (int)position, 1.0f,
+                                                  current_stream()),
+               "torch_mlu::quantize");
+  return q;
+}
+
 // ------------------------------------------------------------------------------------------------
 // the two reference ops
 // ------------------------------------------------------------------------------------------------
@@ -650,6 +666,8 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("quantize(Tensor x, int bitwidth, int position, float scale=1.0) -> Tensor");
   m.def("quantize_dev(Tensor x, int bitwidth, Tensor position) -> Tensor");
   m.def("quantize_nhwc(Tensor x, int bitwidth, int position, int cpad=0) -> Tensor");
+  m.def("quantize_nhwc_frame(Tensor x, int bitwidth, int position, int cpad, int out_h, int out_w, int top, "
+        "int left) -> Tensor");
   m.def("quantize_param(Tensor x, int bitwidth, int mode) -> (Tensor, Tensor, Tensor)");
   m.def("quantize_per_channel(Tensor w, Tensor scales, int bitwidth) -> (Tensor, Tensor, Tensor)");
   m.def("dequantize(Tensor q, int position, float scale=1.0, bool half=False) -> Tensor");
@@ -676,6 +694,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("quantize", &quantize_op);
   m.impl("quantize_dev", &quantize_dev_op);
   m.impl("quantize_nhwc", &quantize_nhwc_op);
+  m.impl("quantize_nhwc_frame", &quantize_nhwc_frame_op);
   m.impl("quantize_param", &quantize_param_op);
   m.impl("quantize_per_channel", &quantize_per_channel_op);
   m.impl("dequantize", &dequantize_op);

@@ -139,6 +139,26 @@ class FusedNet(object):
                   for l in self.layers if l.kind in ("conv", "fc")}
         self._plan_demands()
         self._graph = None
+        # A few-channel int8 network input feeding one k x k convolution: quantize it into a zero frame
+        # (the convolution's padding, materialised) and pad the filter rows to whole groups of 4 taps,
+        # so the first layer fetches filter rows with plain 16-byte loads on the matrix-core route.
+        self.stem = None
+        l0 = self.layers[0]
+        users = [l for l in self.layers if l.src == "input" or (isinstance(l.src, tuple) and "input" in l.src)
+                 or l.add == "input"]
+        if (l0.kind == "conv" and l0.src == "input" and l0.groups == 1 and l0.k > 1 and users == [l0]
+                and self.q[l0.name].bw_x == 8 and self.cdev["input"] == 4):
+            lq = self.q[l0.name]
+            extra = (l0.k + 3) // 4 * 4 - l0.k
+            if extra:
+                lq.qw = torch.nn.functional.pad(lq.qw, (0, 0, 0, extra)).contiguous()  # [Co,kh,kw+extra,4]
+            self.stem = dict(name=l0.name, pad=l0.pad, extra=extra)
+
+    def padding(self, layer):
+        """padding the layer's convolution call gets (the stem's lives in its input frame)"""
+        if self.stem and layer.name == self.stem["name"]:
+            return [0, 0]
+        return [layer.pad, layer.pad]
 
     # which forms of every tensor are needed: 'f' (fp32 NHWC) and/or quantized at (bitwidth, position)
     def _plan_demands(self):
@@ -178,7 +198,12 @@ class FusedNet(object):
         env = {}
         tracing = trace is not None
         for d in self.q_demand["input"]:
-            env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"])
+            if self.stem:
+                sp, h, w = self.stem["pad"], x.shape[2], x.shape[3]
+                env[("input",) + d] = ops.quantize_nhwc_frame(x, d[0], d[1], 4, h + 2 * sp, w + 2 * sp + self.stem["extra"],
+                                                              sp, sp)
+            else:
+                env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"])
         for l in self.layers:
             name = l.name
             if l.kind == "conv":
@@ -187,7 +212,7 @@ class FusedNet(object):
                 resid = env[(l.add, "f")] if l.add else None
                 qd = self.q_demand[name][0] if self.q_demand[name] else None
                 want_y = self.f_demand[name] or tracing or qd is None
-                y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, [l.pad, l.pad],
+                y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, self.padding(l),
                                         [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
                                         self.out_half and name in self.outputs, tracing,
                                         qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
@@ -200,6 +225,10 @@ class FusedNet(object):
                     env[(name,) + d] = ops.quantize(y, d[0], d[1])
                 if tracing:
                     trace[name] = dict(qx=qx, acc=acc, y=y)
+                    if self.stem and name == self.stem["name"]:  # the image inside the frame
+                        sp = self.stem["pad"]
+                        trace[name]["qx_dev"] = qx
+                        trace[name]["qx"] = qx[:, sp:qx.shape[1] - sp, sp:qx.shape[2] - sp - self.stem["extra"]].contiguous()
             elif l.kind == "fc":
                 lq = self.q[name]
                 qx = env[(l.src, lq.bw_x, lq.pos_x)]

@@ -82,6 +82,14 @@ int catchq_quantize_devpos(const void *x, int x_dtype, void *q, int bitwidth, in
 int catchq_quantize_nchw_to_nhwc(const void *x, int x_dtype, void *q, int bitwidth, int n, int c, int h,
                                  int w, int cpad, int position, float scale, catchq_stream_t stream);
 
+/* The same, written into a zero frame: q [N, out_h, out_w, cpad] holds the image at rows top.., columns
+ * left.. and zeros elsewhere -- the zero padding of the convolution that follows
+ * (convolution_forward_internal.cpp:150-153 passes it to the vendor descriptor), materialised once so that a
+ * few-channel first layer can fetch whole filter rows with plain loads.  cpad 4 (int8) or 8. */
+int catchq_quantize_nchw_to_nhwc_frame(const void *x, int x_dtype, void *q, int bitwidth, int n, int c, int h,
+                                       int w, int cpad, int out_h, int out_w, int top, int left, int position,
+                                       float scale, catchq_stream_t stream);
+
 /* cnnlGetQuantizeParamWorkspaceSize + cnnl_quantize_param -> cnnlQuantizeParam
  *                                                          operators/cnnl/internal/quantize_param.cpp:39-96
  * max-abs reduction, then position (mode 0), + scale (1), + offset = 0 (2) written to device memory.

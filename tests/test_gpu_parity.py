@@ -279,6 +279,12 @@ CONV_CASES = [
     (1, 4, 9, 13, 24, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # 4-channel input, 3x3
     (2, 4, 11, 10, 40, 5, 2, (2, 0), (1, 1), (2, 1), 1),       # 4-channel input, 5x2, vertical dilation
     (1, 4, 6, 6, 8, 1, 1, (0, 0), (1, 1), (1, 1), 1),          # 4-channel input, 1x1
+    (2, 4, 36, 37, 64, 7, 8, (0, 0), (2, 2), (1, 1), 1),       # 4-channel framed input, rows of 8 taps (stem form)
+    (1, 4, 12, 20, 24, 3, 4, (1, 0), (1, 1), (1, 1), 1),       # 4-channel, rows of 4 taps, vertical padding only
+    (2, 4, 9, 33, 40, 5, 12, (2, 0), (1, 3), (2, 1), 1),       # 4-channel, rows of 12 taps, stride 3, vertical dilation
+    (2, 4, 100, 101, 64, 7, 8, (0, 0), (2, 2), (1, 1), 1),     # framed stem, 4512 pixels: streaming stem kernel, 7 steps
+    (3, 4, 90, 91, 32, 3, 4, (0, 0), (2, 2), (1, 1), 1),       # framed 3x3 stem (rows of 4 taps, two rows per K step)
+    (1, 4, 70, 72, 40, 4, 4, (0, 0), (1, 1), (2, 1), 1),       # even filter height, stride 1, vertical dilation, Co = 40
     (1, 64, 9, 9, 72, 1, 1, (0, 0), (1, 1), (1, 1), 1),        # Co % 64 != 0
     (1, 32, 5, 5, 30, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # Co % 4 != 0 -> scalar epilogue
     (2, 32, 12, 12, 32, 3, 3, (1, 1), (1, 1), (1, 1), 32),     # depthwise s1
@@ -384,6 +390,18 @@ def test_quantize_conv2d_device_positions(bits, case):
     want = orc.epilogue(acc, pos_x + pos_w, None, bias, None, 0, np.float16)
     got = cabi.quantize_conv2d(cabi.dev(xh), px, cabi.dev(wh), pw, bits[0], bits[1], pad, stride, dil, g, cabi.dev(bias))
     assert same_bits(want, got.cpu().numpy())
+
+
+def test_quantize_into_frame():
+    """NCHW float -> NHWC int8/int16 inside a zero frame equals the plain transposing quantizer placed by hand."""
+    note("quantize frame")
+    r = rng(77)
+    x = (r.standard_normal((2, 3, 9, 11)) * 40).astype(np.float32)
+    for bits, cpad in ((8, 4), (8, 8), (16, 8)):
+        want = np.zeros((2, 9 + 5, 11 + 7, cpad), np.int8 if bits == 8 else np.int16)
+        want[:, 2:11, 3:14, :3] = orc.quantize(np.transpose(x, (0, 2, 3, 1)), bits, -1)
+        got = torch.ops.torch_mlu.quantize_nhwc_frame(cabi.dev(x), bits, -1, cpad, 14, 18, 2, 3)
+        assert np.array_equal(want, got.cpu().numpy())
 
 
 def test_error_statuses():
