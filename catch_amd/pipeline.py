@@ -191,12 +191,23 @@ class FusedNet(object):
                 self.f_demand[l.name] = True
 
     # ------------------------------------------------------------------------------------------
-    def forward(self, x, trace=None):
+    def forward(self, x, trace=None, timers=None):
         """x: [N,3,H,W] fp32 (NCHW) on the device.  trace: optional dict filled with, per conv/fc
-        layer, its quantized input, int32 accumulators and fp32 output (as NHWC tensors)."""
+        layer, its quantized input, int32 accumulators and fp32 output (as NHWC tensors).
+        timers: optional dict; every conv/fc launch is bracketed by a pair of events recorded on
+        the current stream and the pair is appended to timers[layer name] (durations of the
+        launches in their real sequence, caches as the previous layer left them)."""
         ops = torch.ops.torch_mlu
         env = {}
         tracing = trace is not None
+
+        def tick(name):
+            if timers is None:
+                return None
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            timers.setdefault(name, []).append(ev)
+            return ev
         for d in self.q_demand["input"]:
             if self.stem:
                 sp, h, w = self.stem["pad"], x.shape[2], x.shape[3]
@@ -212,11 +223,13 @@ class FusedNet(object):
                 resid = env[(l.add, "f")] if l.add else None
                 qd = self.q_demand[name][0] if self.q_demand[name] else None
                 want_y = self.f_demand[name] or tracing or qd is None
+                tick(name)
                 y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, self.padding(l),
                                         [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
                                         self.out_half and name in self.outputs, tracing,
                                         qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
                                         bool(l.add_after))
+                tick(name)
                 if want_y:
                     env[(name, "f")] = y
                 if qd:
@@ -233,7 +246,9 @@ class FusedNet(object):
                 lq = self.q[name]
                 qx = env[(l.src, lq.bw_x, lq.pos_x)]
                 qx2 = qx.reshape(qx.shape[0], -1)
+                tick(name)
                 y, _, acc = ops.qlinear(qx2, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, tracing, 0, 0, 1.0)
+                tick(name)
                 env[(name, "f")] = y
                 if tracing:
                     trace[name] = dict(qx=qx2, acc=acc, y=y)
