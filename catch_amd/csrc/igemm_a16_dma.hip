@@ -277,17 +277,17 @@ static int pick_a16_tile(const void *a, const void *b, const IgemmParams &p, con
   constexpr int64_t kCUs = 256;
   int tile = forced_tile();
   if (!tile) {
-    if (p.N >= 256 && p.K >= 256 && blocks(128, 256) >= kCUs * 3 / 2) tile = 128256;
-    else if (p.N <= 64 || p.K < 256) tile = 64064;
-    else if (blocks(128, 128) >= kCUs * 3 / 2) tile = 128128;
-    else if (blocks(64, 128) >= kCUs * 3 / 2) tile = 64128;
+    // Measured on every Darknet-53 layer (bs16, 416x416): the 64x64 tile wins or ties everywhere -- two
+    // accumulator sets and the digit split keep a wave busy enough, and small tiles mean more resident
+    // blocks per CU.  Only GEMMs far beyond those sizes take the wide tile.
+    if (p.N >= 256 && p.K >= 256 && (int64_t)p.M * p.N * p.K >= (1ll << 34)) tile = 128256;
     else tile = 64064;
   }
   switch (tile) {
     case 128256: return launch_a16<128, 256, 2, 4, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
-    case 128128: return launch_a16<128, 128, 2, 2, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
-    case 64128: return launch_a16<64, 128, 2, 2, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
-    default: return launch_a16<64, 64, 2, 2, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+    case 128128: return launch_a16<128, 128, 2, 2, 3, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+    case 64128: return launch_a16<64, 128, 2, 2, 3, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
+    default: return launch_a16<64, 64, 2, 2, 3, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
   }
 }
 
