@@ -216,9 +216,9 @@ def test_gemm_wide(bits, m, n, k):
     assert same_bits(orc.epilogue(acc, -20, None, bias), out["y"].cpu().numpy())
 
 
-@pytest.mark.parametrize("m,n,k", [(16384, 768, 256), (8192, 768, 320), (4096, 768, 256), (4096, 3072, 768)])
+@pytest.mark.parametrize("m,n,k", [(16384, 1024, 1024), (8192, 768, 320), (4096, 768, 256), (4096, 3072, 768)])
 def test_gemm_a16_tiles(m, n, k):
-    """int16 x int8 on the matrix cores, one shape per tile configuration, with the extreme digits
+    """int16 x int8 on the matrix cores (the first shape takes the wide 128x256 tile), with the extreme digits
     (-32768, 32767, -1, 0, 255, 256) planted; sampled rows against the oracle, all rows by linearity."""
     note("gemm_a16", m, n, k, cabi.lib().catchq_gemm_route(16, 8, m, n, k))
     r = rng(m + k)
