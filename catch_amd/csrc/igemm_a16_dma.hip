@@ -308,6 +308,109 @@ int gemm_nt_mfma_a16(const void *a, const void *b, int64_t M, int64_t N, int64_t
   return igemm_a16_launch(LOAD_GEMM, a, b, p, e, M * K * 2, N * K, s);
 }
 
+// ---- few-channel first layer, int16 activations -------------------------------------------------
+// Input [N, H, W, 8] int16 already framed by its zero padding, filter rows padded to 4 taps (weights
+// [Co][kh][4][8] int8, the extra tap zero).  A filter row is 64 contiguous bytes of an image row and
+// exactly one MFMA K step (32 elements); the K half a lane owns is two adjacent pixels.  Weights and
+// their column sums live in registers, A fragments come straight from global memory, a wave handles
+// 32 consecutive output pixels x 32 output channels (blockIdx.y selects the channel group).
+typedef int v4i_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int STEPS, int EPI>
+__global__ __launch_bounds__(256, 2) void stem_a16_kernel(const int16_t *__restrict__ X, const int8_t *__restrict__ B,
+                                                         IgemmParams p, EpiDev e, int ngroups) {
+  resolve_exp2(e);
+  typedef typename EpiOf<EPI>::type S;
+  constexpr int EPI_STRIDE = 32 + 8;
+  constexpr int DEPTH = 2;
+  extern __shared__ __attribute__((aligned(16))) int stem_lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int n_base = blockIdx.y * 32;
+  const int rowbytes = p.W * 16;
+
+  v4i fb[STEPS];
+  int wsum = 0;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int n = n_base + frow;
+    fb[s] = v4i{0, 0, 0, 0};
+    if (n < p.N) fb[s] = *reinterpret_cast<const v4i *>(B + (int64_t)n * p.K + s * 32 + fhalf * 16);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) wsum = __builtin_amdgcn_sdot4(fb[s][d], 0x01010101, wsum, false);
+  }
+  const unsigned wcorr = (unsigned)(wsum + __shfl_xor(wsum, 32, 64)) << 7;  // 128 * sum_k w[n][k], n = column of this lane
+  const int n_lane = epi_lane_channel<1>(n_base, lane);
+  const EpiLane L = epi_lane_setup<S>(n_lane, n_lane < p.N, e);
+
+  auto load_a = [&](int g, v4i (&fa)[STEPS][2]) {
+    const unsigned m = (unsigned)g * 32u + (unsigned)frow;
+    const bool ok = g < ngroups && m < (unsigned)p.M;
+    const unsigned mm = ok ? m : 0u;
+    const unsigned t = mm / (unsigned)p.Wo, wo = mm - t * (unsigned)p.Wo;
+    const unsigned img = t / (unsigned)p.Ho, ho = t - img * (unsigned)p.Ho;
+    const int8_t *base = reinterpret_cast<const int8_t *>(X) +
+                         (size_t)((img * (unsigned)p.H + ho * (unsigned)p.sh) * (unsigned)p.W + wo * (unsigned)p.sw) * 16 + fhalf * 32;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int8_t *row = base + (int64_t)s * p.dh * rowbytes;
+      fa[s][0] = *reinterpret_cast<const v4i_a4 *>(row);
+      fa[s][1] = *reinterpret_cast<const v4i_a4 *>(row + 16);
+    }
+  };
+
+  const int gw = blockIdx.x * 4 + wave, nw = gridDim.x * 4;
+  v4i ring[DEPTH][STEPS][2];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_a(gw + d * nw, ring[d]);
+
+  int *stage = stem_lds + wave * 32 * EPI_STRIDE;
+  for (int g0 = gw; g0 < ngroups; g0 += DEPTH * nw) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int g = g0 + d * nw;
+      if (g >= ngroups) break;  // wave-uniform
+      v16i acc_hi, acc_lo;
+      const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        v4i hi, lo;
+        split_i16(ring[d][s][0], ring[d][s][1], hi, lo);
+        acc_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(hi, fb[s], s == 0 ? zero : acc_hi, 0, 0, 0);
+        acc_lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, fb[s], s == 0 ? zero : acc_lo, 0, 0, 0);
+      }
+      load_a(g + DEPTH * nw, ring[d]);
+      v16i acc[1][1];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[0][0][r] = (int)(((unsigned)acc_hi[r] << 8) + (unsigned)acc_lo[r] + wcorr);
+      igemm_epilogue_vec<1, 1, EPI>(acc, stage, (int64_t)g * 32, n_base, lane, p, e, L);
+    }
+  }
+}
+
+// convolution of a framed 8-channel int16 image with 3-row filters of 4 taps (zero tap included);
+// -1 when the shape is not this kernel's
+static int conv2d_stem_a16(const void *x, const void *w, int N, int H, int W, int Co, int kh, int kw, int sh, int sw,
+                           int dh, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
+  if (kw != 4 || kh != 3 || Co > 128 || (int64_t)N * Ho * Wo < 4096) return -1;
+  if ((int64_t)N * Ho * Wo >= (1ll << 31) - 64 || (int64_t)N * H * W >= (1ll << 27)) return -1;  // 32-bit indices
+  IgemmParams p = {};
+  p.M = (int64_t)N * Ho * Wo;
+  p.N = Co;
+  p.K = kh * kw * 8;
+  p.H = H; p.W = W; p.Ho = Ho; p.Wo = Wo; p.kh = kh; p.kw = kw; p.sh = sh; p.sw = sw; p.dh = dh;
+  if (pick_epilogue(p.N, e) == EPI_SCALAR) return -1;
+  constexpr int LDS_BYTES = 4 * 32 * (32 + 8) * 4;
+  const int64_t ngroups = (p.M + 31) / 32;
+  const int ngrp = (p.N + 31) / 32;
+  int blocks = (int)((ngroups + 3) / 4);
+  if (blocks > 256 * 4 / ngrp) blocks = 256 * 4 / ngrp;
+  stem_a16_kernel<3, EPI_VECTOR><<<dim3(blocks, ngrp), 256, LDS_BYTES, s>>>((const int16_t *)x, (const int8_t *)w, p, e,
+                                                                           (int)ngroups);
+  return launch_status();
+}
+
 int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
                     int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
   IgemmParams p = {};
@@ -316,6 +419,10 @@ int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, i
   p.H = H; p.W = W; p.Ci = Ci; p.Ho = Ho; p.Wo = Wo;
   p.kh = kh; p.kw = kw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
   p.K = kh * kw * Ci;
+  if (Ci == 8 && ph == 0 && pw == 0 && dw == 1) {  // framed few-channel image: streaming kernel
+    const int st = conv2d_stem_a16(x, w, N, H, W, Co, kh, kw, sh, sw, dh, Ho, Wo, e, s);
+    if (st >= 0) return st;
+  }
   return igemm_a16_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci * 2, (int64_t)Co * p.K, s);
 }
 

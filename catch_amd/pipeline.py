@@ -146,12 +146,12 @@ class FusedNet(object):
         l0 = self.layers[0]
         users = [l for l in self.layers if l.src == "input" or (isinstance(l.src, tuple) and "input" in l.src)
                  or l.add == "input"]
-        if (l0.kind == "conv" and l0.src == "input" and l0.groups == 1 and l0.k > 1 and users == [l0]
-                and self.q[l0.name].bw_x == 8 and self.cdev["input"] == 4):
+        few = (self.q[l0.name].bw_x, self.cdev["input"]) in ((8, 4), (16, 8)) if l0.kind == "conv" else False
+        if l0.kind == "conv" and l0.src == "input" and l0.groups == 1 and l0.k > 1 and users == [l0] and few:
             lq = self.q[l0.name]
             extra = (l0.k + 3) // 4 * 4 - l0.k
             if extra:
-                lq.qw = torch.nn.functional.pad(lq.qw, (0, 0, 0, extra)).contiguous()  # [Co,kh,kw+extra,4]
+                lq.qw = torch.nn.functional.pad(lq.qw, (0, 0, 0, extra)).contiguous()  # [Co,kh,kw+extra,C]
             self.stem = dict(name=l0.name, pad=l0.pad, extra=extra)
 
     def padding(self, layer):
@@ -211,8 +211,8 @@ class FusedNet(object):
         for d in self.q_demand["input"]:
             if self.stem:
                 sp, h, w = self.stem["pad"], x.shape[2], x.shape[3]
-                env[("input",) + d] = ops.quantize_nhwc_frame(x, d[0], d[1], 4, h + 2 * sp, w + 2 * sp + self.stem["extra"],
-                                                              sp, sp)
+                env[("input",) + d] = ops.quantize_nhwc_frame(x, d[0], d[1], self.cdev["input"], h + 2 * sp,
+                                                              w + 2 * sp + self.stem["extra"], sp, sp)
             else:
                 env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"])
         for l in self.layers:

@@ -350,6 +350,8 @@ def test_conv_leaky_relu_and_residual_order(case, after):
     (2, 8, 13, 13, 32, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # 8 channels: K = 72, ragged last K step
     (1, 24, 9, 9, 255, 1, 1, (0, 0), (1, 1), (1, 1), 1),        # detection head: 255 outputs
     (2, 256, 12, 12, 320, 3, 3, (1, 1), (1, 1), (1, 1), 1),     # wider tile
+    (2, 8, 70, 71, 32, 3, 4, (0, 0), (1, 1), (1, 1), 1),        # framed 8-channel first layer: streaming kernel
+    (1, 8, 100, 101, 40, 3, 4, (0, 0), (2, 2), (2, 1), 1),      # the same, stride 2, vertical dilation, 40 channels
 ])
 def test_conv_wide(bits, case):
     n, ci, h, w, co, kh, kw, pad, stride, dil, g = case
