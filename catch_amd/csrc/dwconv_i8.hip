@@ -1,8 +1,8 @@
 // Depthwise int8 convolution (groups == Ci == Co) on NHWC tensors: a stencil, not a contraction,
 // so no matrix cores.  Two kernels:
 //  * dw3x3_kernel: 3x3, dilation 1, stride 1 or 2 (every depthwise layer of the MobileNet family).
-//    A lane owns 4 channels x (2 rows x 4 columns) of output pixels, slides the input window through
-//    registers and finishes with the vector epilogue of the GEMM kernels; adjacent lanes hold adjacent
+//    A lane owns 4 channels x (2 rows x 4 columns) of output pixels, transposes the input window in
+//    registers so that v_dot4_i32_i8 sums the taps of a filter row, and finishes with the vector epilogue of the GEMM kernels; adjacent lanes hold adjacent
 //    channel quads, so loads and stores of a wave are contiguous runs of the NHWC row.
 //  * dwconv_i8_kernel: any filter up to 5x5, any stride/dilation.  A block owns a strip of output pixels of one image row and all channels of a
 // 64-channel slab; the input rows the strip needs are staged in LDS once and every tap is read
@@ -109,7 +109,6 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
   resolve_exp2(e);
   typedef typename EpiOf<EPI>::type Sp;
   constexpr int PW = DW3_PW, PH = DW3_PH;
-  constexpr int NC = (PW - 1) * S + 3;  // input columns of the window
   constexpr int NR = (PH - 1) * S + 3;  // input rows of the window
   const int item = blockIdx.x * 256 + threadIdx.x;
   if (item >= p.items) return;
@@ -117,17 +116,28 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
   const int ho0 = blockIdx.y * PH, img = blockIdx.z;
   const int c = cq * 4;
 
-  // 36 filter bytes of the four channels ([channel][tap]) -> sign-extended taps
+  // The multiply-accumulate runs on v_dot4_i32_i8, which sums four byte products: the four bytes of
+  // an operand must be four taps of ONE channel.  A pixel's dword holds four channels, so groups of
+  // four horizontally adjacent pixels are transposed (4x4 bytes, 8 byte permutes, the first stage
+  // shared between overlapping groups) into one dword per channel; a filter row is the byte vector
+  // (w0, w1, w2, 0) or, for the output one pixel to the right within the same group, (0, w0, w1, w2).
+  // 36 filter bytes of the four channels ([channel][tap]):
   int wraw[9];
 #pragma unroll
   for (int i = 0; i < 9; ++i) wraw[i] = *reinterpret_cast<const int *>(w + (int64_t)c * 9 + 4 * i);
-  int wu[9][4];
+  int wa[4][3], wb[4][3];  // [channel][filter row]
 #pragma unroll
-  for (int t = 0; t < 9; ++t)
+  for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int b = j * 9 + t;
-      wu[t][j] = (int)(int8_t)(wraw[b >> 2] >> (8 * (b & 3)));
+    for (int r = 0; r < 3; ++r) {
+      unsigned v = 0;
+#pragma unroll
+      for (int q = 0; q < 3; ++q) {
+        const int b = j * 9 + r * 3 + q;
+        v |= (((unsigned)wraw[b >> 2] >> (8 * (b & 3))) & 0xffu) << (8 * q);
+      }
+      wa[j][r] = (int)v;
+      wb[j][r] = (int)(v << 8);
     }
 
   int acc[PH][PW][4];
@@ -138,35 +148,49 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[a][b][j] = 0;
 
+  constexpr int NG = (S == 1) ? 2 : 4;  // transposed groups per input row: pixels 0-3, 2-5 [, 4-7, 6-9]
+  constexpr int NCL = 2 * NG + 2;       // input columns loaded (stride 2: one more than the window, weight 0)
   const int hi0 = ho0 * S - p.ph, wi0 = wg * PW * S - p.pw;
   const int8_t *xi = x + (int64_t)img * p.H * p.W * p.C + c;
 #pragma unroll
   for (int ri = 0; ri < NR; ++ri) {
     const int hi = hi0 + ri;
     const bool row_ok = (unsigned)hi < (unsigned)p.H;
-    int xr[NC];
+    unsigned xr[NCL];
 #pragma unroll
-    for (int col = 0; col < NC; ++col) {
+    for (int col = 0; col < NCL; ++col) {
       const int wi = wi0 + col;
       xr[col] = 0;
       if (row_ok && (unsigned)wi < (unsigned)p.W)
-        xr[col] = *reinterpret_cast<const int *>(xi + ((int64_t)hi * p.W + wi) * p.C);
+        xr[col] = *reinterpret_cast<const unsigned *>(xi + ((int64_t)hi * p.W + wi) * p.C);
+    }
+    // first transposition stage on pixel pairs (2m, 2m+1): bytes (a0,b0,a1,b1) and (a2,b2,a3,b3)
+    unsigned lo[NG + 1], hi2[NG + 1];
+#pragma unroll
+    for (int m = 0; m <= NG; ++m) {
+      lo[m] = __builtin_amdgcn_perm(xr[2 * m + 1], xr[2 * m], 0x05010400u);
+      hi2[m] = __builtin_amdgcn_perm(xr[2 * m + 1], xr[2 * m], 0x07030602u);
     }
 #pragma unroll
-    for (int col = 0; col < NC; ++col) {
-      int xs[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xs[j] = (int)(int8_t)(xr[col] >> (8 * j));
+    for (int g = 0; g < NG; ++g) {
+      // second stage: group g = pixels 2g .. 2g+3, one dword per channel
+      int t[4];
+      t[0] = (int)__builtin_amdgcn_perm(lo[g + 1], lo[g], 0x05040100u);
+      t[1] = (int)__builtin_amdgcn_perm(lo[g + 1], lo[g], 0x07060302u);
+      t[2] = (int)__builtin_amdgcn_perm(hi2[g + 1], hi2[g], 0x05040100u);
+      t[3] = (int)__builtin_amdgcn_perm(hi2[g + 1], hi2[g], 0x07060302u);
 #pragma unroll
       for (int py = 0; py < PH; ++py) {
         const int r = ri - py * S;
         if (r < 0 || r > 2) continue;
 #pragma unroll
-        for (int q = 0; q < 3; ++q) {
-          const int d = col - q;
-          if (d < 0 || d % S != 0 || d / S >= PW) continue;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) acc[py][d / S][j] += xs[j] * wu[r * 3 + q][j];
+        for (int j = 0; j < 4; ++j) {
+          if constexpr (S == 1) {  // group g serves outputs 2g (taps at bytes 0..2) and 2g+1 (bytes 1..3)
+            acc[py][2 * g][j] = __builtin_amdgcn_sdot4(t[j], wa[j][r], acc[py][2 * g][j], false);
+            acc[py][2 * g + 1][j] = __builtin_amdgcn_sdot4(t[j], wb[j][r], acc[py][2 * g + 1][j], false);
+          } else {                 // stride 2: group g starts at input pixel 2g = the window of output g
+            acc[py][g][j] = __builtin_amdgcn_sdot4(t[j], wa[j][r], acc[py][g][j], false);
+          }
         }
       }
     }
