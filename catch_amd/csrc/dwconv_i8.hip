@@ -140,13 +140,7 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
       wb[j][r] = (int)(v << 8);
     }
 
-  int acc[PH][PW][4];
-#pragma unroll
-  for (int a = 0; a < PH; ++a)
-#pragma unroll
-    for (int b = 0; b < PW; ++b)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[a][b][j] = 0;
+  int acc[PH][PW][4];  // every sum starts with filter row 0 (accumulator operand 0), no zeroing pass
 
   constexpr int NG = (S == 1) ? 2 : 4;  // transposed groups per input row: pixels 0-3, 2-5 [, 4-7, 6-9]
   constexpr int NCL = 2 * NG + 2;       // input columns loaded (stride 2: one more than the window, weight 0)
@@ -157,12 +151,11 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
     const int hi = hi0 + ri;
     const bool row_ok = (unsigned)hi < (unsigned)p.H;
     unsigned xr[NCL];
+    const int8_t *rowp = xi + ((int64_t)hi * p.W + wi0) * p.C;  // column 0 of the window (may lie outside: masked below)
 #pragma unroll
     for (int col = 0; col < NCL; ++col) {
-      const int wi = wi0 + col;
       xr[col] = 0;
-      if (row_ok && (unsigned)wi < (unsigned)p.W)
-        xr[col] = *reinterpret_cast<const unsigned *>(xi + ((int64_t)hi * p.W + wi) * p.C);
+      if (row_ok && (unsigned)(wi0 + col) < (unsigned)p.W) xr[col] = *reinterpret_cast<const unsigned *>(rowp + col * p.C);
     }
     // first transposition stage on pixel pairs (2m, 2m+1): bytes (a0,b0,a1,b1) and (a2,b2,a3,b3)
     unsigned lo[NG + 1], hi2[NG + 1];
@@ -186,10 +179,10 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if constexpr (S == 1) {  // group g serves outputs 2g (taps at bytes 0..2) and 2g+1 (bytes 1..3)
-            acc[py][2 * g][j] = __builtin_amdgcn_sdot4(t[j], wa[j][r], acc[py][2 * g][j], false);
-            acc[py][2 * g + 1][j] = __builtin_amdgcn_sdot4(t[j], wb[j][r], acc[py][2 * g + 1][j], false);
+            acc[py][2 * g][j] = __builtin_amdgcn_sdot4(t[j], wa[j][r], r == 0 ? 0 : acc[py][2 * g][j], false);
+            acc[py][2 * g + 1][j] = __builtin_amdgcn_sdot4(t[j], wb[j][r], r == 0 ? 0 : acc[py][2 * g + 1][j], false);
           } else {                 // stride 2: group g starts at input pixel 2g = the window of output g
-            acc[py][g][j] = __builtin_amdgcn_sdot4(t[j], wa[j][r], acc[py][g][j], false);
+            acc[py][g][j] = __builtin_amdgcn_sdot4(t[j], wa[j][r], r == 0 ? 0 : acc[py][g][j], false);
           }
         }
       }

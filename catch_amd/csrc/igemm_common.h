@@ -172,7 +172,7 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     unsigned b[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const float x = (v[t] < hi) ? v[t] : hi;
+      const float x = __builtin_amdgcn_fmed3f(v[t], 0.0f, hi);  // v >= 0: this is min(v, hi), one instruction
       b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
     }
     const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
