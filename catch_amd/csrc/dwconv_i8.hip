@@ -98,7 +98,8 @@ struct Dw3Params {
   int N, H, W, C, ph, pw, Ho, Wo;
   int CQ;     // channel quads
   int WG;     // column groups per output row
-  int items;  // WG * CQ
+  int HG;     // row groups per image
+  int items;  // HG * WG * CQ: work items of one image
 };
 
 constexpr int DW3_PW = 4, DW3_PH = 2;
@@ -110,10 +111,11 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
   typedef typename EpiOf<EPI>::type Sp;
   constexpr int PW = DW3_PW, PH = DW3_PH;
   constexpr int NR = (PH - 1) * S + 3;  // input rows of the window
-  const int item = blockIdx.x * 256 + threadIdx.x;
+  const int item = blockIdx.x * 256 + threadIdx.x;  // (row group, column group, channel quad), channels fastest
   if (item >= p.items) return;
-  const int wg = item / p.CQ, cq = item - wg * p.CQ;
-  const int ho0 = blockIdx.y * PH, img = blockIdx.z;
+  const int t0 = item / p.CQ, cq = item - t0 * p.CQ;
+  const int hg = t0 / p.WG, wg = t0 - hg * p.WG;
+  const int ho0 = hg * PH, img = blockIdx.y;
   const int c = cq * 4;
 
   // The multiply-accumulate runs on v_dot4_i32_i8, which sums four byte products: the four bytes of
@@ -218,12 +220,11 @@ static int dw3x3(const void *x, const void *w, int N, int H, int W, int C, int k
   if (kh != 3 || kw != 3 || dh != 1 || dw != 1 || sh != sw || (sh != 1 && sh != 2)) return -1;
   const int epi = pick_epilogue(C, e);
   if (epi == EPI_SCALAR) return -1;
-  Dw3Params p = {N, H, W, C, ph, pw, Ho, Wo, C / 4, (Wo + DW3_PW - 1) / DW3_PW, 0};
-  const int64_t items = (int64_t)p.WG * p.CQ;
-  const int rows = (Ho + DW3_PH - 1) / DW3_PH;
-  if (items > 0x7fffff00 || rows > 65535 || N > 65535) return -1;
+  Dw3Params p = {N, H, W, C, ph, pw, Ho, Wo, C / 4, (Wo + DW3_PW - 1) / DW3_PW, (Ho + DW3_PH - 1) / DW3_PH, 0};
+  const int64_t items = (int64_t)p.HG * p.WG * p.CQ;
+  if (items > 0x7fffff00 || N > 65535) return -1;
   p.items = (int)items;
-  const dim3 grid((unsigned)((items + 255) / 256), (unsigned)rows, (unsigned)N);
+  const dim3 grid((unsigned)((items + 255) / 256), (unsigned)N);
   const bool s2 = sh == 2;
   switch (epi) {
     case EPI_Q8_RELU6: s2 ? dw3x3_launch<2, EPI_Q8_RELU6>(x, w, p, grid, e, s) : dw3x3_launch<1, EPI_Q8_RELU6>(x, w, p, grid, e, s); break;
