@@ -39,7 +39,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--seq-passes", type=int, default=10, help="eager passes timed launch by launch for the roofline")
     ap.add_argument("--calib-images", type=int, default=8)
-    ap.add_argument("--cpu-images", type=int, default=2)
+    ap.add_argument("--cpu-images", type=int, default=0, help="images of the batch the CPU baseline runs (0: the whole batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -213,7 +213,8 @@ def main():
     if not args.no_extras:
         result["extras"] = extras()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(layers, sd, x[:args.cpu_images], outs[0][:args.cpu_images].float().cpu(),
+        n_cpu = args.cpu_images or batch
+        result["cpu_baseline"] = cpu_baseline(layers, sd, x[:n_cpu], outs[0][:n_cpu].float().cpu(),
                                               fused.outputs[0])
     result["calibration_s"] = round(t_cal, 2)
     print(json.dumps(result))
@@ -249,7 +250,7 @@ def cpu_baseline(layers, sd, x_sample, gpu_logits, out_name):
     from oracle import netref
     sdn = {k: v.detach().cpu().numpy() for k, v in sd.items()}
     t0 = time.time()
-    t, _ = netref.run(layers, sdn, x_sample.numpy())
+    t, _ = netref.run(layers, sdn, x_sample.numpy(), record=False)
     dt = time.time() - t0
     if gpu_logits.dim() == 4:  # logical NCHW -> the oracle's NHWC
         gpu_logits = gpu_logits.permute(0, 2, 3, 1).contiguous()

@@ -21,8 +21,9 @@ def _key(name):
     return "mods." + name.replace(".", "_") + "."
 
 
-def run(layers, sd, x_nchw):
-    """sd: dict of numpy arrays (weight [Co,Ci/g,kh,kw] / [N,K], bias, scale, quantized_mode)."""
+def run(layers, sd, x_nchw, record=True):
+    """sd: dict of numpy arrays (weight [Co,Ci/g,kh,kw] / [N,K], bias, scale, quantized_mode).
+    record=False keeps only the activations (no per-layer quantized inputs / integer sums)."""
     t = {"input": np.ascontiguousarray(np.transpose(np.asarray(x_nchw, np.float32), (0, 2, 3, 1)))}
     rec = {}
     for l in layers:
@@ -47,7 +48,8 @@ def run(layers, sd, x_nchw):
                 resid = None
             y = epilogue(acc, d["pos_x"] + d["pos_w"], d["new_scale"], b, resid, _ACT[l.act], act_slope=LEAKY_SLOPE,
                          resid_after_act=bool(l.add_after))
-            rec[l.name] = dict(qx=qx, acc=acc, y=y, overflow=ovf, pos_x=d["pos_x"], pos_w=d["pos_w"])
+            if record:
+                rec[l.name] = dict(qx=qx, acc=acc, y=y, overflow=ovf, pos_x=d["pos_x"], pos_w=d["pos_w"])
             t[l.name] = y
         elif l.kind == "maxpool":
             t[l.name] = maxpool_nhwc(t[l.src], l.k, l.stride, l.pad)
