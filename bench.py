@@ -226,15 +226,42 @@ def extras():
     import torch
     ops = torch.ops.torch_mlu
     out = {}
+    from catch_amd.pipeline import pos_from_scale
+
+    def gaussian_operands(m, n, k):
+        """X[m,k], W[n,k] ~ N(0,1) (seeds 2, 3), X per-tensor int8, W per-channel int8: the standalone linear config"""
+        x = torch.randn(m, k, generator=torch.Generator().manual_seed(2)).cuda()
+        w = torch.randn(n, k, generator=torch.Generator().manual_seed(3)).cuda()
+        pos_x = pos_from_scale(8, 127.0 / x.abs().max().item())
+        qx = ops.quantize(x, 8, pos_x, 1.0)
+        scales = (127.0 / w.abs().amax(1)).float()
+        qw, new_pos, new_scale = ops.quantize_per_channel(w, scales, 8)
+        return qx, qw, pos_x + int(new_pos.item()), new_scale
+
+    def time_gemm(a, b, exp2, div, bias, iters):
+        return event_time(lambda: ops.qlinear(a, b, exp2, div, bias, 1, True, True, False, 0, 0, 1.0), iters, max(iters // 10, 3))
+
     for (m, n, k) in ((4096, 3072, 768), (4096, 768, 3072)):
-        a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
-        b = torch.randint(-128, 128, (n, k), dtype=torch.int8, device="cuda")
-        bias = torch.randn(n, device="cuda")
-        div = torch.rand(n, device="cuda") + 0.5
-        t = event_time(lambda: ops.qlinear(a, b, -10, div, bias, 1, True, True, False, 0, 0, 1.0), 200, 20)
+        bias = torch.randn(n, generator=torch.Generator().manual_seed(4)).cuda()
+        a, b, exp2, div = gaussian_operands(m, n, k)
+        t = time_gemm(a, b, exp2, div, bias, 200)
         out["linear_%dx%dx%d" % (m, n, k)] = {"us": round(t * 1e6, 2), "tops": round(2 * m * n * k / t / 1e12, 1),
                                              "mfma_frac": round(2 * m * n * k / t / 1e12 / INT8_PEAK_TOPS, 4),
+                                             "operands": "N(0,1) quantized: X per tensor, W per channel",
                                              "epilogue": "per-channel dequant + bias + ReLU, fp16 out"}
+    # a GEMM large enough to be bound by the matrix cores, on two kinds of data: the rate depends on how many
+    # operand bits toggle (the chip lowers its clock under high-toggle matrix work)
+    m = n = k = 8192
+    bias = torch.randn(n, device="cuda")
+    a, b, exp2, div = gaussian_operands(m, n, k)
+    t_g = time_gemm(a, b, exp2, div, bias, 10)
+    a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
+    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, device="cuda")
+    t_u = time_gemm(a, b, -10, div, bias, 10)
+    out["gemm_8192x8192x8192"] = {"us_gaussian_operands": round(t_g * 1e6, 1), "tops_gaussian_operands": round(2 * m * n * k / t_g / 1e12, 1),
+                                  "us_uniform_operands": round(t_u * 1e6, 1), "tops_uniform_operands": round(2 * m * n * k / t_u / 1e12, 1),
+                                  "mfma_frac": round(2 * m * n * k / t_g / 1e12 / INT8_PEAK_TOPS, 4)}
+    del a, b
     n = 64 * 256 * 56 * 56  # one ResNet-50 stage-1 activation, 822 MB of fp32: larger than the 256 MB cache
     x = torch.randn(n, device="cuda")
     t = event_time(lambda: ops.quantize(x, 8, -5, 1.0), 20, 3)
