@@ -15,7 +15,7 @@ from .quantized.observer import (mlu_activation_observer_dict, mlu_weight_observ
                                  mlu_weight_per_channel_observer)
 from .quantized.qconfig import QConfig, custom_mlu_qconfig, default_mlu_qconfig
 
-_QUANT_TYPES = (nn.Linear, nn.Conv2d, "Conv2d")
+_QUANT_TYPES = (nn.Linear, nn.Conv3d, nn.Conv2d, nn.Conv1d, "Conv2d")
 
 
 def compose_qconfig(weight_observer, activation_observer):

@@ -532,6 +532,18 @@ void clear_cache_op() {
   g_rcp_cache.clear();
 }
 
+// quantized activations [N,H,W,Ci] x prepared weight -> floating [N,Ho,Wo,Co]
+Tensor conv_prepared(const Tensor &qx, const Prepared &prep, const Tensor &bias, at::IntArrayRef padding,
+                     at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups, bool half) {
+  Tensor qw = prep.qw.permute({0, 2, 3, 1});  // view of the same memory as [Co,kh,kw,Ci/g], contiguous
+  EpiArgs a;
+  a.exp2 = prep.pos_x + prep.pos_w;
+  if (prep.per_channel) a.chan_div = prep.new_scale;
+  if (has_bias(bias)) a.bias = bias;
+  a.y_half = half;
+  return qconv2d_impl(qx, qw, padding, stride, dilation, groups, a).y;
+}
+
 Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, at::IntArrayRef padding,
                  at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups, const Tensor &q_scale,
                  const Tensor &q_mode) {
@@ -544,14 +556,68 @@ Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
     return w.contiguous(at::MemoryFormat::ChannelsLast);
   });
   Tensor qx = quantize_to_nhwc(input, prep->bw_x, prep->pos_x, input.size(1));
-  Tensor qw = prep->qw.permute({0, 2, 3, 1});  // view of the same memory as [Co,kh,kw,Ci/g], contiguous
-  EpiArgs a;
-  a.exp2 = prep->pos_x + prep->pos_w;
-  if (prep->per_channel) a.chan_div = prep->new_scale;
-  if (has_bias(bias)) a.bias = bias;
-  a.y_half = half;
-  EpiOut o = qconv2d_impl(qx, qw, padding, stride, dilation, groups, a);
-  return o.y.permute({0, 3, 1, 2});  // logical NCHW over channels-last memory, like the reference
+  Tensor y = conv_prepared(qx, *prep, bias, padding, stride, dilation, groups, half);
+  return y.permute({0, 3, 1, 2});  // logical NCHW over channels-last memory, like the reference
+}
+
+// [N,C,L] x [Co,Ci/g,k]: a convolution over images of one row (the reference's module calls
+// torch.ops.torch_mlu.conv1d with the conv2d argument list: core/quantized/modules/conv.py:276-286)
+Tensor conv1d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, at::IntArrayRef padding,
+                 at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups, const Tensor &q_scale,
+                 const Tensor &q_mode) {
+  TORCH_CHECK(input.dim() == 3 && weight.dim() == 3, "torch_mlu::conv1d expects 3-d input and weight");
+  TORCH_CHECK(padding.size() == 1 && stride.size() == 1 && dilation.size() == 1, "1-d conv parameters expected");
+  const bool half = fp_dtype(input, "quantify only support input float/half") == CATCHQ_F16;
+  c10::DeviceGuard guard(input.device());
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w) {
+    return w.unsqueeze(2).contiguous(at::MemoryFormat::ChannelsLast);  // memory [Co][1][k][Ci/g]
+  });
+  Tensor qx = quantize_to_nhwc(input.unsqueeze(2), prep->bw_x, prep->pos_x, input.size(1));
+  Tensor y = conv_prepared(qx, *prep, bias, {0, padding[0]}, {1, stride[0]}, {1, dilation[0]}, groups, half);
+  return y.squeeze(1).permute({0, 2, 1});  // [N,Lo,Co] memory seen as [N,Co,Lo]
+}
+
+// [N,C,D,H,W] x [Co,Ci/g,kd,kh,kw].  The depth taps are folded into the channel dimension of a 2-d
+// convolution over the N*Do output depth slices: channel c*kd+t of slice (n, od) is input channel c at
+// depth od*sd - pd + t*dd.  Quantization is per element, so folding the quantized integers gives the
+// integers the 3-d convolution would read, and the int32 sums are the same.  With kd == 1 and depth
+// stride 1 the fold is a view (the reference's pseudo-conv3d case, internal/quantize_util.cpp:57-139;
+// module: core/quantized/modules/conv.py:345-354).
+Tensor conv3d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, at::IntArrayRef padding,
+                 at::IntArrayRef stride, at::IntArrayRef dilation, int64_t groups, const Tensor &q_scale,
+                 const Tensor &q_mode) {
+  TORCH_CHECK(input.dim() == 5 && weight.dim() == 5, "torch_mlu::conv3d expects 5-d input and weight");
+  TORCH_CHECK(padding.size() == 3 && stride.size() == 3 && dilation.size() == 3, "3-d conv parameters expected");
+  const bool half = fp_dtype(input, "quantify only support input float/half") == CATCHQ_F16;
+  c10::DeviceGuard guard(input.device());
+  const int64_t n = input.size(0), c = input.size(1), dd_in = input.size(2), h = input.size(3), w = input.size(4);
+  const int64_t kd = weight.size(2), pd = padding[0], sd = stride[0], dd = dilation[0];
+  TORCH_CHECK(sd > 0 && dd > 0 && pd >= 0, "depth stride/dilation must be positive, padding non-negative");
+  TORCH_CHECK(groups > 0 && c == weight.size(1) * groups, "channel mismatch: input ", c, ", weight ",
+              weight.size(1), " x groups ", groups);
+  const int64_t d_out = (dd_in + 2 * pd - dd * (kd - 1) - 1) / sd + 1;
+  TORCH_CHECK(dd_in + 2 * pd >= dd * (kd - 1) + 1 && d_out > 0, "Calculated output size is too small");
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &wt) {
+    // [Co, (Ci/g)*kd, kh, kw] with the depth tap fastest inside a channel, stored [Co][kh][kw][(Ci/g)*kd]
+    return wt.reshape({wt.size(0), wt.size(1) * wt.size(2), wt.size(3), wt.size(4)})
+        .contiguous(at::MemoryFormat::ChannelsLast);
+  });
+  // [N,C,D*H,W] -> integers in [N,D,H,W,C] order
+  Tensor q = quantize_to_nhwc(input.contiguous().view({n, c, dd_in * h, w}), prep->bw_x, prep->pos_x, c)
+                 .view({n, dd_in, h, w, c});
+  Tensor qx;
+  if (kd == 1 && sd == 1 && pd == 0) {
+    qx = q.view({n * dd_in, h, w, c});
+  } else {
+    if (pd > 0) q = at::constant_pad_nd(q, {0, 0, 0, 0, 0, 0, pd, pd}, 0);
+    std::vector<Tensor> taps;
+    for (int64_t t = 0; t < kd; ++t)
+      taps.push_back(q.slice(1, t * dd, t * dd + (d_out - 1) * sd + 1, sd));  // [N,Do,H,W,C]
+    qx = at::stack(taps, 5).view({n * d_out, h, w, c * kd});
+  }
+  Tensor y = conv_prepared(qx, *prep, bias, {padding[1], padding[2]}, {stride[1], stride[2]},
+                           {dilation[1], dilation[2]}, groups, half);
+  return y.view({n, d_out, y.size(1), y.size(2), y.size(3)}).permute({0, 4, 1, 2, 3});  // logical NCDHW
 }
 
 // cnnl_quantize_convolution_internal(input, input_position, weight, weight_position, bias, padding, stride,
@@ -662,6 +728,10 @@ std::string conv2d_route_op(int64_t x_bits, int64_t w_bits, at::IntArrayRef in_n
 TORCH_LIBRARY(torch_mlu, m) {
   m.def("conv2d(Tensor input, Tensor weight, Tensor bias, int[] padding, int[] stride, int[] dilation, "
         "int groups, Tensor q_scale, Tensor q_mode) -> Tensor");
+  m.def("conv1d(Tensor input, Tensor weight, Tensor bias, int[] padding, int[] stride, int[] dilation, "
+        "int groups, Tensor q_scale, Tensor q_mode) -> Tensor");
+  m.def("conv3d(Tensor input, Tensor weight, Tensor bias, int[] padding, int[] stride, int[] dilation, "
+        "int groups, Tensor q_scale, Tensor q_mode) -> Tensor");
   m.def("linear(Tensor input, Tensor weight, Tensor bias, Tensor q_scale, Tensor q_mode) -> Tensor");
   m.def("quantize(Tensor x, int bitwidth, int position, float scale=1.0) -> Tensor");
   m.def("quantize_dev(Tensor x, int bitwidth, Tensor position) -> Tensor");
@@ -690,6 +760,8 @@ TORCH_LIBRARY(torch_mlu, m) {
 
 TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA key
   m.impl("conv2d", &conv2d_op);
+  m.impl("conv1d", &conv1d_op);
+  m.impl("conv3d", &conv3d_op);
   m.impl("linear", &linear_op);
   m.impl("quantize", &quantize_op);
   m.impl("quantize_dev", &quantize_dev_op);

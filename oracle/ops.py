@@ -9,7 +9,7 @@ logical NCHW on input/output like the ops, NHWC inside.
 """
 import numpy as np
 
-from . import (conv2d_nhwc, epilogue, gemm_nt, per_channel_params, pos_from_scale, quantize,
+from . import (conv2d_nhwc, conv_out_size, epilogue, gemm_nt, per_channel_params, pos_from_scale, quantize,
                quantize_per_channel)
 
 
@@ -60,6 +60,48 @@ def conv2d(x, weight, bias, padding, stride, dilation, groups, q_scale, q_mode, 
     r = None if resid is None else np.ascontiguousarray(np.transpose(resid, (0, 2, 3, 1)))
     y = epilogue(acc, d["pos_x"] + d["pos_w"], d["new_scale"], b, r, act, out_dtype)
     d.update(qx=qx, qw=qw, acc=acc, overflow=ovf, y=np.transpose(y, (0, 3, 1, 2)))
+    return d
+
+
+def conv1d(x, weight, bias, padding, stride, dilation, groups, q_scale, q_mode):
+    """x [N,Ci,L], weight [Co,Ci/g,k]: the module of core/quantized/modules/conv.py:258-312 in the
+    reference; a 1-d convolution is the 2-d one over images with a single row.  -> y [N,Co,Lo]"""
+    x, weight = np.asarray(x), np.asarray(weight)
+    d = conv2d(x[:, :, None, :], weight[:, :, None, :], bias, (0, padding[0]), (1, stride[0]), (1, dilation[0]),
+               groups, q_scale, q_mode)
+    d["y"] = d["y"][:, :, 0, :]
+    return d
+
+
+def conv3d(x, weight, bias, padding, stride, dilation, groups, q_scale, q_mode):
+    """x [N,Ci,D,H,W], weight [Co,Ci/g,kd,kh,kw] (core/quantized/modules/conv.py:314-380 in the
+    reference).  A 3-d convolution is the sum over the kd depth taps of 2-d convolutions of input depth
+    slices with the tap's 2-d filters: the integer sums are added tap by tap, slices outside the
+    volume contribute nothing, and the result goes through the same epilogue.  -> y [N,Co,Do,Ho,Wo]"""
+    d = decode_qparams(q_scale, q_mode)
+    x = np.asarray(x)
+    out_dtype = np.float16 if x.dtype == np.float16 else np.float32
+    n, ci, dep, h, w = x.shape
+    co, _, kd, kh, kw = weight.shape
+    qx = quantize(np.ascontiguousarray(np.transpose(x, (0, 2, 3, 4, 1))), d["bw_x"], d["pos_x"])  # N D H W C
+    w_all = np.ascontiguousarray(np.transpose(np.asarray(weight, dtype=np.float32), (0, 2, 3, 4, 1)))  # O D H W I
+    qw = _quantize_weight(w_all.reshape(co, kd * kh, kw, -1), d).reshape(w_all.shape)
+    do = conv_out_size(dep, kd, padding[0], stride[0], dilation[0])
+    ho = conv_out_size(h, kh, padding[1], stride[1], dilation[1])
+    wo = conv_out_size(w, kw, padding[2], stride[2], dilation[2])
+    acc = np.zeros((n, do, ho, wo, co), np.int64)
+    for od in range(do):
+        for t in range(kd):
+            z = od * stride[0] - padding[0] + t * dilation[0]
+            if z < 0 or z >= dep:
+                continue
+            a, _ = conv2d_nhwc(np.ascontiguousarray(qx[:, z]), np.ascontiguousarray(qw[:, t]), tuple(padding[1:]),
+                               tuple(stride[1:]), tuple(dilation[1:]), groups)
+            acc[:, od] += a
+    ovf = int(((acc > 2 ** 31 - 1) | (acc < -2 ** 31)).sum())
+    b = None if bias is None else np.asarray(bias, dtype=np.float32)
+    y = epilogue(acc, d["pos_x"] + d["pos_w"], d["new_scale"], b, None, 0, out_dtype)
+    d.update(qx=qx, qw=qw, acc=acc, overflow=ovf, y=np.transpose(y, (0, 4, 1, 2, 3)))
     return d
 
 

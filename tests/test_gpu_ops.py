@@ -253,3 +253,80 @@ def test_quantize_conv2d_op_matches_conv2d_op():
     assert torch.equal(got, want)
     with pytest.raises(Exception):
         torch.ops.torch_mlu.quantize_conv2d(x, px.cpu(), w, pw, b, [1, 1], [1, 1], [1, 1], 1, 8, 8)
+
+
+@pytest.mark.parametrize("bw,per_channel,half", [("int8", False, False), ("int8", True, True), ("int16", True, False)])
+def test_conv1d_module_swap(bw, per_channel, half):
+    """nn.Conv1d -> MLUConv1d -> torch_mlu::conv1d (core/quantized/modules/conv.py:258-312 in the reference)"""
+    note("conv1d module", bw, per_channel, half)
+    torch.manual_seed(21)
+    model = nn.Sequential(nn.Conv1d(24, 40, 5, 2, 3, 2, 2, True)).eval().float()
+    x = torch.randn(3, 24, 77)
+    want_float = model(x).numpy()
+    ckpt = calibrate(model, x, bw, per_channel)
+    qmodel = quantize_dynamic_mlu(model)
+    qmodel.load_state_dict(ckpt)
+    conv = qmodel[0]
+    assert type(conv).__name__ == "MLUConv1d"
+    xin = x.half() if half else x
+    if half:
+        qmodel.half()
+    got = qmodel.to("cuda")(xin.to("cuda"))
+    assert got.shape == want_float.shape and got.dtype == xin.dtype
+    ref = oops.conv1d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
+                      (3,), (2,), (2,), 2, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
+    assert same_bits(ref["y"], got.cpu().numpy())
+    assert rel_rms(want_float, got.float().cpu().numpy()) <= 0.02
+
+
+CONV3D_CASES = [
+    # N, Ci, D, H, W, Co, k, pad, stride, dil, groups
+    (2, 16, 6, 12, 12, 32, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (1, 12, 7, 9, 10, 8, (2, 3, 1), (1, 0, 1), (2, 1, 2), (2, 1, 1), 2),
+    (2, 8, 5, 10, 10, 24, (1, 3, 3), (0, 1, 1), (1, 2, 2), (1, 1, 1), 1),   # depth folds into the batch (a view)
+    (2, 8, 5, 10, 10, 24, (1, 3, 3), (1, 1, 1), (2, 1, 1), (1, 1, 1), 1),   # kd == 1 with depth stride and padding
+    (1, 32, 4, 6, 6, 16, (3, 1, 1), (0, 0, 0), (1, 1, 1), (1, 1, 1), 1),    # kh == kw == 1
+]
+
+
+@pytest.mark.parametrize("case", CONV3D_CASES)
+@pytest.mark.parametrize("bw,half", [("int8", False), ("int16", False), ("int8", True)])
+def test_conv3d_module_swap(case, bw, half):
+    """nn.Conv3d -> MLUConv3d -> torch_mlu::conv3d (core/quantized/modules/conv.py:314-380 in the reference)"""
+    note("conv3d module", case, bw, half)
+    n, ci, d, h, w, co, k, pad, stride, dil, g = case
+    torch.manual_seed(co + d)
+    model = nn.Sequential(nn.Conv3d(ci, co, k, stride, pad, dil, g, True)).eval().float()
+    x = torch.randn(n, ci, d, h, w)
+    want_float = model(x).numpy()
+    ckpt = calibrate(model, x, bw, False)
+    qmodel = quantize_dynamic_mlu(model)
+    qmodel.load_state_dict(ckpt)
+    conv = qmodel[0]
+    assert type(conv).__name__ == "MLUConv3d"
+    xin = x.half() if half else x
+    if half:
+        qmodel.half()
+    got = qmodel.to("cuda")(xin.to("cuda"))
+    assert got.shape == want_float.shape and got.dtype == xin.dtype
+    ref = oops.conv3d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
+                      pad, stride, dil, g, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
+    assert same_bits(ref["y"], got.cpu().numpy())
+    assert rel_rms(want_float, got.float().cpu().numpy()) <= 0.02
+
+
+def test_conv3d_refuses_per_channel_calibration_and_bad_shapes():
+    note("conv3d errors")
+    model = nn.Sequential(nn.Conv3d(4, 4, 3)).eval()
+    qconfig = {"use_avg": False, "data_scale": 1.0, "per_channel": True, "firstconv": False}
+    with pytest.raises(AssertionError, match="per_channel"):
+        quantize_dynamic_mlu(model, qconfig, dtype="int8", gen_quant=True)
+    x = torch.randn(1, 4, 2, 5, 5).cuda()
+    w = torch.randn(4, 4, 3, 3, 3).cuda()
+    q_scale, q_mode = torch.tensor([30.0, 30.0]).cuda(), torch.tensor([1], dtype=torch.int32).cuda()
+    with pytest.raises(RuntimeError, match="Calculated output size is too small"):
+        torch.ops.torch_mlu.conv3d(x, w, torch.zeros(4).cuda(), [0, 0, 0], [1, 1, 1], [1, 1, 1], 1, q_scale, q_mode)
+    with pytest.raises(RuntimeError, match="expects 5-d"):
+        torch.ops.torch_mlu.conv3d(x[0], w, torch.zeros(4).cuda(), [0, 0, 0], [1, 1, 1], [1, 1, 1], 1, q_scale, q_mode)
+    with pytest.raises(RuntimeError, match="expects 3-d"):
+        torch.ops.torch_mlu.conv1d(x, w, torch.zeros(4).cuda(), [0], [1], [1], 1, q_scale, q_mode)

@@ -185,6 +185,31 @@ def test_state_dict_packing(bw, per_channel):
     assert torch.equal(q(x), model(x))  # CPU tensors: float path
 
 
+@pytest.mark.parametrize("nd", [1, 3])
+def test_conv1d_conv3d_modules_calibrate_and_pack(nd):
+    """nn.Conv1d / nn.Conv3d are swapped like nn.Conv2d (core/quantized/default_mappings.py:10-16 and
+    core/quantized/modules/conv.py:258-380 in the reference)"""
+    quantize_dynamic_mlu = _tool()
+    torch.manual_seed(nd)
+    conv = nn.Conv1d(4, 6, 3, 2, 1) if nd == 1 else nn.Conv3d(4, 6, (1, 3, 3), 1, (0, 1, 1))
+    model = nn.Sequential(conv).eval()
+    x = torch.randn(2, 4, 11) if nd == 1 else torch.randn(2, 4, 3, 6, 6)
+    calib = quantize_dynamic_mlu(model, {"per_channel": False, "firstconv": False}, dtype="int16", gen_quant=True)
+    assert type(calib[0]).__name__ == "MLUConv%dd" % nd
+    assert torch.equal(calib(x), model(x))
+    sd = calib.state_dict()
+    assert sd["0.scale"][0].item() == pytest.approx(32767.0 / x.abs().max().item(), rel=1e-6)
+    assert sd["0.scale"][1].item() == pytest.approx(32767.0 / conv.weight.abs().max().item(), rel=1e-6)
+    assert sd["0.quantized_mode"].tolist() == [2]
+    q = quantize_dynamic_mlu(model)
+    q.load_state_dict(sd)
+    assert q[0]._get_name() == "MLUConv%dd" % nd and q[0].scale.numel() == 2
+    assert torch.equal(q(x), model(x))  # CPU tensors: float path
+    if nd == 3:
+        with pytest.raises(AssertionError, match="per_channel"):
+            quantize_dynamic_mlu(model, {"per_channel": True, "firstconv": False}, dtype="int8", gen_quant=True)
+
+
 def test_first_conv_mean_std():
     quantize_dynamic_mlu = _tool()
     model = nn.Sequential(nn.Conv2d(3, 4, 3)).eval()

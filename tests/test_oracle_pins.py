@@ -355,3 +355,56 @@ def test_dequantized_float_conv_agrees():
     wd = orc.dequantize(np.transpose(r["qw"], (0, 3, 1, 2)), r["pos_w"]).astype(np.float64)
     want = F.conv2d(torch.from_numpy(xd), torch.from_numpy(wd), None, 1, 1).numpy()
     np.testing.assert_allclose(r["y"], want, rtol=1e-6, atol=1e-6)
+
+
+# ---------------------------------------------------------------- 1-d and 3-d convolutions
+@pytest.mark.parametrize("case", [
+    # N, Ci, L, Co, k, pad, stride, dil, groups
+    (2, 6, 33, 8, 3, 1, 1, 1, 1),
+    (3, 8, 40, 12, 5, 2, 2, 2, 4),
+    (1, 4, 9, 4, 1, 0, 1, 1, 1),
+])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_conv1d_dequantized_float_conv_agrees(case, per_channel):
+    """torch's float64 conv1d of the dequantized integers pins the oracle's 1-d composition"""
+    n, ci, length, co, k, pad, stride, dil, g = case
+    x = rng.standard_normal((n, ci, length)).astype(np.float32)
+    w = (rng.standard_normal((co, ci // g, k)) * 0.1).astype(np.float32)
+    q_scale, q_mode = _calibrate(x, w, 8, per_channel)
+    r = oops.conv1d(x, w, None, (pad,), (stride,), (dil,), g, q_scale, q_mode)
+    xq = torch.from_numpy(np.transpose(r["qx"][:, 0], (0, 2, 1)).astype(np.float64))
+    wq = torch.from_numpy(np.transpose(r["qw"][:, 0], (0, 2, 1)).astype(np.float64))
+    want_acc = F.conv1d(xq, wq, None, stride, pad, dil, g).numpy().astype(np.int64)
+    assert np.array_equal(want_acc, np.transpose(r["acc"][:, 0], (0, 2, 1)))
+    want = want_acc * 2.0 ** (r["pos_x"] + r["pos_w"])
+    if per_channel:
+        want = want / r["new_scale"].astype(np.float64)[None, :, None]
+    np.testing.assert_allclose(r["y"], want, rtol=1e-6, atol=1e-6)
+    assert _rel_rms(F.conv1d(torch.from_numpy(x), torch.from_numpy(w), None, stride, pad, dil, g).numpy(), r["y"]) <= 0.03
+
+
+@pytest.mark.parametrize("case", [
+    # N, Ci, D, H, W, Co, (kd,kh,kw), pad, stride, dil, groups
+    (2, 4, 6, 8, 8, 8, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (1, 6, 7, 9, 5, 4, (2, 3, 1), (1, 0, 1), (2, 1, 2), (2, 1, 1), 2),
+    (2, 3, 5, 6, 6, 5, (1, 3, 3), (0, 1, 1), (1, 2, 2), (1, 1, 1), 1),   # kd == 1: depth folds into the batch
+    (1, 8, 4, 5, 5, 8, (3, 1, 1), (0, 0, 0), (1, 1, 1), (1, 1, 1), 1),   # kh == kw == 1
+])
+@pytest.mark.parametrize("xbits", [8, 16])
+def test_conv3d_vs_torch_float64(case, xbits):
+    """the oracle's sum over depth taps against torch's float64 conv3d of the same integers"""
+    n, ci, d, h, w, co, k, pad, stride, dil, g = case
+    x = rng.standard_normal((n, ci, d, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((co, ci // g) + k) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(co).astype(np.float32)
+    q_scale, q_mode = _calibrate(x, wt, xbits, False)
+    r = oops.conv3d(x, wt, bias, pad, stride, dil, g, q_scale, q_mode)
+    assert r["qx"].dtype == (np.int8 if xbits == 8 else np.int16)
+    xq = torch.from_numpy(np.transpose(r["qx"], (0, 4, 1, 2, 3)).astype(np.float64))
+    wq = torch.from_numpy(np.transpose(r["qw"], (0, 4, 1, 2, 3)).astype(np.float64))
+    want_acc = F.conv3d(xq, wq, None, stride, pad, dil, g).numpy().astype(np.int64)
+    assert np.array_equal(want_acc, np.transpose(r["acc"], (0, 4, 1, 2, 3)))
+    want = want_acc * 2.0 ** (r["pos_x"] + r["pos_w"]) + bias.astype(np.float64)[None, :, None, None, None]
+    np.testing.assert_allclose(r["y"], want, rtol=1e-6, atol=1e-6)
+    ref = F.conv3d(torch.from_numpy(x), torch.from_numpy(wt), torch.from_numpy(bias), stride, pad, dil, g).numpy()
+    assert _rel_rms(ref, r["y"]) <= 0.03
