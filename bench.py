@@ -73,14 +73,30 @@ def layer_profile(fused, x, iters=20):
     fused.forward(x, trace=trace)  # materialise every layer's quantized input once
     torch.cuda.synchronize()
     for l in fused.layers:
-        if l.kind not in ("conv", "fc"):
+        if l.kind not in ("conv", "fc") or l.name in fused._fused_away:
             continue
         lq = fused.q[l.name]
         qx = trace[l.name].get("qx_dev", trace[l.name]["qx"])  # the tensor the kernel reads
         qd = fused.q_demand[l.name][0] if fused.q_demand[l.name] else None
         want_y = fused.f_demand[l.name] or qd is None
         y_half = fused.out_half and l.name in fused.outputs
-        if l.kind == "conv":
+        ds = fused.shortcut_of.get(l.name) if l.kind == "conv" else None
+        extra_macs = extra_bytes = 0
+        if ds is not None:  # the block's projection shortcut runs inside this launch
+            dq = fused.q[ds.name]
+            sx = trace[ds.name]["qx"]
+            resid = None
+            n_pix = trace[l.name]["y"].numel() // trace[l.name]["y"].shape[-1]
+            extra_macs = trace[l.name]["y"].numel() * dq.qw.shape[-1]
+            extra_bytes = n_pix * sx.shape[-1] * sx.element_size() + dq.qw.numel() * dq.qw.element_size()
+
+            def run(l=l, lq=lq, qx=qx, qd=qd, want_y=want_y, ds=ds, dq=dq, sx=sx):
+                return ops.qconv2d_shortcut(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, sx, dq.qw, ds.stride, dq.exp2,
+                                            dq.chan_div, dq.bias, fused.padding(l), [l.stride, l.stride], [1, 1],
+                                            {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}[l.act], want_y, y_half,
+                                            qd[0] if qd else 0, qd[1] if qd else 0, 1.0, 0.1, bool(l.add_after))
+            route = "mfma+sc"
+        elif l.kind == "conv":
             resid = torch.zeros_like(trace[l.name]["y"]) if l.add else None
 
             def run(l=l, lq=lq, qx=qx, qd=qd, want_y=want_y, resid=resid):
@@ -98,8 +114,8 @@ def layer_profile(fused, x, iters=20):
             route = "gemm"
         y = trace[l.name]["y"]
         n_out = y.numel()
-        macs = n_out * (lq.qw.numel() // lq.qw.shape[0])
-        bytes_alg = qx.numel() * qx.element_size() + lq.qw.numel() * lq.qw.element_size()
+        macs = n_out * (lq.qw.numel() // lq.qw.shape[0]) + extra_macs
+        bytes_alg = qx.numel() * qx.element_size() + lq.qw.numel() * lq.qw.element_size() + extra_bytes
         bytes_alg += ((2 if y_half else 4) * n_out if want_y else 0) + (n_out * (qd[0] // 8) if qd else 0) + (4 * n_out if resid is not None else 0)
         t = event_time(run, iters)
         rows.append(dict(name=l.name, route=route, t=t, ops=2 * macs, bytes=bytes_alg))
@@ -190,7 +206,7 @@ def main():
         print("sum of conv/fc launches: %.1f us repeated back to back, %.1f us in sequence; graph step: %.1f us" % (
             t_all * 1e6, sum(r["t_seq"] for r in rows) * 1e6, ms_per_step * 1e3), file=sys.stderr)
     roofline = {"bound": "hbm", "kernel": "%s (all %d launches of one step)" % (
-                    "igemm_a16_dma_kernel" if detector else "igemm_i8_dma_kernel", len(conv_rows)),
+                    "igemm_a16_dma_kernel" if detector else "igemm_i8_dma_kernel + igemm_i8_dual_kernel", len(conv_rows)),
                 "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, batch)),

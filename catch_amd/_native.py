@@ -31,6 +31,14 @@ class ConvDesc(ctypes.Structure):
                                             "stride_w", "dil_h", "dil_w", "groups")]
 
 
+class Shortcut(ctypes.Structure):
+    """struct catchq_shortcut"""
+    _fields_ = [("x", ctypes.c_void_p), ("w", ctypes.c_void_p), ("x_bits", ctypes.c_int), ("w_bits", ctypes.c_int),
+                ("in_h", ctypes.c_int), ("in_w", ctypes.c_int), ("ci", ctypes.c_int), ("stride", ctypes.c_int),
+                ("exp2", ctypes.c_int), ("chan_div", ctypes.c_void_p), ("chan_rcp", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p)]
+
+
 # name -> (restype, argtypes); every symbol include/catchq.h declares
 _I, _I64, _F, _P, _SZ = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 SIGNATURES = {
@@ -54,6 +62,10 @@ SIGNATURES = {
     "catchq_global_avgpool_nhwc": (_I, [_P, _P, _I, _I, _I, _P]),
     "catchq_quantize_conv2d_workspace_size": (_I, [ctypes.POINTER(ConvDesc), _I, _I, ctypes.POINTER(_SZ)]),
     "catchq_quantize_conv2d_nhwc": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, ctypes.POINTER(ConvDesc), _P, _P, _I, _P, _SZ, _P]),
+    "catchq_conv2d_shortcut_workspace_size": (_I, [_I, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Shortcut),
+                                                   ctypes.POINTER(_SZ)]),
+    "catchq_conv2d_shortcut_nhwc": (_I, [_P, _I, _P, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Epilogue),
+                                         ctypes.POINTER(Shortcut), _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
 }

@@ -16,6 +16,9 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
 int gemm_nt_mfma_a16(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
 int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
                     int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
+int conv2d_dual_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
+                   int sh, int sw, int dh, int dw, int Ho, int Wo, const void *xs, const void *ws, int Hs, int Ws, int Cs,
+                   int ss, const EpiDev &e, const ShortcutDev &sc, hipStream_t s);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -138,6 +141,86 @@ CATCHQ_API int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int 
       return conv2d_direct(x, x_bits, w, w_bits, cd, e, s);
     }
   }
+}
+
+// shapes the two-branch kernel serves (pointer alignment is checked at the call)
+static bool shortcut_fusable(int x_bits, int w_bits, const catchq_conv_desc_t *d, const catchq_shortcut_t *sc) {
+  return x_bits == 8 && w_bits == 8 && sc->x_bits == 8 && sc->w_bits == 8 && d->groups == 1 && d->ci % 16 == 0 &&
+         sc->ci % 16 == 0 && d->kh * d->kw <= 32 && d->co % 4 == 0 &&
+         (int64_t)d->n * d->h * d->w * d->ci < (1ll << 31) && (int64_t)d->co * d->kh * d->kw * d->ci < (1ll << 31) &&
+         (int64_t)d->n * sc->in_h * sc->in_w * sc->ci < (1ll << 31) && (int64_t)d->co * sc->ci < (1ll << 31);
+}
+
+static int check_shortcut(const catchq_conv_desc_t *d, const catchq_shortcut_t *sc, int ho, int wo) {
+  if (!sc) return CATCHQ_ERR_ARG;
+  if ((sc->x_bits != 8 && sc->x_bits != 16) || (sc->w_bits != 8 && sc->w_bits != 16)) return CATCHQ_ERR_BITWIDTH;
+  if (sc->in_h <= 0 || sc->in_w <= 0 || sc->ci <= 0 || sc->stride <= 0) return CATCHQ_ERR_SHAPE;
+  if (catchq_conv_out_size(sc->in_h, 1, 0, sc->stride, 1) != ho || catchq_conv_out_size(sc->in_w, 1, 0, sc->stride, 1) != wo)
+    return CATCHQ_ERR_SHAPE;
+  if (sc->exp2 < -126 || sc->exp2 > 126) return CATCHQ_ERR_ARG;
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_conv2d_shortcut_workspace_size(int x_bits, int w_bits, const catchq_conv_desc_t *desc,
+                                                     const catchq_shortcut_t *shortcut, size_t *bytes) {
+  int ho, wo;
+  int st = check_conv(desc, &ho, &wo);
+  if (st != CATCHQ_OK) return st;
+  if (!bytes) return CATCHQ_ERR_ARG;
+  if ((x_bits != 8 && x_bits != 16) || (w_bits != 8 && w_bits != 16)) return CATCHQ_ERR_BITWIDTH;
+  st = check_shortcut(desc, shortcut, ho, wo);
+  if (st != CATCHQ_OK) return st;
+  *bytes = shortcut_fusable(x_bits, w_bits, desc, shortcut) ? 0 : (size_t)desc->n * ho * wo * desc->co * 4;
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void *w, int w_bits,
+                                           const catchq_conv_desc_t *desc, const catchq_epilogue_t *epilogue,
+                                           const catchq_shortcut_t *shortcut, void *workspace, size_t workspace_bytes,
+                                           catchq_stream_t stream) {
+  int ho, wo;
+  int st = check_conv(desc, &ho, &wo);
+  if (st != CATCHQ_OK) return st;
+  if ((x_bits != 8 && x_bits != 16) || (w_bits != 8 && w_bits != 16)) return CATCHQ_ERR_BITWIDTH;
+  st = check_epi(epilogue);
+  if (st != CATCHQ_OK) return st;
+  st = check_shortcut(desc, shortcut, ho, wo);
+  if (st != CATCHQ_OK) return st;
+  if (epilogue->resid) return CATCHQ_ERR_ARG;  // the shortcut is the residual
+  if (desc->n == 0) return CATCHQ_OK;
+  if (!x || !w || !shortcut->x || !shortcut->w) return CATCHQ_ERR_ARG;
+  const catchq_conv_desc_t &d = *desc;
+  const catchq_shortcut_t &sc = *shortcut;
+  if (shortcut_fusable(x_bits, w_bits, desc, shortcut) && !epilogue->exp2_dev[0] && !epilogue->exp2_dev[1]) {
+    EpiDev e = make_epi(epilogue);
+    e.resid_after = epilogue->resid_after_act ? 1 : 0;
+    ShortcutDev sd;
+    sd.exp2 = sc.exp2;
+    sd.chan_div = sc.chan_div;
+    sd.chan_rcp = (sc.chan_div && sc.chan_rcp && sc.exp2 >= -64 && sc.exp2 <= 64) ? sc.chan_rcp : nullptr;
+    sd.bias = sc.bias;
+    const int st2 = conv2d_dual_i8(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h, d.stride_w,
+                                   d.dil_h, d.dil_w, ho, wo, sc.x, sc.w, sc.in_h, sc.in_w, sc.ci, sc.stride, e, sd,
+                                   as_stream(stream));
+    if (st2 >= 0) return st2;
+  }
+  // two launches: the shortcut's fp32 output goes through the workspace
+  const size_t need = (size_t)d.n * ho * wo * d.co * 4;
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return CATCHQ_ERR_ARG;
+  catchq_conv_desc_t ds = {d.n, sc.in_h, sc.in_w, sc.ci, d.co, 1, 1, 0, 0, sc.stride, sc.stride, 1, 1, 1};
+  catchq_epilogue_t es;
+  memset(&es, 0, sizeof(es));
+  es.exp2 = sc.exp2;
+  es.chan_div = sc.chan_div;
+  es.chan_rcp = sc.chan_rcp;
+  es.bias = sc.bias;
+  es.y = workspace;
+  es.y_dtype = CATCHQ_F32;
+  st = catchq_conv2d_nhwc(sc.x, sc.x_bits, sc.w, sc.w_bits, &ds, &es, stream);
+  if (st != CATCHQ_OK) return st;
+  catchq_epilogue_t em = *epilogue;
+  em.resid = (const float *)workspace;
+  return catchq_conv2d_nhwc(x, x_bits, w, w_bits, desc, &em, stream);
 }
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }

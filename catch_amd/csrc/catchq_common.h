@@ -96,6 +96,14 @@ struct EpiDev {
   const int *exp2_a, *exp2_b;  // device-resident positions added to exp2 (resolve_exp2)
 };
 
+// The second operand pair of a two-branch launch: the projection shortcut of a residual block.  Its
+// integer sums are dequantized (divisor or reciprocal form, bias) exactly like a launch of their own
+// with fp32 output would do, and the values serve as the residual of the main branch.
+struct ShortcutDev {
+  int exp2;
+  const float *chan_div, *chan_rcp, *bias;
+};
+
 inline EpiDev make_epi(const catchq_epilogue_t *e) {
   EpiDev d;
   d.exp2 = e->exp2;

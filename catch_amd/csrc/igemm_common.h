@@ -36,7 +36,8 @@ __device__ __forceinline__ int xcd_remap(int bid, int nb) {
 }
 
 inline bool vec_epilogue_ok(int N, const EpiDev &e) {
-  return N % 4 == 0 && aligned16(e.chan_div) && aligned16(e.chan_rcp) && aligned16(e.bias) && aligned16(e.resid) && aligned16(e.y) &&
+  // (N < 2^24: the per-lane part of an element index, at most 32 rows, fits 32 bits with room to spare)
+  return N % 4 == 0 && N < (1 << 24) && aligned16(e.chan_div) && aligned16(e.chan_rcp) && aligned16(e.bias) && aligned16(e.resid) && aligned16(e.y) &&
          aligned16(e.acc_out) && aligned16(e.q);
 }
 
@@ -134,20 +135,38 @@ __device__ __forceinline__ EpiLane epi_lane_setup(int n, bool n_ok, const EpiDev
   return L;
 }
 
-// four integer sums of one pixel (channels n..n+3, linear index idx) -> all requested outputs
-template <class S>
-__device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLane &L, int64_t idx, const EpiDev &e) {
-  if (S::acc(e)) *reinterpret_cast<v4i *>(e.acc_out + idx) = a;
+// dequantization and bias of one integer sum: channel t of the lane's four
+__device__ __forceinline__ float epi_dequant1(int a, int t, const EpiLane &L, int exp2) {
+  float x = (float)a;
+  if (L.use_rcp) x = div_by_rcp(x, L.div[t], L.rcp[t]);
+  else {
+    x = __builtin_ldexpf(x, exp2);
+    if (L.use_div) x = x / L.div[t];
+  }
+  if (L.use_bias) x = x + L.bias[t];
+  return x;
+}
+
+// Where an output element lives: a 64-bit element index, or a wave-uniform 64-bit part plus a 32-bit
+// per-lane part (then the uniform part stays in scalar registers and a store needs one vector add).
+struct EpiAt64 {
+  int64_t idx;
+  template <class T> __device__ __forceinline__ T *at(T *base) const { return base + idx; }
+};
+struct EpiAtSplit {
+  int64_t uni;   // same for every lane of the wave
+  unsigned off;  // this lane's part
+  template <class T> __device__ __forceinline__ T *at(T *base) const { return (base + uni) + off; }
+};
+
+// four integer sums of one pixel (channels n..n+3 at `where`) -> all requested outputs
+template <class S, class At>
+__device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLane &L, const At where, const EpiDev &e) {
+  if (S::acc(e)) *reinterpret_cast<v4i *>(where.at(e.acc_out)) = a;
   float v[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    float x = (float)a[t];
-    if (L.use_rcp) x = div_by_rcp(x, L.div[t], L.rcp[t]);
-    else {
-      x = __builtin_ldexpf(x, e.exp2);
-      if (L.use_div) x = x / L.div[t];
-    }
-    if (L.use_bias) x = x + L.bias[t];
+    float x = epi_dequant1(a[t], t, L, e.exp2);
     if (L.use_res && !L.res_after) x = x + res[t];
     if (L.act == CATCHQ_ACT_LEAKY) x = (x > 0.0f) ? x : x * e.act_slope;
     else if (L.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
@@ -158,10 +177,10 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
   if (S::y16(e)) {
     __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
                     __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
-    *reinterpret_cast<v2i *>(reinterpret_cast<__half *>(e.y) + idx) = *reinterpret_cast<v2i *>(h);
+    *reinterpret_cast<v2i *>(where.at(reinterpret_cast<__half *>(e.y))) = *reinterpret_cast<v2i *>(h);
   } else if (S::y32(e)) {
     v4f o = {v[0], v[1], v[2], v[3]};
-    *reinterpret_cast<v4f *>(reinterpret_cast<float *>(e.y) + idx) = o;
+    *reinterpret_cast<v4f *>(where.at(reinterpret_cast<float *>(e.y))) = o;
   }
   if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
     // values are >= 0 and never NaN here, the requantization scale is 1:
@@ -177,7 +196,7 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     }
     const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
     const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
-    *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = lo | hi2;
+    *reinterpret_cast<unsigned *>(where.at(reinterpret_cast<int8_t *>(e.q))) = lo | hi2;
   } else if (S::q8(e)) {
     int b[4];
     if (L.unit_q) {
@@ -190,7 +209,7 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     // four clamped values -> four bytes: two byte permutes and a merge
     const unsigned lo = __builtin_amdgcn_perm((unsigned)b[1], (unsigned)b[0], 0x0c0c0400u);
     const unsigned hi = __builtin_amdgcn_perm((unsigned)b[3], (unsigned)b[2], 0x04000c0cu);
-    *reinterpret_cast<unsigned *>(reinterpret_cast<int8_t *>(e.q) + idx) = lo | hi;
+    *reinterpret_cast<unsigned *>(where.at(reinterpret_cast<int8_t *>(e.q))) = lo | hi;
   } else if (S::q16(e)) {
     v2i pk;
     unsigned h[4];
@@ -199,8 +218,12 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
       h[t] = (unsigned)(L.unit_q ? quant1_unit<16>(v[t], e.q_neg_pos) : quant1<16>(v[t], e.q_scale, e.q_neg_pos)) & 0xffffu;
     pk[0] = (int)(h[0] | (h[1] << 16));
     pk[1] = (int)(h[2] | (h[3] << 16));
-    *reinterpret_cast<v2i *>(reinterpret_cast<int16_t *>(e.q) + idx) = pk;
+    *reinterpret_cast<v2i *>(where.at(reinterpret_cast<int16_t *>(e.q))) = pk;
   }
+}
+template <class S>
+__device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLane &L, int64_t idx, const EpiDev &e) {
+  epi_vec4<S, EpiAt64>(a, res, L, EpiAt64{idx}, e);
 }
 
 // this lane's four channels within a wave tile of TN*32 columns starting at n_w
@@ -208,7 +231,10 @@ template <int TN>
 __device__ __forceinline__ int epi_lane_channel(int n_w, int lane) { return n_w + (lane % (TN * 8)) * 4; }
 
 // Vector epilogue of one wave with the lane's per-channel constants supplied by the caller (kernels
-// that run many row groups against the same columns set them up once).
+// that run many row groups against the same columns set them up once).  m_w and n_w are the same for
+// every lane of the wave.  An element's index splits into the uniform (m_w + i*32) * N + n_w and a
+// 32-bit per-lane rest, and a wave whose tile lies wholly inside the matrix (the usual case) runs
+// without any per-lane bounds checks.
 template <int TM, int TN, int EPI>
 __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
                                                    const IgemmParams &p, const EpiDev &e, const EpiLane &L) {
@@ -218,40 +244,108 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
   const int frow = lane & 31, fhalf = lane >> 5;
   constexpr int CPR = WN / 4;    // 4-channel groups per staged row
   constexpr int RPI = 64 / CPR;  // rows the wave moves per iteration
+  constexpr int NIT = 32 / RPI;
+  const int cg = lane % CPR, rsub = lane / CPR;
+  const bool use_res = L.use_res;
+  const unsigned lane_off = (unsigned)rsub * (unsigned)p.N + (unsigned)(cg * 4);
+  const unsigned it_step = (unsigned)RPI * (unsigned)p.N;
+  auto tile = [&](auto full_c) {
+    constexpr bool FULL = decltype(full_c)::value;
+    const bool n_ok = FULL || (n_w + cg * 4 < p.N);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int64_t uni = (m_w + i * 32) * (int64_t)p.N + n_w;
+      const int64_t left = p.M - (m_w + i * 32);
+      const int rows = FULL ? 32 : (left < 0 ? 0 : (left > 32 ? 32 : (int)left));  // uniform
+      // residual rows of this 32-row block: all loads in flight before the staging below
+      v4f resv[NIT];
+      if (use_res) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
+          if (FULL || (n_ok && it * RPI + rsub < rows))
+            resv[it] = *reinterpret_cast<const v4f *>((e.resid + uni) + (lane_off + it * it_step));
+        }
+      }
+      // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
+      // all reads first: one LDS latency per 32 rows instead of one per iteration
+      v4i av[NIT];
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+        av[it] = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        if (!FULL && !(n_ok && it * RPI + rsub < rows)) continue;
+        epi_vec4<S>(av[it], use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, EpiAtSplit{uni, lane_off + it * it_step}, e);
+      }
+    }
+  };
+  // wave-uniform: the whole TM*32 x WN tile inside the matrix?
+  if (m_w + TM * 32 <= p.M && n_w + WN <= p.N) tile(std::true_type{});
+  else tile(std::false_type{});
+}
+
+// Vector epilogue of one wave whose residual comes from a second set of accumulators (same tile,
+// same layout) instead of memory: both sets go through the wave's staging area, the shortcut's first.
+template <int TM, int TN, int EPI>
+__device__ __forceinline__ void igemm_epilogue_dual(v16i (&acc)[TM][TN], v16i (&acc_sc)[TM][TN], int *stage, int64_t m_w,
+                                                    int n_w, int lane, const IgemmParams &p, const EpiDev &e,
+                                                    const ShortcutDev &sc) {
+  typedef typename EpiOf<EPI>::type S;
+  static_assert(EPI != EPI_SCALAR, "the two-branch epilogue is the vector one");
+  constexpr int WN = TN * 32;
+  constexpr int EPI_STRIDE = WN + 8;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  constexpr int CPR = WN / 4;
+  constexpr int RPI = 64 / CPR;
   const int cg = lane % CPR, rsub = lane / CPR;
   const int n = n_w + cg * 4;
   const bool n_ok = n < p.N;
-  const bool use_res = L.use_res;
+  EpiLane L = epi_lane_setup<S>(n, n_ok, e);
+  L.use_res = true;
+  L.res_after = e.resid_after != 0;
+  EpiDev e_sc = {};
+  e_sc.exp2 = sc.exp2; e_sc.chan_div = sc.chan_div; e_sc.chan_rcp = sc.chan_rcp; e_sc.bias = sc.bias;
+  const EpiLane L_sc = epi_lane_setup<EpiGeneric>(n, n_ok, e_sc);
+  const unsigned lane_off = (unsigned)rsub * (unsigned)p.N + (unsigned)(cg * 4);
+  const unsigned it_step = (unsigned)RPI * (unsigned)p.N;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    // residual rows of this 32-row block: all loads in flight before the staging below
-    v4f resv[32 / RPI];
-    if (use_res) {
+    // shortcut sums -> fp32 residual values in the row-major layout of the stores
 #pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it) {
-        const int64_t m = m_w + i * 32 + it * RPI + rsub;
-        resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
-        if (n_ok && m < p.M) resv[it] = *reinterpret_cast<const v4f *>(e.resid + m * p.N + n);
-      }
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc_sc[i][j][r];
+    v4f resv[32 / RPI];
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const v4i a = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) resv[it][t] = epi_dequant1(a[t], t, L_sc, sc.exp2);
     }
-    // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
+    // the wave's LDS operations complete in order: these stores cannot overtake the reads above
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
-    const int64_t mbase = m_w + i * 32;
-    // all reads first: one LDS latency per 32 rows instead of one per iteration
+    const int64_t uni = (m_w + i * 32) * (int64_t)p.N + n_w;
+    const int64_t left = p.M - (m_w + i * 32);
+    const int rows = left < 0 ? 0 : (left > 32 ? 32 : (int)left);
     v4i av[32 / RPI];
 #pragma unroll
     for (int it = 0; it < 32 / RPI; ++it)
       av[it] = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
 #pragma unroll
     for (int it = 0; it < 32 / RPI; ++it) {
-      const int64_t m = mbase + it * RPI + rsub;
-      if (!n_ok || m >= p.M) continue;
-      const int64_t idx = m * p.N + n;
-      epi_vec4<S>(av[it], use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, idx, e);
+      if (!n_ok || it * RPI + rsub >= rows) continue;
+      epi_vec4<S>(av[it], resv[it], L, EpiAtSplit{uni, lane_off + it * it_step}, e);
     }
   }
 }
@@ -292,5 +386,6 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
 // eligible (operand of 2 GiB or more, four-channel stem) and the caller takes the register-staged kernel
 int igemm_dma_launch(int load, const void *a, const void *b, IgemmParams p, const EpiDev &e, int64_t a_bytes,
                      int64_t b_bytes, hipStream_t s);
+
 
 }  // namespace catchq

@@ -304,6 +304,59 @@ EpiOut qconv2d_impl(const Tensor &qx, const Tensor &qw, at::IntArrayRef padding,
   return o;
 }
 
+// The last convolution of a residual block with the block's 1x1 projection shortcut (sx [N,Hs,Ws,Cs],
+// sw [Co,Cs] or [Co,1,1,Cs], stride s_stride, no padding) evaluated in the same launch; a.resid must be unset.
+EpiOut qconv2d_shortcut_impl(const Tensor &qx, const Tensor &qw, at::IntArrayRef padding, at::IntArrayRef stride,
+                             at::IntArrayRef dilation, const EpiArgs &a, const Tensor &sx, const Tensor &sw,
+                             int64_t s_stride, int64_t s_exp2, const c10::optional<Tensor> &s_chan_div,
+                             const c10::optional<Tensor> &s_bias) {
+  TORCH_CHECK(qx.dim() == 4 && qw.dim() == 4 && qx.is_contiguous() && qw.is_contiguous(),
+              "qconv2d expects contiguous NHWC activations and [Co,kh,kw,Ci/g] weights");
+  TORCH_CHECK(sx.dim() == 4 && sx.is_contiguous() && sw.is_contiguous() && sw.numel() == qw.size(0) * sx.size(3) &&
+                  sx.size(0) == qx.size(0),
+              "shortcut: expected NHWC activations of the same batch and a [Co,Ci] filter");
+  TORCH_CHECK(padding.size() == 2 && stride.size() == 2 && dilation.size() == 2, "2-d conv parameters expected");
+  TORCH_CHECK(qx.size(3) == qw.size(3), "channel mismatch: input ", qx.size(3), ", weight ", qw.size(3));
+  TORCH_CHECK(!(a.resid.has_value() && a.resid->defined()), "the shortcut is the residual: resid must not be given");
+  catchq_conv_desc_t d;
+  d.n = (int)qx.size(0); d.h = (int)qx.size(1); d.w = (int)qx.size(2); d.ci = (int)qx.size(3);
+  d.co = (int)qw.size(0); d.kh = (int)qw.size(1); d.kw = (int)qw.size(2);
+  d.pad_h = (int)padding[0]; d.pad_w = (int)padding[1];
+  d.stride_h = (int)stride[0]; d.stride_w = (int)stride[1];
+  d.dil_h = (int)dilation[0]; d.dil_w = (int)dilation[1];
+  d.groups = 1;
+  const int ho = catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h);
+  const int wo = catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w);
+  TORCH_CHECK(ho > 0 && wo > 0, "Calculated output size is too small");
+  catchq_epilogue_t e;
+  std::vector<Tensor> keep;
+  EpiOut o = prepare_epilogue(a, {d.n, ho, wo, d.co}, d.co, qx.options(), &e, &keep);
+  catchq_shortcut_t sc;
+  std::memset(&sc, 0, sizeof(sc));
+  sc.x = sx.data_ptr(); sc.w = sw.data_ptr();
+  sc.x_bits = bits_of(sx); sc.w_bits = bits_of(sw);
+  sc.in_h = (int)sx.size(1); sc.in_w = (int)sx.size(2); sc.ci = (int)sx.size(3);
+  sc.stride = (int)s_stride;
+  TORCH_CHECK(s_exp2 >= -126 && s_exp2 <= 126, "position sum out of range");
+  sc.exp2 = (int)s_exp2;
+  Tensor cd = as_f32_vec(s_chan_div, d.co, "shortcut chan_div"), bs = as_f32_vec(s_bias, d.co, "shortcut bias");
+  if (cd.defined()) {
+    sc.chan_div = cd.data_ptr<float>();
+    keep.push_back(cd);
+    Tensor rcp = reciprocals_for(cd);
+    if (rcp.defined()) { sc.chan_rcp = rcp.data_ptr<float>(); keep.push_back(rcp); }
+  }
+  if (bs.defined()) { sc.bias = bs.data_ptr<float>(); keep.push_back(bs); }
+  size_t ws_bytes = 0;
+  check_status(catchq_conv2d_shortcut_workspace_size(bits_of(qx), bits_of(qw), &d, &sc, &ws_bytes),
+               "torch_mlu::qconv2d_shortcut");
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, qx.options().dtype(at::kChar));
+  check_status(catchq_conv2d_shortcut_nhwc(qx.data_ptr(), bits_of(qx), qw.data_ptr(), bits_of(qw), &d, &e, &sc,
+                                           ws.data_ptr(), ws_bytes, current_stream()),
+               "torch_mlu::qconv2d_shortcut");
+  return o;
+}
+
 EpiOut qlinear_impl(const Tensor &qx, const Tensor &qw, const EpiArgs &a) {
   TORCH_CHECK(qx.dim() == 2 && qw.dim() == 2 && qx.is_contiguous() && qw.is_contiguous(), "dimension not support");
   TORCH_CHECK(qx.size(1) == qw.size(1), "size mismatch: ", qx.sizes(), " x ", qw.sizes(), "^T");
@@ -342,6 +395,22 @@ std::tuple<Tensor, Tensor, Tensor> qconv2d_op(const Tensor &qx, const Tensor &qw
   return tup(qconv2d_impl(qx, qw, padding, stride, dilation, groups,
                           make_args(exp2, chan_div, bias, resid, act, want_y, y_half, want_acc, q_bitwidth,
                                     q_position, q_scale, act_slope, resid_after_act)));
+}
+
+std::tuple<Tensor, Tensor> qconv2d_shortcut_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
+                                               const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias,
+                                               const Tensor &sx, const Tensor &sw, int64_t s_stride, int64_t s_exp2,
+                                               const c10::optional<Tensor> &s_chan_div,
+                                               const c10::optional<Tensor> &s_bias, at::IntArrayRef padding,
+                                               at::IntArrayRef stride, at::IntArrayRef dilation, int64_t act, bool want_y,
+                                               bool y_half, int64_t q_bitwidth, int64_t q_position, double q_scale,
+                                               double act_slope, bool resid_after_act) {
+  c10::DeviceGuard guard(qx.device());
+  EpiOut o = qconv2d_shortcut_impl(qx, qw, padding, stride, dilation,
+                                   make_args(exp2, chan_div, bias, c10::nullopt, act, want_y, y_half, false, q_bitwidth,
+                                             q_position, q_scale, act_slope, resid_after_act),
+                                   sx, sw, s_stride, s_exp2, s_chan_div, s_bias);
+  return std::make_tuple(o.y, o.q);
 }
 
 std::tuple<Tensor, Tensor, Tensor> qlinear_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
@@ -746,6 +815,10 @@ TORCH_LIBRARY(torch_mlu, m) {
         "int[] padding, int[] stride, int[] dilation, int groups, int act=0, bool want_y=True, "
         "bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
         "float act_slope=0.0, bool resid_after_act=False) -> (Tensor, Tensor, Tensor)");
+  m.def("qconv2d_shortcut(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, Tensor sx, Tensor sw, "
+        "int s_stride, int s_exp2, Tensor? s_chan_div, Tensor? s_bias, int[] padding, int[] stride, int[] dilation, "
+        "int act=0, bool want_y=True, bool y_half=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
+        "float act_slope=0.0, bool resid_after_act=False) -> (Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
         "bool want_y=True, bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, "
         "float q_scale=1.0) -> (Tensor, Tensor, Tensor)");
@@ -773,6 +846,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("mm_q", &mm_q_op);
   m.impl("quantize_conv2d", &quantize_conv2d_op);
   m.impl("qconv2d", &qconv2d_op);
+  m.impl("qconv2d_shortcut", &qconv2d_shortcut_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);
   m.impl("global_avgpool_nhwc", &global_avgpool_nhwc_op);

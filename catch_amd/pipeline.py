@@ -115,7 +115,7 @@ def _decode(layer, sd, device, ci_dev, co_dev):
 
 
 class FusedNet(object):
-    def __init__(self, layers, state_dict, device="cuda", out_half=False):
+    def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True):
         self.layers = list(layers)
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
@@ -153,6 +153,25 @@ class FusedNet(object):
             if extra:
                 lq.qw = torch.nn.functional.pad(lq.qw, (0, 0, 0, extra)).contiguous()  # [Co,kh,kw+extra,C]
             self.stem = dict(name=l0.name, pad=l0.pad, extra=extra)
+        # Projection shortcuts (1x1 convolution, no activation, consumed only as the residual of one
+        # convolution): evaluated inside that convolution's launch, their fp32 output is never stored.
+        # shortcut_of: main layer name -> shortcut layer; a traced pass runs them as launches of their own.
+        self.shortcut_of = {}
+        if fuse_shortcuts:
+            by_name = {l.name: l for l in self.layers}
+            for l in self.layers:
+                ds = by_name.get(l.add) if l.kind == "conv" and l.add else None
+                if ds is None or ds.kind != "conv" or l.groups != 1:
+                    continue
+                readers = [m for m in self.layers
+                           if m.src == ds.name or (isinstance(m.src, tuple) and ds.name in m.src) or m.add == ds.name]
+                lq, dq = self.q[l.name], self.q[ds.name]
+                if (ds.k == 1 and ds.pad == 0 and ds.groups == 1 and ds.act == "none" and not ds.add
+                        and readers == [l] and ds.name not in self.outputs and not self.q_demand[ds.name]
+                        and (lq.bw_x, lq.bw_w, dq.bw_x, dq.bw_w) == (8, 8, 8, 8)
+                        and not (self.stem and self.stem["name"] in (l.name, ds.name))):
+                    self.shortcut_of[l.name] = ds
+        self._fused_away = set(ds.name for ds in self.shortcut_of.values())
 
     def padding(self, layer):
         """padding the layer's convolution call gets (the stem's lives in its input frame)"""
@@ -217,18 +236,31 @@ class FusedNet(object):
                 env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"])
         for l in self.layers:
             name = l.name
+            if l.kind == "conv" and not tracing and name in self._fused_away:
+                continue
             if l.kind == "conv":
                 lq = self.q[name]
                 qx = env[(l.src, lq.bw_x, lq.pos_x)]
-                resid = env[(l.add, "f")] if l.add else None
                 qd = self.q_demand[name][0] if self.q_demand[name] else None
                 want_y = self.f_demand[name] or tracing or qd is None
+                ds = None if tracing else self.shortcut_of.get(name)
                 tick(name)
-                y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, self.padding(l),
-                                        [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
-                                        self.out_half and name in self.outputs, tracing,
-                                        qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
-                                        bool(l.add_after))
+                if ds is not None:
+                    dq = self.q[ds.name]
+                    y, q = ops.qconv2d_shortcut(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias,
+                                                env[(ds.src, dq.bw_x, dq.pos_x)], dq.qw, ds.stride, dq.exp2,
+                                                dq.chan_div, dq.bias, self.padding(l), [l.stride, l.stride], [1, 1],
+                                                _ACT_CODE[l.act], want_y, self.out_half and name in self.outputs,
+                                                qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
+                                                bool(l.add_after))
+                    acc = None
+                else:
+                    resid = env[(l.add, "f")] if l.add else None
+                    y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, self.padding(l),
+                                            [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
+                                            self.out_half and name in self.outputs, tracing,
+                                            qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
+                                            bool(l.add_after))
                 tick(name)
                 if want_y:
                     env[(name, "f")] = y

@@ -190,6 +190,36 @@ int catchq_quantize_conv2d_nhwc(const void *x, int x_dtype, const int32_t *x_pos
                                 const catchq_conv_desc_t *desc, const float *bias, void *y, int y_dtype,
                                 void *workspace, size_t workspace_bytes, catchq_stream_t stream);
 
+/* Last convolution of a residual block with the block's projection shortcut evaluated in the same launch.
+ * In the reference a block with a projection ends in two torch_mlu::conv2d calls (cnnl_conv2d,
+ * operators/cnnl/quantify_conv_forward.cpp:56-147: the 1x1 shortcut and the block's last convolution) and a
+ * float add (cnnl_add, operators/cnnl/add.cpp), i.e. the shortcut's fp32 output is written and read back.  Here
+ *   s[r][c] = float(acc_s[r][c]) * 2^shortcut.exp2 [/ shortcut.chan_div[c]] [+ shortcut.bias[c]]
+ * (acc_s = the 1x1 convolution of shortcut.x [n, in_h, in_w, ci] with shortcut.w [co, ci], stride `stride`
+ * in both directions, no padding; its output grid must equal the main convolution's) takes the place of
+ * resid[r][c] in the epilogue above; epilogue->resid must be NULL.  s is computed by the same operations, in
+ * the same order, as a catchq_conv2d_nhwc call of its own with fp32 output would store.
+ * The workspace is only used when no fused kernel serves the shapes (then the shortcut runs as a launch of its
+ * own into it): catchq_conv2d_shortcut_workspace_size returns 0 for int8 x int8 operands on both branches with
+ * ci % 16 == 0 on both, groups == 1, at most 32 filter taps and co % 4 == 0 (all pointers 16-byte aligned, no
+ * exp2_dev, no acc_out), and rows * co * 4 bytes otherwise. */
+typedef struct catchq_shortcut {
+  const void *x;         /* device [n, in_h, in_w, ci], x_bits wide */
+  const void *w;         /* device [co, ci], w_bits wide */
+  int x_bits, w_bits;
+  int in_h, in_w, ci;    /* n and co are the main convolution's */
+  int stride;
+  int exp2;
+  const float *chan_div; /* device [co] or NULL */
+  const float *chan_rcp; /* device [co] or NULL, as in catchq_epilogue_t */
+  const float *bias;     /* device [co] or NULL */
+} catchq_shortcut_t;
+int catchq_conv2d_shortcut_workspace_size(int x_bits, int w_bits, const catchq_conv_desc_t *desc,
+                                          const catchq_shortcut_t *shortcut, size_t *bytes);
+int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void *w, int w_bits, const catchq_conv_desc_t *desc,
+                                const catchq_epilogue_t *epilogue, const catchq_shortcut_t *shortcut, void *workspace,
+                                size_t workspace_bytes, catchq_stream_t stream);
+
 /* ------------------------------------------------------------------ neighbours of the convolutions */
 
 /* Max pooling over an NHWC tensor whose elements are int8, int16 (quantized activations) or fp32

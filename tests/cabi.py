@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 from catch_amd import _native
-from catch_amd._native import ConvDesc, Epilogue, check
+from catch_amd._native import ConvDesc, Epilogue, Shortcut, check
 
 F32, F16 = 0, 1
 _INT = {8: torch.int8, 16: torch.int16, 31: torch.int32, 32: torch.int32}
@@ -130,6 +130,26 @@ def conv2d_nhwc(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1, 
     check(lib().catchq_conv2d_nhwc(ptr(x), x.element_size() * 8, ptr(w), w.element_size() * 8, ctypes.byref(d),
                                    ctypes.byref(e), stream()))
     return out
+
+
+def conv2d_shortcut_nhwc(x, w, sx, sw, sc_stride, sc_exp2, sc_chan_div=None, sc_bias=None, sc_chan_rcp=None, padding=(0, 0),
+                         stride=(1, 1), dilation=(1, 1), exp2=0, chan_div=None, bias=None, act=0, y_dtype=torch.float32,
+                         q_bw=0, q_pos=0, q_scale=1.0, chan_rcp=None, act_slope=0.0, resid_after_act=False):
+    """-> (outputs, workspace bytes the library asked for)"""
+    d = conv_desc(x.shape, w.shape, padding, stride, dilation, 1)
+    ho = lib().catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h)
+    wo = lib().catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w)
+    e, out = _epilogue((d.n, ho, wo, d.co), x.device, exp2, chan_div, bias, None, act, y_dtype, False, q_bw, q_pos,
+                       q_scale, chan_rcp, act_slope, resid_after_act)
+    sc = Shortcut(ptr(sx), ptr(sw), sx.element_size() * 8, sw.element_size() * 8, sx.shape[1], sx.shape[2], sx.shape[3],
+                  sc_stride, sc_exp2, ptr(sc_chan_div), ptr(sc_chan_rcp), ptr(sc_bias))
+    need = ctypes.c_size_t()
+    check(lib().catchq_conv2d_shortcut_workspace_size(x.element_size() * 8, w.element_size() * 8, ctypes.byref(d),
+                                                      ctypes.byref(sc), ctypes.byref(need)))
+    ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=x.device)
+    check(lib().catchq_conv2d_shortcut_nhwc(ptr(x), x.element_size() * 8, ptr(w), w.element_size() * 8, ctypes.byref(d),
+                                            ctypes.byref(e), ctypes.byref(sc), ptr(ws), need.value, stream()))
+    return out, need.value
 
 
 def quantize_conv2d(x, pos_x, w, pos_w, x_bits=8, w_bits=8, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1,

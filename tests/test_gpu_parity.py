@@ -394,6 +394,65 @@ def test_quantize_conv2d_device_positions(bits, case):
     assert same_bits(want, got.cpu().numpy())
 
 
+SHORTCUT_CASES = [
+    # N, H, W, Ci, Co, k, pad, stride (main conv);  Hs, Ws, Cs, shortcut stride;  x bits, expected workspace use
+    (2, 14, 14, 64, 256, 1, 0, 1, 14, 14, 64, 1, 8, False),     # first block of a bottleneck stage: both 1x1 s1
+    (2, 7, 7, 128, 512, 1, 0, 1, 14, 14, 256, 2, 8, False),     # later stages: shortcut reads every other pixel
+    (3, 9, 11, 32, 64, 3, 1, 1, 9, 11, 16, 1, 8, False),        # basic block: 3x3 main convolution, ragged extents
+    (1, 16, 16, 64, 128, 3, 1, 2, 16, 16, 48, 2, 8, False),     # main convolution strided as well
+    (2, 40, 40, 256, 1024, 1, 0, 1, 80, 80, 512, 2, 8, False),  # long K on both branches, many tiles
+    (2, 20, 21, 64, 128, 1, 0, 1, 20, 21, 64, 1, 8, False),     # short K, Co >= 128: 64x128 tiles
+    (2, 6, 6, 32, 36, 1, 0, 1, 6, 6, 16, 1, 8, False),          # Co % 32 != 0
+    (2, 6, 6, 24, 32, 1, 0, 1, 6, 6, 16, 1, 8, True),           # Ci % 16 != 0: two launches through the workspace
+    (2, 6, 6, 32, 30, 1, 0, 1, 6, 6, 16, 1, 8, True),           # Co % 4 != 0
+    (1, 8, 8, 32, 32, 3, 1, 1, 8, 8, 16, 1, 16, True),          # int16 activations
+]
+
+
+@pytest.mark.parametrize("case", SHORTCUT_CASES)
+def test_conv_with_projection_shortcut(case):
+    """catchq_conv2d_shortcut_nhwc against the oracle's two convolutions in sequence: shortcut (dequant + bias,
+    fp32) -> main convolution with that tensor as its residual, ReLU, fp32 and requantized outputs."""
+    n, h, w, ci, co, k, pad, stride, hs, ws_, cs, ss, xbits, uses_ws = case
+    note("conv_shortcut", case)
+    r = rng(sum(case[:12]))
+    x, wt = _ints(r, (n, h, w, ci), xbits), _ints(r, (co, k, k, ci), 8)
+    sx, sw = _ints(r, (n, hs, ws_, cs), xbits), _ints(r, (co, 1, 1, cs), 8)
+    acc, ovf = orc.conv2d_nhwc(x, wt, (pad, pad), (stride, stride), (1, 1), 1)
+    acc_s, ovf_s = orc.conv2d_nhwc(sx, sw, (0, 0), (ss, ss), (1, 1), 1)
+    assert ovf == 0 and ovf_s == 0 and acc.shape == acc_s.shape
+    div, div_s = r.uniform(0.6, 3.5, co).astype(np.float32), r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias, bias_s = r.standard_normal(co).astype(np.float32), r.standard_normal(co).astype(np.float32)
+    e_main, e_sc = (-10, -12) if xbits == 8 else (-18, -20)
+    y_s = orc.epilogue(acc_s, e_sc, div_s, bias_s, None, 0)
+    xd, wd, sxd, swd = cabi.dev(x), cabi.dev(wt), cabi.dev(sx), cabi.dev(sw)
+    for act, after, with_rcp in ((1, False, True), (1, False, False), (3, True, True), (0, False, True)):
+        out, ws_bytes = cabi.conv2d_shortcut_nhwc(
+            xd, wd, sxd, swd, ss, e_sc, cabi.dev(div_s), cabi.dev(bias_s), cabi.dev(np.float32(1) / div_s) if with_rcp else None,
+            (pad, pad), (stride, stride), (1, 1), exp2=e_main, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=act,
+            q_bw=8, q_pos=-3, chan_rcp=cabi.dev(np.float32(1) / div) if with_rcp else None, act_slope=0.1,
+            resid_after_act=after)
+        assert (ws_bytes > 0) == uses_ws
+        y = orc.epilogue(acc, e_main, div, bias, y_s, act, act_slope=0.1, resid_after_act=after)
+        assert same_bits(y, out["y"].cpu().numpy()), (act, after, with_rcp)
+        assert same_bits(orc.quantize(y, 8, -3), out["q"].cpu().numpy()), (act, after, with_rcp)
+    # no divisors, no biases, fp16 output only
+    out, _ = cabi.conv2d_shortcut_nhwc(xd, wd, sxd, swd, ss, e_sc, padding=(pad, pad), stride=(stride, stride),
+                                       exp2=e_main, act=2, y_dtype=torch.float16)
+    y = orc.epilogue(acc, e_main, None, None, orc.epilogue(acc_s, e_sc, None, None, None, 0), 2, np.float16)
+    assert same_bits(y, out["y"].cpu().numpy())
+
+
+def test_conv_shortcut_argument_checks():
+    note("conv_shortcut errors")
+    x = torch.zeros((1, 8, 8, 16), dtype=torch.int8, device="cuda")
+    w = torch.zeros((16, 1, 1, 16), dtype=torch.int8, device="cuda")
+    with pytest.raises(Exception):  # shortcut grid 4x4 != main grid 8x8
+        cabi.conv2d_shortcut_nhwc(x, w, x, w, 2, 0)
+    with pytest.raises(Exception):  # non-positive stride
+        cabi.conv2d_shortcut_nhwc(x, w, x, w, 0, 0)
+
+
 def test_quantize_into_frame():
     """NCHW float -> NHWC int8/int16 inside a zero frame equals the plain transposing quantizer placed by hand."""
     note("quantize frame")

@@ -94,6 +94,29 @@ def test_resnet50_small_batch_and_graph_replay():
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("depth,expect", [(18, ["l2.0.c2", "l3.0.c2", "l4.0.c2"]),
+                                          (50, ["l1.0.c3", "l2.0.c3", "l3.0.c3", "l4.0.c3"])])
+def test_projection_shortcuts_fused_into_block_end(depth, expect):
+    """the projection shortcuts run inside the launch of the block's last convolution; logits identical to
+    the plan that runs them as launches of their own (which the traced pass checks against the oracle)"""
+    note("shortcut fusion, resnet", depth)
+    layers = nets.resnet(depth)
+    net = nets.FloatNet(layers, seed=3).eval()
+    x = torch.randn(3, 3, 96, 96, generator=torch.Generator().manual_seed(4))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd)
+    plain = pipeline.FusedNet(layers, sd, fuse_shortcuts=False)
+    assert sorted(fused.shortcut_of) == expect and not plain.shortcut_of
+    assert sorted(l.name for l in fused.shortcut_of.values()) == [e.rsplit(".", 1)[0] + ".ds" for e in expect]
+    timers = {}
+    a = fused.forward(x.cuda(), timers=timers)
+    b = plain.forward(x.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert not any(n.endswith(".ds") for n in timers)  # no launch of their own
+    check_against_oracle(layers, sd, x, fused)
+
+
 def test_mobilenet_v2_small():
     """MobileNetV2: depthwise stencil kernel, ReLU6, linear bottlenecks with residual adds, channel
     counts (24, 144) that the device layout pads to multiples of 16."""
