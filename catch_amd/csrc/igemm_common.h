@@ -234,8 +234,9 @@ __device__ __forceinline__ int epi_lane_channel(int n_w, int lane) { return n_w 
 // that run many row groups against the same columns set them up once).  m_w and n_w are the same for
 // every lane of the wave.  An element's index splits into the uniform (m_w + i*32) * N + n_w and a
 // 32-bit per-lane rest, and a wave whose tile lies wholly inside the matrix (the usual case) runs
-// without any per-lane bounds checks.
-template <int TM, int TN, int EPI>
+// without any per-lane bounds checks (FAST_PATH = false leaves that copy of the code out: kernels that
+// unroll the epilogue several times over cannot afford the registers its free scheduling takes).
+template <int TM, int TN, int EPI, bool FAST_PATH = true>
 __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
                                                    const IgemmParams &p, const EpiDev &e, const EpiLane &L) {
   typedef typename EpiOf<EPI>::type S;
@@ -247,7 +248,7 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
   constexpr int NIT = 32 / RPI;
   const int cg = lane % CPR, rsub = lane / CPR;
   const bool use_res = L.use_res;
-  const unsigned lane_off = (unsigned)rsub * (unsigned)p.N + (unsigned)(cg * 4);
+  const unsigned lane_off0 = (unsigned)rsub * (unsigned)p.N + (unsigned)(cg * 4);
   const unsigned it_step = (unsigned)RPI * (unsigned)p.N;
   auto tile = [&](auto full_c) {
     constexpr bool FULL = decltype(full_c)::value;
@@ -257,6 +258,10 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
       const int64_t uni = (m_w + i * 32) * (int64_t)p.N + n_w;
       const int64_t left = p.M - (m_w + i * 32);
       const int rows = FULL ? 32 : (left < 0 ? 0 : (left > 32 ? 32 : (int)left));  // uniform
+      // Opaque copy: a kernel that calls this in a loop would otherwise keep every iteration's byte
+      // offsets (loop invariants) in registers across the whole loop; recomputing them costs one add each.
+      unsigned lane_off = lane_off0;
+      asm volatile("" : "+v"(lane_off));
       // residual rows of this 32-row block: all loads in flight before the staging below
       v4f resv[NIT];
       if (use_res) {
@@ -286,7 +291,7 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
     }
   };
   // wave-uniform: the whole TM*32 x WN tile inside the matrix?
-  if (m_w + TM * 32 <= p.M && n_w + WN <= p.N) tile(std::true_type{});
+  if (FAST_PATH && m_w + TM * 32 <= p.M && n_w + WN <= p.N) tile(std::true_type{});
   else tile(std::false_type{});
 }
 

@@ -15,6 +15,7 @@ namespace catchq {
 
 constexpr int PW_MAX_KS = 3;  // K <= 96; supported (K steps, N fragments) pairs: KS * NF <= 6
 constexpr int PW_DEPTH = 3;   // row groups whose loads are in flight per wave
+constexpr bool PW_FAST = false;  // the check-free copy of the epilogue costs occupancy here and gains nothing (measured)
 
 // widest power-of-two run of 32-column fragments the epilogue handles in one go
 constexpr int pw_part(int nf) { return nf >= 4 ? 4 : nf >= 2 ? 2 : 1; }
@@ -25,15 +26,15 @@ __device__ __forceinline__ void pw_epilogue(v16i (&acc)[1][NF], int *stage, int6
                                             const EpiDev &e, const EpiLane &l_head, const EpiLane &l_tail) {
   constexpr int P = pw_part(NF);
   if constexpr (P == NF) {
-    igemm_epilogue_vec<1, NF, EPI>(acc, stage, m, 0, lane, p, e, l_head);
+    igemm_epilogue_vec<1, NF, EPI, PW_FAST>(acc, stage, m, 0, lane, p, e, l_head);
   } else {
     v16i head[1][P], tail[1][NF - P];
 #pragma unroll
     for (int j = 0; j < P; ++j) head[0][j] = acc[0][j];
 #pragma unroll
     for (int j = P; j < NF; ++j) tail[0][j - P] = acc[0][j];
-    igemm_epilogue_vec<1, P, EPI>(head, stage, m, 0, lane, p, e, l_head);
-    igemm_epilogue_vec<1, NF - P, EPI>(tail, stage, m, P * 32, lane, p, e, l_tail);
+    igemm_epilogue_vec<1, P, EPI, PW_FAST>(head, stage, m, 0, lane, p, e, l_head);
+    igemm_epilogue_vec<1, NF - P, EPI, PW_FAST>(tail, stage, m, P * 32, lane, p, e, l_tail);
   }
 }
 
