@@ -265,8 +265,18 @@ static int launch_a16(const void *a, const void *b, IgemmParams p, const EpiDev 
   const int64_t nb = tiles_m * p.tiles_n;
   if (nb > 0x7fffffff) return CATCHQ_ERR_SHAPE;
   p.nblocks = (int)nb;
-  if (pick_epilogue(p.N, e) == EPI_SCALAR)
+  const int epi = pick_epilogue(p.N, e);
+  if (epi == EPI_SCALAR)
     return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_SCALAR>(a, b, p, e, a_bytes, b_bytes, s);
+  if constexpr (BM == 64 && BN == 64) {  // the tile of every detector layer: leaky ReLU, int16 requantization
+    switch (epi) {
+      case EPI_LK_Q16: return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_LK_Q16>(a, b, p, e, a_bytes, b_bytes, s);
+      case EPI_LK_Y_Q16: return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_LK_Y_Q16>(a, b, p, e, a_bytes, b_bytes, s);
+      case EPI_LK_RESA_Q16: return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_LK_RESA_Q16>(a, b, p, e, a_bytes, b_bytes, s);
+      case EPI_LK_RESA_Y_Q16: return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_LK_RESA_Y_Q16>(a, b, p, e, a_bytes, b_bytes, s);
+      default: break;
+    }
+  }
   return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_VECTOR>(a, b, p, e, a_bytes, b_bytes, s);
 }
 

@@ -77,7 +77,18 @@ enum {
   EPI_RES_Y = 5,    // ... + residual + ReLU -> fp32                                   (last block)
   EPI_Y16_RELU = 6, // reciprocal-form dequant + bias + ReLU -> fp16                  (standalone linear)
   EPI_Q8_RELU6 = 7, // reciprocal-form dequant + bias + ReLU6 -> int8
-  EPI_COUNT = 8
+  EPI_RES_Q8 = 8,   // ... + residual + ReLU -> int8 only                             (last block of a stage)
+  // linear bottlenecks (no activation), reciprocal-form dequant + bias:
+  EPI_LIN_Q8 = 9,          // -> int8
+  EPI_LIN_Y_Q8 = 10,       // -> fp32 and int8
+  EPI_LIN_RES_Q8 = 11,     // + residual -> int8
+  EPI_LIN_RES_Y_Q8 = 12,   // + residual -> fp32 and int8
+  // per-tensor weights (no divisor), bias, leaky ReLU, int16 requantization:
+  EPI_LK_Q16 = 13,         // -> int16
+  EPI_LK_Y_Q16 = 14,       // -> fp32 and int16
+  EPI_LK_RESA_Q16 = 15,    // residual added after the activation -> int16
+  EPI_LK_RESA_Y_Q16 = 16,  // residual added after the activation -> fp32 and int16
+  EPI_COUNT = 17
 };
 template <int EPI> struct EpiOf { typedef EpiGeneric type; };
 template <> struct EpiOf<EPI_Q8_RELU> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_RELU, 0, 8, 0> type; };
@@ -86,21 +97,36 @@ template <> struct EpiOf<EPI_Y32> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_NONE, 1,
 template <> struct EpiOf<EPI_RES_Y> { typedef EpiSpec<1, 1, 1, CATCHQ_ACT_RELU, 1, 0, 0> type; };
 template <> struct EpiOf<EPI_Y16_RELU> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_RELU, 2, 0, 0> type; };
 template <> struct EpiOf<EPI_Q8_RELU6> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_RELU6, 0, 8, 0> type; };
+template <> struct EpiOf<EPI_RES_Q8> { typedef EpiSpec<1, 1, 1, CATCHQ_ACT_RELU, 0, 8, 0> type; };
+template <> struct EpiOf<EPI_LIN_Q8> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_NONE, 0, 8, 0> type; };
+template <> struct EpiOf<EPI_LIN_Y_Q8> { typedef EpiSpec<1, 1, 0, CATCHQ_ACT_NONE, 1, 8, 0> type; };
+template <> struct EpiOf<EPI_LIN_RES_Q8> { typedef EpiSpec<1, 1, 1, CATCHQ_ACT_NONE, 0, 8, 0> type; };
+template <> struct EpiOf<EPI_LIN_RES_Y_Q8> { typedef EpiSpec<1, 1, 1, CATCHQ_ACT_NONE, 1, 8, 0> type; };
+template <> struct EpiOf<EPI_LK_Q16> { typedef EpiSpec<0, 1, 0, CATCHQ_ACT_LEAKY, 0, 16, 0> type; };
+template <> struct EpiOf<EPI_LK_Y_Q16> { typedef EpiSpec<0, 1, 0, CATCHQ_ACT_LEAKY, 1, 16, 0> type; };
+template <> struct EpiOf<EPI_LK_RESA_Q16> { typedef EpiSpec<0, 1, 2, CATCHQ_ACT_LEAKY, 0, 16, 0> type; };
+template <> struct EpiOf<EPI_LK_RESA_Y_Q16> { typedef EpiSpec<0, 1, 2, CATCHQ_ACT_LEAKY, 1, 16, 0> type; };
 
-// which variant serves this launch (the specialised ones also need a unit requantization scale)
+// which variant serves this launch (the specialised ones also need a unit requantization scale);
+// a kernel family that has no instance of the variant returned uses the generic EPI_VECTOR
 inline int pick_epilogue(int N, const EpiDev &e) {
   if (!vec_epilogue_ok(N, e)) return EPI_SCALAR;
-  const bool rcp = e.chan_rcp != nullptr, bias = e.bias != nullptr, resid = e.resid != nullptr;
+  if (e.acc_out || (e.q && e.q_scale != 1.0f) || (e.chan_div && !e.chan_rcp)) return EPI_VECTOR;
+  const int div = e.chan_rcp ? 1 : 0, bias = e.bias ? 1 : 0;
+  const int res = !e.resid ? 0 : (e.resid_after ? 2 : 1);
   const int ym = !e.y ? 0 : (e.y_f16 ? 2 : 1);
   const int qm = !e.q ? 0 : e.q_bw;
-  if (!rcp || !bias || e.acc_out || (qm && e.q_scale != 1.0f) || e.resid_after || e.act == CATCHQ_ACT_LEAKY)
-    return EPI_VECTOR;
-  if (!resid && e.act == CATCHQ_ACT_RELU && ym == 0 && qm == 8) return EPI_Q8_RELU;
-  if (resid && e.act == CATCHQ_ACT_RELU && ym == 1 && qm == 8) return EPI_RES_Y_Q8;
-  if (!resid && e.act == CATCHQ_ACT_NONE && ym == 1 && qm == 0) return EPI_Y32;
-  if (resid && e.act == CATCHQ_ACT_RELU && ym == 1 && qm == 0) return EPI_RES_Y;
-  if (!resid && e.act == CATCHQ_ACT_RELU && ym == 2 && qm == 0) return EPI_Y16_RELU;
-  if (!resid && e.act == CATCHQ_ACT_RELU6 && ym == 0 && qm == 8) return EPI_Q8_RELU6;
+  static const struct { int epi, div, bias, res, act, ym, qm; } rows[] = {
+      {EPI_Q8_RELU, 1, 1, 0, CATCHQ_ACT_RELU, 0, 8},        {EPI_RES_Y_Q8, 1, 1, 1, CATCHQ_ACT_RELU, 1, 8},
+      {EPI_Y32, 1, 1, 0, CATCHQ_ACT_NONE, 1, 0},            {EPI_RES_Y, 1, 1, 1, CATCHQ_ACT_RELU, 1, 0},
+      {EPI_Y16_RELU, 1, 1, 0, CATCHQ_ACT_RELU, 2, 0},       {EPI_Q8_RELU6, 1, 1, 0, CATCHQ_ACT_RELU6, 0, 8},
+      {EPI_RES_Q8, 1, 1, 1, CATCHQ_ACT_RELU, 0, 8},         {EPI_LIN_Q8, 1, 1, 0, CATCHQ_ACT_NONE, 0, 8},
+      {EPI_LIN_Y_Q8, 1, 1, 0, CATCHQ_ACT_NONE, 1, 8},       {EPI_LIN_RES_Q8, 1, 1, 1, CATCHQ_ACT_NONE, 0, 8},
+      {EPI_LIN_RES_Y_Q8, 1, 1, 1, CATCHQ_ACT_NONE, 1, 8},   {EPI_LK_Q16, 0, 1, 0, CATCHQ_ACT_LEAKY, 0, 16},
+      {EPI_LK_Y_Q16, 0, 1, 0, CATCHQ_ACT_LEAKY, 1, 16},     {EPI_LK_RESA_Q16, 0, 1, 2, CATCHQ_ACT_LEAKY, 0, 16},
+      {EPI_LK_RESA_Y_Q16, 0, 1, 2, CATCHQ_ACT_LEAKY, 1, 16}};
+  for (const auto &r : rows)
+    if (r.div == div && r.bias == bias && r.res == res && r.act == e.act && r.ym == ym && r.qm == qm) return r.epi;
   return EPI_VECTOR;
 }
 

@@ -135,6 +135,8 @@ static int pw_pick_epi(const void *a, const void *b, const IgemmParams &p, const
     case EPI_SCALAR: return -1;
     case EPI_Q8_RELU6: return pw_launch<KS, NF, EPI_Q8_RELU6>(a, b, p, e, s);
     case EPI_Q8_RELU: return pw_launch<KS, NF, EPI_Q8_RELU>(a, b, p, e, s);
+    case EPI_LIN_Q8: return pw_launch<KS, NF, EPI_LIN_Q8>(a, b, p, e, s);
+    case EPI_LIN_Y_Q8: return pw_launch<KS, NF, EPI_LIN_Y_Q8>(a, b, p, e, s);
     default: return pw_launch<KS, NF, EPI_VECTOR>(a, b, p, e, s);
   }
 }

@@ -394,6 +394,55 @@ def test_quantize_conv2d_device_positions(bits, case):
     assert same_bits(want, got.cpu().numpy())
 
 
+# (per-channel divisor with reciprocals, residual: 0 none / 1 before / 2 after the activation, activation, fp output, q bits):
+# one row per specialised epilogue instance of the kernels (these skip the run-time branches of the generic one)
+EPILOGUE_ROWS = [
+    (True, 0, 1, None, 8), (True, 1, 1, torch.float32, 8), (True, 0, 0, torch.float32, 0), (True, 1, 1, torch.float32, 0),
+    (True, 0, 1, torch.float16, 0), (True, 0, 2, None, 8), (True, 1, 1, None, 8), (True, 0, 0, None, 8),
+    (True, 0, 0, torch.float32, 8), (True, 1, 0, None, 8), (True, 1, 0, torch.float32, 8), (False, 0, 3, None, 16),
+    (False, 0, 3, torch.float32, 16), (False, 2, 3, None, 16), (False, 2, 3, torch.float32, 16),
+]
+EPILOGUE_SHAPES = [
+    # N, Ci, H, W, Co, k, pad, x bits
+    (2, 128, 10, 10, 64, 1, 0, 8),     # LDS-ring kernel, 64x64 tiles
+    (1, 64, 24, 24, 256, 1, 0, 8),     # 64x128 tiles when a residual is added
+    (1, 32, 70, 70, 16, 1, 0, 8),      # streaming pointwise kernel
+    (1, 32, 12, 12, 64, 3, 1, 16),     # int16 activations
+    (1, 16, 20, 20, 16, 3, 1, 8),      # depthwise (groups = 16)
+]
+
+
+@pytest.mark.parametrize("shape", EPILOGUE_SHAPES)
+def test_specialised_epilogues(shape):
+    n, ci, h, w, co, k, pad, xbits = shape
+    g = ci if (k == 3 and ci == co == 16) else 1
+    note("specialised epilogues", shape)
+    r = rng(sum(shape))
+    x, wt = _ints(r, (n, h, w, ci), xbits), _ints(r, (co, k, k, ci // g), 8)
+    acc, ovf = orc.conv2d_nhwc(x, wt, (pad, pad), (1, 1), (1, 1), g)
+    assert ovf == 0
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = r.standard_normal(co).astype(np.float32)
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    xd, wd = cabi.dev(x), cabi.dev(wt)
+    exp2 = -10 if xbits == 8 else -18
+    for per_channel, res_mode, act, y_dtype, q_bw in EPILOGUE_ROWS:
+        out = cabi.conv2d_nhwc(xd, wd, (pad, pad), (1, 1), (1, 1), g, exp2=exp2,
+                               chan_div=cabi.dev(div) if per_channel else None, bias=cabi.dev(bias),
+                               resid=cabi.dev(resid) if res_mode else None, act=act, y_dtype=y_dtype, want_acc=False,
+                               q_bw=q_bw, q_pos=-3 if q_bw == 8 else -10,
+                               chan_rcp=cabi.dev(np.float32(1) / div) if per_channel else None, act_slope=0.1,
+                               resid_after_act=res_mode == 2)
+        y = orc.epilogue(acc, exp2, div if per_channel else None, bias, resid if res_mode else None, act,
+                         act_slope=0.1, resid_after_act=res_mode == 2)
+        row = (per_channel, res_mode, act, y_dtype, q_bw)
+        if y_dtype is not None:
+            want = y.astype(np.float16) if y_dtype == torch.float16 else y
+            assert same_bits(want, out["y"].cpu().numpy()), row
+        if q_bw:
+            assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10), out["q"].cpu().numpy()), row
+
+
 SHORTCUT_CASES = [
     # N, H, W, Ci, Co, k, pad, stride (main conv);  Hs, Ws, Cs, shortcut stride;  x bits, expected workspace use
     (2, 14, 14, 64, 256, 1, 0, 1, 14, 14, 64, 1, 8, False),     # first block of a bottleneck stage: both 1x1 s1
