@@ -27,7 +27,7 @@ INT8_PEAK_TOPS = 5000.0
 # HBM bytes moved by the igemm launches of one ResNet-50 bs64 step, from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy in the same runs):
 # 2.326e9 read + 2.166e9 written.  Valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = {("resnet50", 64): 4.493e9}
+MEASURED_TRAFFIC_BYTES = {("resnet50", 64): 3.606e9}
 
 
 def parse():
