@@ -416,8 +416,12 @@ static int conv2d_stem_a16(const void *x, const void *w, int N, int H, int W, in
   const int ngrp = (p.N + 31) / 32;
   int blocks = (int)((ngroups + 3) / 4);
   if (blocks > 256 * 4 / ngrp) blocks = 256 * 4 / ngrp;
-  stem_a16_kernel<3, EPI_VECTOR><<<dim3(blocks, ngrp), 256, LDS_BYTES, s>>>((const int16_t *)x, (const int8_t *)w, p, e,
-                                                                           (int)ngroups);
+  if (pick_epilogue(p.N, e) == EPI_LK_Q16)  // a detector's first layer: leaky ReLU, int16 out
+    stem_a16_kernel<3, EPI_LK_Q16><<<dim3(blocks, ngrp), 256, LDS_BYTES, s>>>((const int16_t *)x, (const int8_t *)w, p, e,
+                                                                             (int)ngroups);
+  else
+    stem_a16_kernel<3, EPI_VECTOR><<<dim3(blocks, ngrp), 256, LDS_BYTES, s>>>((const int16_t *)x, (const int8_t *)w, p, e,
+                                                                             (int)ngroups);
   return launch_status();
 }
 
