@@ -486,6 +486,7 @@ struct Prepared {
   const void *w_ptr = nullptr;
   int bw_x = 8, bw_w = 8, pos_x = 0, pos_w = 0;
   bool per_channel = false;
+  int variant = 0;   // caller's layout choice for qw (part of the cache key)
   Tensor qw;         // conv: [Co,kh,kw,Ci/g]; linear: [N,K]
   Tensor new_scale;  // device fp32 [Co] when per_channel
   Prepared() : w_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)),
@@ -521,14 +522,25 @@ c10::weak_intrusive_ptr<c10::TensorImpl> weak_of(const Tensor &t) {
   return c10::weak_intrusive_ptr<c10::TensorImpl>(t.getIntrusivePtr());
 }
 
-// Decode the two q-param encodings and quantize the weight (dense, dim 0 slowest).
-std::shared_ptr<Prepared> prepare(const Tensor &w_dense, const Tensor &weight, const Tensor &q_scale,
+// Decode the two q-param encodings and quantize the weight (make_dense(weight, activation bit width)
+// returns it dense, dim 0 slowest, in the layout the caller's kernel wants).
+template <typename MakeDense>
+std::shared_ptr<Prepared> prepare(MakeDense make_dense, const Tensor &weight, const Tensor &q_scale,
                                   const Tensor &q_mode) {
   auto p = std::make_shared<Prepared>();
   Tensor s_host = q_scale.to(at::kCPU).to(at::kFloat).contiguous();
   Tensor m_host = q_mode.to(at::kCPU).to(at::kInt).contiguous();
   const float *s = s_host.data_ptr<float>();
   const int32_t *m = m_host.data_ptr<int32_t>();
+  int bw_act = 8;
+  if (m_host.numel() == 1) {
+    TORCH_CHECK(m[0] >= 1 && m[0] <= 4, "quantized_mode must be 1, 2, 3 or 4, got ", m[0]);
+    bw_act = (m[0] == 1 || m[0] == 3) ? 8 : 16;
+  } else {
+    TORCH_CHECK(m_host.numel() == 2 && s_host.numel() == 2, "q_scale/q_mode must hold two values each");
+    bw_act = (int)s[0];
+  }
+  const Tensor w_dense = make_dense(weight, bw_act);
   if (m_host.numel() == 1) {
     // CNML-compatible encoding: q_mode in {1:int8, 2:int16, 3:int8 per-channel, 4:int16 per-channel},
     // q_scale = [s_in, s_w | 0, s_c0 ...]   (quantify_conv_forward.cpp:77-131; linear.cpp:81-144)
@@ -569,18 +581,19 @@ std::shared_ptr<Prepared> prepare(const Tensor &w_dense, const Tensor &weight, c
 
 template <typename MakeDense>
 std::shared_ptr<Prepared> prepared_for(const Tensor &weight, const Tensor &q_scale, const Tensor &q_mode,
-                                       MakeDense make_dense) {
+                                       MakeDense make_dense, int variant = 0) {
   const bool use_cache = cache_enabled();
   const c10::TensorImpl *key = weight.unsafeGetTensorImpl();
   if (use_cache) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
     if (it != g_cache.end()) {
-      if (still_valid(*it->second, weight, q_scale, q_mode)) return it->second;
+      if (it->second->variant == variant && still_valid(*it->second, weight, q_scale, q_mode)) return it->second;
       g_cache.erase(it);
     }
   }
-  auto p = prepare(make_dense(weight), weight, q_scale, q_mode);
+  auto p = prepare(make_dense, weight, q_scale, q_mode);
+  p->variant = variant;
   if (use_cache) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     if (g_cache.size() > 4096) {  // drop entries whose weight is gone
@@ -620,12 +633,40 @@ Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   TORCH_CHECK(input.dim() == 4 && weight.dim() == 4, "torch_mlu::conv2d expects 4-d input and weight");
   const bool half = fp_dtype(input, "quantify only support input float/half") == CATCHQ_F16;
   c10::DeviceGuard guard(input.device());
-  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w) {
+  // An image of fewer than four channels (grey, RGB): the int8 path quantizes it into a zero frame that
+  // holds the convolution's padding, with a fourth all-zero channel, and pads the filter rows to whole
+  // groups of four taps -- the shape of the streaming first-layer kernel (int16 activations take eight
+  // channels and stay unframed).  Everything added is zeros on one side of every product.
+  const int64_t ci = input.size(1), kw = weight.size(3);
+  const bool few = groups == 1 && ci < 4 && weight.size(1) == ci;
+  const int64_t kw_extra = (kw + 3) / 4 * 4 - kw;
+  const bool can_frame = few && dilation.size() == 2 && dilation[1] == 1 && padding.size() == 2;
+  auto prep = prepared_for(weight, q_scale, q_mode, [&](const Tensor &w, int bw_act) {
+    Tensor wd = w;
+    if (few) {
+      const int64_t cpad = (bw_act == 8 ? 4 : 8) - ci;
+      const int64_t taps = (bw_act == 8 && can_frame) ? kw_extra : 0;
+      wd = at::constant_pad_nd(w, {0, taps, 0, 0, 0, cpad}, 0);
+    }
     // the memory of a channels-last [Co,Ci/g,kh,kw] tensor is [Co][kh][kw][Ci/g]
-    return w.contiguous(at::MemoryFormat::ChannelsLast);
-  });
-  Tensor qx = quantize_to_nhwc(input, prep->bw_x, prep->pos_x, input.size(1));
-  Tensor y = conv_prepared(qx, *prep, bias, padding, stride, dilation, groups, half);
+    return wd.contiguous(at::MemoryFormat::ChannelsLast);
+  }, (few ? 1 : 0) | (can_frame ? 2 : 0));
+  Tensor qx;
+  std::vector<int64_t> pad(padding.begin(), padding.end());
+  if (few && prep->bw_x == 8 && can_frame) {
+    const Tensor xc = input.contiguous();
+    const int64_t h = input.size(2), w_in = input.size(3);
+    qx = at::empty({input.size(0), h + 2 * pad[0], w_in + 2 * pad[1] + kw_extra, 4}, input.options().dtype(at::kChar));
+    check_status(catchq_quantize_nchw_to_nhwc_frame(xc.data_ptr(), half ? CATCHQ_F16 : CATCHQ_F32, qx.data_ptr(), 8,
+                                                    (int)input.size(0), (int)ci, (int)h, (int)w_in, 4, (int)qx.size(1),
+                                                    (int)qx.size(2), (int)pad[0], (int)pad[1], prep->pos_x, 1.0f,
+                                                    current_stream()),
+                 "torch_mlu::quantize");
+    pad = {0, 0};
+  } else {
+    qx = quantize_to_nhwc(input, prep->bw_x, prep->pos_x, few ? (prep->bw_x == 8 ? 4 : 8) : ci);
+  }
+  Tensor y = conv_prepared(qx, *prep, bias, pad, stride, dilation, groups, half);
   return y.permute({0, 3, 1, 2});  // logical NCHW over channels-last memory, like the reference
 }
 
@@ -638,7 +679,7 @@ Tensor conv1d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   TORCH_CHECK(padding.size() == 1 && stride.size() == 1 && dilation.size() == 1, "1-d conv parameters expected");
   const bool half = fp_dtype(input, "quantify only support input float/half") == CATCHQ_F16;
   c10::DeviceGuard guard(input.device());
-  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w) {
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w, int) {
     return w.unsqueeze(2).contiguous(at::MemoryFormat::ChannelsLast);  // memory [Co][1][k][Ci/g]
   });
   Tensor qx = quantize_to_nhwc(input.unsqueeze(2), prep->bw_x, prep->pos_x, input.size(1));
@@ -666,7 +707,7 @@ Tensor conv3d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
               weight.size(1), " x groups ", groups);
   const int64_t d_out = (dd_in + 2 * pd - dd * (kd - 1) - 1) / sd + 1;
   TORCH_CHECK(dd_in + 2 * pd >= dd * (kd - 1) + 1 && d_out > 0, "Calculated output size is too small");
-  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &wt) {
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &wt, int) {
     // [Co, (Ci/g)*kd, kh, kw] with the depth tap fastest inside a channel, stored [Co][kh][kw][(Ci/g)*kd]
     return wt.reshape({wt.size(0), wt.size(1) * wt.size(2), wt.size(3), wt.size(4)})
         .contiguous(at::MemoryFormat::ChannelsLast);
@@ -738,7 +779,7 @@ Tensor linear_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   TORCH_CHECK(input.dim() >= 1 && input.size(-1) == weight.size(1), "size mismatch: input ", input.sizes(),
               ", weight ", weight.sizes());
   c10::DeviceGuard guard(input.device());
-  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w) { return w.contiguous(); });
+  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w, int) { return w.contiguous(); });
   Tensor x2 = input.contiguous().view({-1, input.size(-1)});
   Tensor qx = quantize_op(x2, prep->bw_x, prep->pos_x, 1.0);
   EpiArgs a;  // output is fp32 whatever the input type (operators/cnnl/matmul.cpp:72-74)

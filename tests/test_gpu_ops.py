@@ -330,3 +330,36 @@ def test_conv3d_refuses_per_channel_calibration_and_bad_shapes():
         torch.ops.torch_mlu.conv3d(x[0], w, torch.zeros(4).cuda(), [0, 0, 0], [1, 1, 1], [1, 1, 1], 1, q_scale, q_mode)
     with pytest.raises(RuntimeError, match="expects 3-d"):
         torch.ops.torch_mlu.conv1d(x, w, torch.zeros(4).cuda(), [0], [1], [1], 1, q_scale, q_mode)
+
+
+@pytest.mark.parametrize("ci,k,pad,stride,dil,mode", [
+    (3, 7, 3, 2, 1, 1), (3, 3, 1, 1, 1, 3), (1, 5, 2, 2, 1, 1), (2, 3, 0, 1, 1, 3), (3, 3, 1, 1, 2, 1),
+    (3, 3, 1, 2, 1, 2), (1, 3, 1, 1, 1, 4), (3, (3, 5), (1, 2), (1, 2), (2, 1), 1)])
+def test_conv2d_few_input_channels(ci, k, pad, stride, dil, mode):
+    """images of 1-3 channels: the op frames / pads them for the matrix-core routes (int8: zero frame + fourth
+    channel + filter rows of whole groups of 4 taps; int16: eight channels); same integers, same outputs"""
+    note("conv2d few channels", ci, k, pad, stride, dil, mode)
+    torch.manual_seed(ci * 10 + mode)
+    two = lambda v: (v, v) if isinstance(v, int) else tuple(v)
+    k, pad, stride, dil = two(k), two(pad), two(stride), two(dil)
+    x = torch.randn(2, ci, 40, 44)
+    w = torch.randn(24, ci, *k) * 0.2
+    b = torch.randn(24)
+    qmax = 127.0 if mode in (1, 3) else 32767.0
+    if mode > 2:
+        q_scale = torch.cat([torch.tensor([qmax / x.abs().max().item(), 0.0]), qmax / w.reshape(24, -1).abs().max(1)[0]])
+    else:
+        q_scale = torch.tensor([qmax / x.abs().max().item(), qmax / w.abs().max().item()])
+    q_mode = torch.tensor([mode], dtype=torch.int32)
+    ref = oops.conv2d(x.numpy(), w.numpy(), b.numpy(), pad, stride, dil, 1, q_scale.numpy(), q_mode.numpy())
+    wc, qs, qm = w.cuda(), q_scale.cuda(), q_mode.cuda()  # the same tensor objects in every call: cache hits
+    for xin in (x.cuda(), x.cuda().contiguous(memory_format=torch.channels_last)):
+        got = torch.ops.torch_mlu.conv2d(xin, wc, b.cuda(), list(pad), list(stride), list(dil), 1, qs, qm)
+        assert same_bits(ref["y"], got.cpu().numpy())
+    # the same weight with another dilation: the cached, laid-out weight must not be reused blindly
+    dil2 = (1, 2) if dil[1] == 1 else (1, 1)
+    ref2 = oops.conv2d(x.numpy(), w.numpy(), b.numpy(), pad, stride, dil2, 1, q_scale.numpy(), q_mode.numpy())
+    got2 = torch.ops.torch_mlu.conv2d(x.cuda(), wc, b.cuda(), list(pad), list(stride), list(dil2), 1, qs, qm)
+    assert same_bits(ref2["y"], got2.cpu().numpy())
+    got = torch.ops.torch_mlu.conv2d(x.cuda(), wc, b.cuda(), list(pad), list(stride), list(dil), 1, qs, qm)
+    assert same_bits(ref["y"], got.cpu().numpy())
