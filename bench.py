@@ -228,6 +228,8 @@ def main():
 
     if not args.no_extras:
         result["extras"] = extras()
+        if args.workload == "resnet50":
+            result["extras"]["dropin_modules"] = dropin_flow(net, x, args.calib_images, out)
     if not args.no_cpu_baseline:
         n_cpu = args.cpu_images or batch
         result["cpu_baseline"] = cpu_baseline(layers, sd, x[:n_cpu], outs[0][:n_cpu].float().cpu(),
@@ -284,6 +286,24 @@ def extras():
     out["quantize_f32_to_i8"] = {"elements": n, "us": round(t * 1e6, 1), "gbs": round(5 * n / t / 1e9, 1),
                                  "hbm_frac": round(5 * n / t / 1e9 / HBM_PEAK_GBS, 4)}
     return out
+
+
+def dropin_flow(net, x, calib_images, fused_logits):
+    """the same network and batch through the module-swap flow of the reference (quantize_dynamic_mlu, one
+    torch_mlu::conv2d / linear call per layer, fp32 tensors and ATen ReLU / add / pooling between them)"""
+    import torch
+    from catch_amd.core.mlu_quantize import quantize_dynamic_mlu
+    spec = {"use_avg": False, "data_scale": 1.0, "per_channel": True, "firstconv": False}
+    calib = quantize_dynamic_mlu(net, spec, dtype="int8", gen_quant=True)
+    calib(x[:calib_images])
+    q = quantize_dynamic_mlu(net)
+    q.load_state_dict(calib.state_dict())
+    q = q.to("cuda")
+    xg = x.cuda()
+    t = event_time(lambda: q(xg), 10, 3)
+    y = q(xg)
+    return {"ms_per_step": round(t * 1e3, 3), "images_per_s": round(x.shape[0] / t, 1),
+            "logits_equal_fused": bool(torch.equal(y, fused_logits))}
 
 
 def cpu_baseline(layers, sd, x_sample, gpu_logits, out_name):

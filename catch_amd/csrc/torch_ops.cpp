@@ -633,21 +633,26 @@ Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   TORCH_CHECK(input.dim() == 4 && weight.dim() == 4, "torch_mlu::conv2d expects 4-d input and weight");
   const bool half = fp_dtype(input, "quantify only support input float/half") == CATCHQ_F16;
   c10::DeviceGuard guard(input.device());
-  // An image of fewer than four channels (grey, RGB): the int8 path quantizes it into a zero frame that
-  // holds the convolution's padding, with a fourth all-zero channel, and pads the filter rows to whole
-  // groups of four taps -- the shape of the streaming first-layer kernel (int16 activations take eight
-  // channels and stay unframed).  Everything added is zeros on one side of every product.
+  // Channel counts the matrix-core routes cannot take are padded with zero channels on both operands
+  // (int8: multiples of 16, int16: multiples of 8); zeros on one side of every added product.  An image of
+  // fewer than four channels (grey, RGB) takes four, and the int8 path also quantizes it into a zero frame
+  // that holds the convolution's padding and pads the filter rows to whole groups of four taps -- the
+  // shape of the streaming first-layer kernel (int16 activations take eight channels and stay unframed).
   const int64_t ci = input.size(1), kw = weight.size(3);
-  const bool few = groups == 1 && ci < 4 && weight.size(1) == ci;
+  const bool dense = groups == 1 && weight.size(1) == ci;
+  const bool few = dense && ci < 4;
+  auto device_channels = [&](int bw_act) -> int64_t {
+    if (!dense) return ci;
+    if (bw_act == 8) return ci < 4 ? 4 : (ci + 15) / 16 * 16;
+    return (ci + 7) / 8 * 8;
+  };
   const int64_t kw_extra = (kw + 3) / 4 * 4 - kw;
   const bool can_frame = few && dilation.size() == 2 && dilation[1] == 1 && padding.size() == 2;
   auto prep = prepared_for(weight, q_scale, q_mode, [&](const Tensor &w, int bw_act) {
     Tensor wd = w;
-    if (few) {
-      const int64_t cpad = (bw_act == 8 ? 4 : 8) - ci;
-      const int64_t taps = (bw_act == 8 && can_frame) ? kw_extra : 0;
-      wd = at::constant_pad_nd(w, {0, taps, 0, 0, 0, cpad}, 0);
-    }
+    const int64_t cpad = device_channels(bw_act) - ci;
+    const int64_t taps = (few && bw_act == 8 && can_frame) ? kw_extra : 0;
+    if (cpad > 0 || taps > 0) wd = at::constant_pad_nd(w, {0, taps, 0, 0, 0, cpad}, 0);
     // the memory of a channels-last [Co,Ci/g,kh,kw] tensor is [Co][kh][kw][Ci/g]
     return wd.contiguous(at::MemoryFormat::ChannelsLast);
   }, (few ? 1 : 0) | (can_frame ? 2 : 0));
@@ -664,7 +669,7 @@ Tensor conv2d_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
                  "torch_mlu::quantize");
     pad = {0, 0};
   } else {
-    qx = quantize_to_nhwc(input, prep->bw_x, prep->pos_x, few ? (prep->bw_x == 8 ? 4 : 8) : ci);
+    qx = quantize_to_nhwc(input, prep->bw_x, prep->pos_x, device_channels(prep->bw_x));
   }
   Tensor y = conv_prepared(qx, *prep, bias, pad, stride, dilation, groups, half);
   return y.permute({0, 3, 1, 2});  // logical NCHW over channels-last memory, like the reference
@@ -779,9 +784,22 @@ Tensor linear_op(const Tensor &input, const Tensor &weight, const Tensor &bias, 
   TORCH_CHECK(input.dim() >= 1 && input.size(-1) == weight.size(1), "size mismatch: input ", input.sizes(),
               ", weight ", weight.sizes());
   c10::DeviceGuard guard(input.device());
-  auto prep = prepared_for(weight, q_scale, q_mode, [](const Tensor &w, int) { return w.contiguous(); });
-  Tensor x2 = input.contiguous().view({-1, input.size(-1)});
-  Tensor qx = quantize_op(x2, prep->bw_x, prep->pos_x, 1.0);
+  // K is padded with zeros on both operands to what the matrix-core routes take (16 int8 / 8 int16 values)
+  const int64_t k = weight.size(1);
+  auto device_k = [&](int bw_act) { return bw_act == 8 ? (k + 15) / 16 * 16 : (k + 7) / 8 * 8; };
+  auto prep = prepared_for(weight, q_scale, q_mode, [&](const Tensor &w, int bw_act) {
+    const int64_t kpad = device_k(bw_act) - k;
+    return kpad > 0 ? at::constant_pad_nd(w, {0, kpad}, 0).contiguous() : w.contiguous();
+  });
+  Tensor x2 = input.contiguous().view({-1, k});
+  Tensor qx;
+  if (device_k(prep->bw_x) != k && x2.size(0) > 0)  // rows as pixels of a [M, K, 1, 1] image, zero channels appended
+    qx = quantize_to_nhwc(x2.view({x2.size(0), k, 1, 1}), prep->bw_x, prep->pos_x, device_k(prep->bw_x))
+             .view({x2.size(0), device_k(prep->bw_x)});
+  else if (device_k(prep->bw_x) != k)
+    qx = at::empty({0, device_k(prep->bw_x)}, x2.options().dtype(int_type(prep->bw_x)));
+  else
+    qx = quantize_op(x2, prep->bw_x, prep->pos_x, 1.0);
   EpiArgs a;  // output is fp32 whatever the input type (operators/cnnl/matmul.cpp:72-74)
   a.exp2 = prep->pos_x + prep->pos_w;
   if (prep->per_channel) a.chan_div = prep->new_scale;
