@@ -84,8 +84,18 @@ __global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const float *_
     const int c = (int)(idx % C);
     const int64_t n = idx / C;
     const float *src = x + n * HW * C + c;
+    // the sum runs over the pixels in order (one fp32 addition each: the order is part of the result);
+    // eight loads are requested before their additions so that the thread has more than one in flight
     float s = 0.0f;
-    for (int p = 0; p < HW; ++p) s = s + src[(int64_t)p * C];
+    int p = 0;
+    for (; p + 8 <= HW; p += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(p + u) * C];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s = s + v[u];
+    }
+    for (; p < HW; ++p) s = s + src[(int64_t)p * C];
     y[idx] = s / (float)HW;
   }
 }
