@@ -147,17 +147,19 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
   constexpr int NG = (S == 1) ? 2 : 4;  // transposed groups per input row: pixels 0-3, 2-5 [, 4-7, 6-9]
   constexpr int NCL = 2 * NG + 2;       // input columns loaded (stride 2: one more than the window, weight 0)
   const int hi0 = ho0 * S - p.ph, wi0 = wg * PW * S - p.pw;
-  const int8_t *xi = x + (int64_t)img * p.H * p.W * p.C + c;
+  // addresses = a per-image base (the same for the whole block: scalar registers) + a 32-bit offset
+  const int8_t *xi = x + (int64_t)img * p.H * p.W * p.C;
 #pragma unroll
   for (int ri = 0; ri < NR; ++ri) {
     const int hi = hi0 + ri;
     const bool row_ok = (unsigned)hi < (unsigned)p.H;
     unsigned xr[NCL];
-    const int8_t *rowp = xi + ((int64_t)hi * p.W + wi0) * p.C;  // column 0 of the window (may lie outside: masked below)
+    const unsigned rowo = (unsigned)((hi * p.W + wi0) * p.C + c);  // column 0 of the window (may lie outside: masked below)
 #pragma unroll
     for (int col = 0; col < NCL; ++col) {
       xr[col] = 0;
-      if (row_ok && (unsigned)(wi0 + col) < (unsigned)p.W) xr[col] = *reinterpret_cast<const unsigned *>(rowp + col * p.C);
+      if (row_ok && (unsigned)(wi0 + col) < (unsigned)p.W)
+        xr[col] = *reinterpret_cast<const unsigned *>(xi + (rowo + (unsigned)(col * p.C)));
     }
     // first transposition stage on pixel pairs (2m, 2m+1): bytes (a0,b0,a1,b1) and (a2,b2,a3,b3)
     unsigned lo[NG + 1], hi2[NG + 1];
@@ -200,11 +202,11 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
     for (int px = 0; px < PW; ++px) {
       const int wo = wg * PW + px;
       if (wo >= p.Wo) continue;
-      const int64_t idx = (((int64_t)img * p.Ho + ho) * p.Wo + wo) * p.C + c;
+      const EpiAtSplit at = {(int64_t)img * p.Ho * p.Wo * p.C, (unsigned)((ho * p.Wo + wo) * p.C + c)};
       v4f res = {0.f, 0.f, 0.f, 0.f};
-      if (L.use_res) res = *reinterpret_cast<const v4f *>(e.resid + idx);
+      if (L.use_res) res = *reinterpret_cast<const v4f *>(at.at(e.resid));
       const v4i a = {acc[py][px][0], acc[py][px][1], acc[py][px][2], acc[py][px][3]};
-      epi_vec4<Sp>(a, res, L, idx, e);
+      epi_vec4<Sp>(a, res, L, at, e);
     }
   }
 }
@@ -223,6 +225,7 @@ static int dw3x3(const void *x, const void *w, int N, int H, int W, int C, int k
   Dw3Params p = {N, H, W, C, ph, pw, Ho, Wo, C / 4, (Wo + DW3_PW - 1) / DW3_PW, (Ho + DW3_PH - 1) / DW3_PH, 0};
   const int64_t items = (int64_t)p.HG * p.WG * p.CQ;
   if (items > 0x7fffff00 || N > 65535) return -1;
+  if ((int64_t)H * W * C >= (1ll << 31) || (int64_t)Ho * Wo * C >= (1ll << 31)) return -1;  // 32-bit offsets within an image
   p.items = (int)items;
   const dim3 grid((unsigned)((items + 255) / 256), (unsigned)N);
   const bool s2 = sh == 2;
