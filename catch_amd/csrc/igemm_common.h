@@ -51,6 +51,10 @@ struct EpiSpec {
   static constexpr bool kGeneric = DIV < 0;
   static constexpr int kAct = ACT;
   static constexpr int kQ = QM;
+  // ReLU / ReLU6 feeding nothing but an int8 requantization: the activation folds into the clamp of the
+  // quantizer, 0 <= x <= min(6, 127 * 2^pos)
+  static constexpr bool kFoldAct = DIV >= 0 && QM == 8 && YM == 0 && ACC == 0 && RESID != 2 &&
+                                   (ACT == CATCHQ_ACT_RELU || ACT == CATCHQ_ACT_RELU6);
   static __device__ __forceinline__ bool rcp(const EpiDev &e) { return DIV < 0 ? e.chan_rcp != nullptr : DIV == 1; }
   static __device__ __forceinline__ bool truediv(const EpiDev &e) {
     return DIV < 0 ? (e.chan_div != nullptr && e.chan_rcp == nullptr) : DIV == 2;
@@ -194,10 +198,12 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
   for (int t = 0; t < 4; ++t) {
     float x = epi_dequant1(a[t], t, L, e.exp2);
     if (L.use_res && !L.res_after) x = x + res[t];
-    if (L.act == CATCHQ_ACT_LEAKY) x = (x > 0.0f) ? x : x * e.act_slope;
-    else if (L.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
-    if (L.act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
-    if (L.use_res && L.res_after) x = x + res[t];
+    if constexpr (!S::kFoldAct) {
+      if (L.act == CATCHQ_ACT_LEAKY) x = (x > 0.0f) ? x : x * e.act_slope;
+      else if (L.act >= CATCHQ_ACT_RELU) x = (x > 0.0f) ? x : 0.0f;
+      if (L.act == CATCHQ_ACT_RELU6) x = (x < 6.0f) ? x : 6.0f;
+      if (L.use_res && L.res_after) x = x + res[t];
+    }
     v[t] = x;
   }
   if (S::y16(e)) {
@@ -209,15 +215,20 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     *reinterpret_cast<v4f *>(where.at(reinterpret_cast<float *>(e.y))) = o;
   }
   if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
-    // values are >= 0 and never NaN here, the requantization scale is 1:
+    // values are >= 0 and never NaN here (or, with the activation folded in, are made so by the median:
+    // for a NaN operand it returns the smallest of the other two, 0, which is what ReLU makes of a NaN);
+    // the requantization scale is 1:
     //   sat(rne(x * 2^-pos)) = low byte of the float  fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23)
     // (the product is exact, so the fma rounds once, to an integer, ties to even; clamping before
-    // the rounding equals clamping after it because the bound is an integer multiple of 2^pos)
-    const float hi = __builtin_ldexpf(127.0f, -e.q_neg_pos), sc = __builtin_ldexpf(1.0f, e.q_neg_pos);
+    // the rounding equals clamping after it because the bound is an integer multiple of 2^pos; a ReLU6
+    // bound of 6 below that one takes its place: min(min(x, 6), hi) = min(x, min(6, hi)))
+    float hi = __builtin_ldexpf(127.0f, -e.q_neg_pos);
+    const float sc = __builtin_ldexpf(1.0f, e.q_neg_pos);
+    if constexpr (S::kFoldAct && S::kAct == CATCHQ_ACT_RELU6) hi = (hi < 6.0f) ? hi : 6.0f;
     unsigned b[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const float x = __builtin_amdgcn_fmed3f(v[t], 0.0f, hi);  // v >= 0: this is min(v, hi), one instruction
+      const float x = __builtin_amdgcn_fmed3f(v[t], 0.0f, hi);  // one instruction for max(0, min(v, hi))
       b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
     }
     const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);

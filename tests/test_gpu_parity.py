@@ -443,6 +443,34 @@ def test_specialised_epilogues(shape):
             assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10), out["q"].cpu().numpy()), row
 
 
+@pytest.mark.parametrize("shape", [EPILOGUE_SHAPES[0], EPILOGUE_SHAPES[2], EPILOGUE_SHAPES[4]])
+@pytest.mark.parametrize("act", [1, 2])
+def test_relu_folded_into_requantization_handles_non_finite_values(shape, act):
+    """ReLU / ReLU6 -> int8 only: the kernels fold the activation into the quantizer's clamp.  NaN, +inf and -inf
+    (here from the bias) must still come out as ReLU then quantize make them: 0, the saturation value, 0; and a
+    requantization position at which the ReLU6 bound, not the int8 range, is the smaller clamp"""
+    n, ci, h, w, co, k, pad, xbits = shape
+    g = ci if (k == 3 and ci == co == 16) else 1
+    note("folded relu", shape, act)
+    r = rng(sum(shape) + act)
+    x, wt = _ints(r, (n, h, w, ci), xbits), _ints(r, (co, k, k, ci // g), 8)
+    acc, _ = orc.conv2d_nhwc(x, wt, (pad, pad), (1, 1), (1, 1), g)
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = r.standard_normal(co).astype(np.float32)
+    bias[0], bias[1], bias[2] = np.nan, np.inf, -np.inf
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    for q_pos, exp2, with_res in ((-3, -10, False), (-6, -10, False), (-4, -9, True)):
+        out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), (pad, pad), (1, 1), (1, 1), g, exp2=exp2, chan_div=cabi.dev(div),
+                               bias=cabi.dev(bias), resid=cabi.dev(resid) if with_res else None, act=act, y_dtype=None,
+                               want_acc=False, q_bw=8, q_pos=q_pos, chan_rcp=cabi.dev(np.float32(1) / div))
+        y = orc.epilogue(acc, exp2, div, bias, resid if with_res else None, act)
+        want = orc.quantize(y, 8, q_pos)
+        got = out["q"].cpu().numpy()
+        assert same_bits(want, got), (q_pos, exp2, with_res)
+        assert not got[..., 0].any() and not got[..., 2].any()
+        assert (got[..., 1] == min(127, int(6 * 2 ** -q_pos) if act == 2 else 127)).all()
+
+
 SHORTCUT_CASES = [
     # N, H, W, Ci, Co, k, pad, stride (main conv);  Hs, Ws, Cs, shortcut stride;  x bits, expected workspace use
     (2, 14, 14, 64, 256, 1, 0, 1, 14, 14, 64, 1, 8, False),     # first block of a bottleneck stage: both 1x1 s1
