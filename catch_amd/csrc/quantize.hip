@@ -158,25 +158,29 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw_nhwc_frame_kernel(cons
                                                                            int n, int c, int h, int w, int oh, int ow,
                                                                            int top, int left, int pos, float scale) {
   typedef typename QRange<BW>::type TQ;
-  const int64_t total = (int64_t)n * oh * ow, hw = (int64_t)h * w;
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < total; p += stride) {
-    const int ox = (int)(p % ow);
-    const int64_t t = p / ow;
-    const int oy = (int)(t % oh);
-    const int64_t img = t / oh;
-    const int iy = oy - top, ix = ox - left;
-    const bool inside = (unsigned)iy < (unsigned)h && (unsigned)ix < (unsigned)w;
-    TQ out[CPAD];
+  // blockIdx.y walks the output rows (image, oy), threads the pixels of a row: the row's coordinates are
+  // scalar arithmetic, a pixel costs no division
+  const int64_t hw = (int64_t)h * w, rows = (int64_t)n * oh;
+  for (int64_t row = blockIdx.y; row < rows; row += gridDim.y) {
+    const int64_t img = row / oh;
+    const int oy = (int)(row - img * oh), iy = oy - top;
+    const bool row_inside = (unsigned)iy < (unsigned)h;
+    const TIn *src = x + img * c * hw + (int64_t)iy * w;
+    TQ *dst = q + row * ow * CPAD;
+    for (int ox = blockIdx.x * kThreads + threadIdx.x; ox < ow; ox += gridDim.x * kThreads) {
+      const int ix = ox - left;
+      const bool inside = row_inside && (unsigned)ix < (unsigned)w;
+      TQ out[CPAD];
 #pragma unroll
-    for (int ch = 0; ch < CPAD; ++ch) {
-      out[ch] = 0;
-      if (inside && ch < c) out[ch] = (TQ)quant1<BW>(ld_f(x, (img * c + ch) * hw + (int64_t)iy * w + ix), scale, -pos);
+      for (int ch = 0; ch < CPAD; ++ch) {
+        out[ch] = 0;
+        if (inside && ch < c) out[ch] = (TQ)quant1<BW>(ld_f(src, ch * hw + ix), scale, -pos);
+      }
+      constexpr int BYTES = CPAD * sizeof(TQ);
+      if constexpr (BYTES == 4) *reinterpret_cast<int *>(dst + ox * CPAD) = *reinterpret_cast<int *>(out);
+      else if constexpr (BYTES == 8) *reinterpret_cast<v2i *>(dst + ox * CPAD) = *reinterpret_cast<v2i *>(out);
+      else *reinterpret_cast<v4i *>(dst + ox * CPAD) = *reinterpret_cast<v4i *>(out);
     }
-    constexpr int BYTES = CPAD * sizeof(TQ);
-    if constexpr (BYTES == 4) *reinterpret_cast<int *>(q + p * CPAD) = *reinterpret_cast<int *>(out);
-    else if constexpr (BYTES == 8) *reinterpret_cast<v2i *>(q + p * CPAD) = *reinterpret_cast<v2i *>(out);
-    else *reinterpret_cast<v4i *>(q + p * CPAD) = *reinterpret_cast<v4i *>(out);
   }
 }
 
@@ -372,8 +376,10 @@ template <typename TIn, int BW, int CPAD>
 static int launch_frame(const void *x, void *q, int n, int c, int h, int w, int oh, int ow, int top, int left, int pos,
                         float scale, hipStream_t s) {
   typedef typename QRange<BW>::type TQ;
-  quantize_nchw_nhwc_frame_kernel<TIn, BW, CPAD><<<grid_for((int64_t)n * oh * ow, kThreads), kThreads, 0, s>>>(
-      (const TIn *)x, (TQ *)q, n, c, h, w, oh, ow, top, left, pos, scale);
+  const int64_t rows = (int64_t)n * oh;
+  const dim3 grid((unsigned)((ow + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+  quantize_nchw_nhwc_frame_kernel<TIn, BW, CPAD><<<grid, kThreads, 0, s>>>((const TIn *)x, (TQ *)q, n, c, h, w, oh, ow,
+                                                                          top, left, pos, scale);
   return launch_status();
 }
 
