@@ -234,6 +234,13 @@ def main():
         n_cpu = args.cpu_images or batch
         result["cpu_baseline"] = cpu_baseline(layers, sd, x[:n_cpu], outs[0][:n_cpu].float().cpu(),
                                               fused.outputs[0])
+        # for context: what the reference's modules do with CPU tensors -- the float network (conv.py:175-177)
+        import torch as _t
+        t0 = time.time()
+        net(x[:n_cpu])
+        result["cpu_baseline"]["float_torch_cpu"] = {"value": round(n_cpu / (time.time() - t0), 2), "unit": "images/s",
+                                                     "threads": _t.get_num_threads(),
+                                                     "what": "the same network in fp32 through PyTorch's CPU kernels"}
     result["calibration_s"] = round(t_cal, 2)
     print(json.dumps(result))
 
