@@ -27,7 +27,7 @@ bool range_for(int bitwidth, Range *r) {
 
 }  // namespace
 
-CATCHQ_API int catchq_version(void) { return 100; }
+CATCHQ_API int catchq_version(void) { return 102; }
 
 CATCHQ_API const char *catchq_status_string(int status) {
   switch (status) {
