@@ -150,6 +150,45 @@ class MLUPerChannelMinMaxObserver(_MLUObserverBase):
         return "min_val={}, max_val={}".format(self.min_vals, self.max_vals)
 
 
+class MLULrnObserver(MLUMinMaxObserver):
+    """Range observer of a local-response-normalisation input (observer.py:172-199 in the reference): the same
+    running min / max as MLUMinMaxObserver, but the scale describes the squared values the layer sums."""
+
+    def calculate_qparams(self):
+        self.scale = self._calculate_qparams(self.min_val ** 2, self.max_val ** 2)
+
+
+class MLUNormObserver(_MLUObserverBase):
+    """Observer of an L2-normalisation input (observer.py:252-294 in the reference).  The layer squares its
+    input (scaled by 1 / max) and takes the root of the channel sums; both intermediate tensors get a range,
+    [min, max] of x'^2 and of sqrt(sum_c x'^2) + 1e-10, hence two scales."""
+
+    def __init__(self, dtype="int8", qscheme=mlu_qscheme):
+        super().__init__(dtype=dtype, qscheme=qscheme)
+        self.boundary_1 = None
+        self.boundary_2 = None
+        self.scale = None
+
+    def forward(self, x_orig):
+        if not self._accept() or self.dtype not in _QMAX:
+            return
+        x = x_orig.detach()
+        squares = (x * (1.0 / x.max().item())).pow(2)
+        norms = squares.sum(dim=1).sqrt() + 1e-10
+        new = ([squares.min().item(), squares.max().item()], [norms.min().item(), norms.max().item()])
+        if self.boundary_1 is None or self.boundary_2 is None:
+            self.boundary_1, self.boundary_2 = new
+        else:
+            self.boundary_1 = [min(self.boundary_1[0], new[0][0]), max(self.boundary_1[1], new[0][1])]
+            self.boundary_2 = [min(self.boundary_2[0], new[1][0]), max(self.boundary_2[1], new[1][1])]
+
+    def calculate_qparams(self):
+        self.scale = [self._calculate_qparams(*self.boundary_1), self._calculate_qparams(*self.boundary_2)]
+
+    def extra_repr(self):
+        return "boundary_1={}, boundary_2={}".format(self.boundary_1, self.boundary_2)
+
+
 class NoopObserver(Observer):
     def __init__(self, dtype=torch.float16):
         if dtype != torch.float16:
@@ -176,6 +215,14 @@ def mlu_activation_observer(dtype, qscheme):
 
 def mlu_minmax_observer(dtype, qscheme):
     return MLUMinMaxObserver.with_args(dtype=dtype, qscheme=qscheme)
+
+
+def mlu_norm_observer(dtype, qscheme):
+    return MLUNormObserver.with_args(dtype=dtype, qscheme=qscheme)
+
+
+def mlu_lrn_observer(dtype, qscheme):
+    return MLULrnObserver.with_args(dtype=dtype, qscheme=qscheme)
 
 
 def mlu_weight_per_channel_observer(dtype, qscheme):

@@ -230,3 +230,24 @@ def test_missing_native_library_is_loud(tmp_path, monkeypatch):
     monkeypatch.setattr(_native, "KERNEL_LIB", str(tmp_path / "nope.so"))
     with pytest.raises(ImportError, match="catch_amd/build.py"):
         _native.kernel_lib()
+
+
+def test_lrn_and_norm_observers():
+    """observer.py:172-199 and :252-294 in the reference: the LRN observer's scale describes the squared range;
+    the norm observer keeps two ranges, of the max-normalised squares and of the channel norms"""
+    from catch_amd.core.quantized import observer as obs
+    x = torch.tensor([[[[1.0, 3.0]], [[2.0, 0.5]]]])  # [1, 2, 1, 2], non-negative like a post-ReLU tensor
+    lrn = obs.mlu_lrn_observer("int8", {"iteration": 2})()
+    lrn(x)
+    lrn(x * 0.5)
+    lrn(x * 100)  # beyond `iteration`: ignored
+    lrn.calculate_qparams()
+    assert (lrn.min_val, lrn.max_val) == (0.25, 3.0)
+    assert lrn.scale == 127.0 / 9.0
+    norm = obs.mlu_norm_observer("int16", {"iteration": 1})()
+    norm(x)
+    norm.calculate_qparams()
+    sq = (x / 3.0) ** 2
+    nr = sq.sum(1).sqrt() + 1e-10
+    assert norm.boundary_1 == [sq.min().item(), sq.max().item()] and norm.boundary_2 == [nr.min().item(), nr.max().item()]
+    assert norm.scale == [32767.0 / sq.max().item(), 32767.0 / nr.max().item()]
