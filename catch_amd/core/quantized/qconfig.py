@@ -4,8 +4,8 @@ from collections import namedtuple
 
 import torch.nn as nn
 
-from .observer import (NoopObserver, default_mlu_observer, mlu_activation_observer, mlu_weight_observer,
-                       mlu_weight_per_channel_observer)
+from .observer import (NoopObserver, default_mlu_observer, mlu_activation_observer, mlu_norm_observer,
+                       mlu_weight_observer, mlu_weight_per_channel_observer)
 
 
 class QConfig(namedtuple("QConfig", ["activation", "weight"])):
@@ -29,6 +29,10 @@ def mlu_activation_qconfig(dtype, qscheme):
 
 def custom_mlu_qconfig(dtype, qscheme):
     return QConfig(weight=mlu_weight_observer(dtype), activation=mlu_activation_observer(dtype, qscheme))
+
+
+def norm_mlu_qconfig(dtype, qscheme):
+    return QConfig(weight=mlu_weight_observer(dtype), activation=mlu_norm_observer(dtype, qscheme))
 
 
 def mlu_per_channel_qconfig(dtype, qscheme):
