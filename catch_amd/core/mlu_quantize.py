@@ -90,6 +90,7 @@ def quantize_dynamic_mlu(model, qconfig_spec=None, dtype=None, mapping=None, inp
                 w_obs = mlu_weight_per_channel_observer(dtype, qconfig_spec)
             a_obs = mlu_activation_observer_dict[qconfig_spec.get("method", "minmax")](dtype, qconfig_spec)
             per_type = {t: compose_qconfig(w_obs, a_obs) for t in _QUANT_TYPES}
+            per_type[nn.Conv3d] = compose_qconfig(mlu_weight_observer(dtype), a_obs)  # 3-d: per-tensor weights only
         else:
             per_type = {t: custom_mlu_qconfig(dtype, qconfig_spec) for t in _QUANT_TYPES}
     else:
