@@ -363,3 +363,35 @@ def test_conv2d_few_input_channels(ci, k, pad, stride, dil, mode):
     assert same_bits(ref2["y"], got2.cpu().numpy())
     got = torch.ops.torch_mlu.conv2d(x.cuda(), wc, b.cuda(), list(pad), list(stride), list(dil), 1, qs, qm)
     assert same_bits(ref["y"], got.cpu().numpy())
+
+
+@pytest.mark.parametrize("k,co,h,w", [(1, 1, 101, 130), (3, 37, 120, 150), (7, 64, 100, 333), (10, 100, 160, 104)])
+def test_conv2d_first_qint(k, co, h, w):
+    """test/magicmind/op_test/test_conv.py:160-229 in the reference: an RGBA image with raw 0..255 pixel values goes
+    to the device, the module normalises it with the mean / std recorded at calibration (firstconv), half input,
+    stride (1, 4), padding (2, 2); rel-RMS <= 0.02 against the float model on the normalised image"""
+    note("conv2d first conv", k, co, h, w)
+    torch.manual_seed(k * 100 + co)
+    mean, std = [0.485, 0.456, 0.406, 0.449], [0.229, 0.224, 0.225, 0.226]
+    raw = torch.randint(0, 255, (1, 4, h, w)).float()
+    x_cpu = (raw / 255.0 - torch.tensor(mean).view(1, 4, 1, 1)) / torch.tensor(std).view(1, 4, 1, 1)
+    model = nn.Sequential(nn.Conv2d(4, co, k, (1, 4), (2, 2), (1, 1), 1, True)).eval().float()
+    want_float = model(x_cpu).numpy()
+    qconfig = {"use_avg": False, "data_scale": 1.0, "mean": mean, "std": std, "firstconv": True, "per_channel": True}
+    calib = quantize_dynamic_mlu(model, qconfig, dtype="int8", gen_quant=True)
+    calib(x_cpu)
+    ckpt = calib.state_dict()
+    np.testing.assert_allclose(ckpt["0.input_mean"].flatten().numpy(), np.array(mean) * 255, rtol=1e-6)
+    qmodel = quantize_dynamic_mlu(model)
+    qmodel.load_state_dict(ckpt)
+    qmodel.half().to("cuda")
+    conv = qmodel[0]
+    got = qmodel(raw.half().to("cuda"))
+    assert got.dtype == torch.float16 and got.shape == want_float.shape
+    assert rel_rms(want_float, got.float().cpu().numpy()) <= 0.02
+    # exact: the oracle on the tensor the module hands to the op
+    x_norm = ((raw.half().cuda() - conv.input_mean) / conv.input_std)
+    assert x_norm.dtype == torch.float16
+    ref = oops.conv2d(x_norm.cpu().numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
+                      (2, 2), (1, 4), (1, 1), 1, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
+    assert same_bits(ref["y"], got.cpu().numpy())
