@@ -208,8 +208,14 @@ def test_quantized_model(ci):
     ckpt = calibrate(net, x, "int8", True)
     qnet = quantize_dynamic_mlu(net)
     qnet.load_state_dict(ckpt)
-    got = qnet.to("cuda")(x.to("cuda")).cpu().numpy()
-    assert rel_rms(want, got) <= 0.02
+    qnet = qnet.to("cuda")
+    got = qnet(x.to("cuda"))
+    assert rel_rms(want, got.cpu().numpy()) <= 0.02
+    # the reference runs this model through torch.jit.trace (test_quantization.py:66-70): the traced module, with
+    # the torch_mlu::conv2d nodes in its graph, gives the eager result
+    traced = torch.jit.trace(qnet, x.to("cuda"), check_trace=False)
+    assert "torch_mlu::conv2d" in str(traced.inlined_graph)
+    assert torch.equal(traced(x.to("cuda")), got)
 
 
 def test_helper_ops():
