@@ -40,6 +40,8 @@ def parse():
     ap.add_argument("--seq-passes", type=int, default=10, help="eager passes timed launch by launch for the roofline")
     ap.add_argument("--calib-images", type=int, default=8)
     ap.add_argument("--cpu-images", type=int, default=0, help="images of the batch the CPU baseline runs (0: the whole batch)")
+    ap.add_argument("--fractional-scale", action="store_true",
+                    help="quantize with position and fractional scale (steps of absmax/qmax) instead of power-of-two steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -157,7 +159,11 @@ def main():
         sd = pipeline.calibrate(net, x[:args.calib_images], "int8", True)
         what = "int8 (per-channel W, per-tensor act), batch %d, 3x224x224 N(0,1)" % batch
     t_cal = time.time() - t0
-    fused = pipeline.FusedNet(layers, sd, out_half=detector)
+    if args.fractional_scale:
+        if detector:
+            sys.exit("--fractional-scale needs a checkpoint of scales; the detector's holds bit widths and positions")
+        what += ", position + fractional scale"
+    fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale)
     xg = x.cuda()
     static_in, replay = fused.capture(xg)
     static_in.copy_(xg)
@@ -228,12 +234,12 @@ def main():
 
     if not args.no_extras:
         result["extras"] = extras()
-        if args.workload == "resnet50":
+        if args.workload == "resnet50" and not args.fractional_scale:  # the modules quantize in power-of-two steps
             result["extras"]["dropin_modules"] = dropin_flow(net, x, args.calib_images, out)
     if not args.no_cpu_baseline:
         n_cpu = args.cpu_images or batch
         result["cpu_baseline"] = cpu_baseline(layers, sd, x[:n_cpu], outs[0][:n_cpu].float().cpu(),
-                                              fused.outputs[0])
+                                              fused.outputs[0], args.fractional_scale)
         # for context: what the reference's modules do with CPU tensors -- the float network (conv.py:175-177)
         import torch as _t
         t0 = time.time()
@@ -313,14 +319,14 @@ def dropin_flow(net, x, calib_images, fused_logits):
             "logits_equal_fused": bool(torch.equal(y, fused_logits))}
 
 
-def cpu_baseline(layers, sd, x_sample, gpu_logits, out_name):
+def cpu_baseline(layers, sd, x_sample, gpu_logits, out_name, fractional_scale=False):
     """the oracle's unfused execution of the same network on a few images of the same batch"""
     import numpy as np
     import oracle as orc
     from oracle import netref
     sdn = {k: v.detach().cpu().numpy() for k, v in sd.items()}
     t0 = time.time()
-    t, _ = netref.run(layers, sdn, x_sample.numpy(), record=False)
+    t, _ = netref.run(layers, sdn, x_sample.numpy(), record=False, fractional_scale=fractional_scale)
     dt = time.time() - t0
     if gpu_logits.dim() == 4:  # logical NCHW -> the oracle's NHWC
         gpu_logits = gpu_logits.permute(0, 2, 3, 1).contiguous()

@@ -433,32 +433,32 @@ Tensor mm_q_op(const Tensor &a, int64_t pos_a, const Tensor &b, int64_t pos_b) {
 }
 
 // fp NCHW (or channels-last) activations -> NHWC integer tensor [N,H,W,cpad]
-Tensor quantize_to_nhwc(const Tensor &x, int bw, int pos, int64_t cpad) {
+Tensor quantize_to_nhwc(const Tensor &x, int bw, int pos, int64_t cpad, float scale = 1.0f) {
   const int dt = fp_dtype(x, "quantify only support input float/half");
   TORCH_CHECK(x.dim() == 4, "a 4-d activation tensor is expected");
   const int64_t n = x.size(0), c = x.size(1), h = x.size(2), w = x.size(3);
   if (cpad < c) cpad = c;
   Tensor q = at::empty({n, h, w, cpad}, x.options().dtype(int_type(bw)));
   if (cpad == c && x.is_contiguous(at::MemoryFormat::ChannelsLast)) {
-    check_status(catchq_quantize(x.data_ptr(), dt, q.data_ptr(), bw, x.numel(), pos, 1.0f, current_stream()),
+    check_status(catchq_quantize(x.data_ptr(), dt, q.data_ptr(), bw, x.numel(), pos, scale, current_stream()),
                  "torch_mlu::quantize");
     return q;
   }
   Tensor xc = x.is_contiguous() ? x : x.contiguous();
   check_status(catchq_quantize_nchw_to_nhwc(xc.data_ptr(), dt, q.data_ptr(), bw, (int)n, (int)c, (int)h, (int)w,
-                                            (int)cpad, pos, 1.0f, current_stream()),
+                                            (int)cpad, pos, scale, current_stream()),
                "torch_mlu::quantize");
   return q;
 }
 
-Tensor quantize_nhwc_op(const Tensor &x, int64_t bitwidth, int64_t position, int64_t cpad) {
+Tensor quantize_nhwc_op(const Tensor &x, int64_t bitwidth, int64_t position, int64_t cpad, double scale) {
   c10::DeviceGuard guard(x.device());
-  return quantize_to_nhwc(x, (int)bitwidth, (int)position, cpad);
+  return quantize_to_nhwc(x, (int)bitwidth, (int)position, cpad, (float)scale);
 }
 
 // [N,C,H,W] floating -> [N, out_h, out_w, cpad] integers, the image at (top, left), zeros around it
 Tensor quantize_nhwc_frame_op(const Tensor &x, int64_t bitwidth, int64_t position, int64_t cpad, int64_t out_h,
-                              int64_t out_w, int64_t top, int64_t left) {
+                              int64_t out_w, int64_t top, int64_t left, double scale) {
   c10::DeviceGuard guard(x.device());
   const int dt = fp_dtype(x, "quantify only support input float/half");
   TORCH_CHECK(x.dim() == 4, "a 4-d activation tensor is expected");
@@ -466,7 +466,7 @@ Tensor quantize_nhwc_frame_op(const Tensor &x, int64_t bitwidth, int64_t positio
   Tensor q = at::empty({x.size(0), out_h, out_w, cpad}, x.options().dtype(int_type(bitwidth)));
   check_status(catchq_quantize_nchw_to_nhwc_frame(xc.data_ptr(), dt, q.data_ptr(), (int)bitwidth, (int)x.size(0),
                                                   (int)x.size(1), (int)x.size(2), (int)x.size(3), (int)cpad,
-                                                  (int)out_h, (int)out_w, (int)top, (int)left, (int)position, 1.0f,
+                                                  (int)out_h, (int)out_w, (int)top, (int)left, (int)position, (float)scale,
                                                   current_stream()),
                "torch_mlu::quantize");
   return q;
@@ -863,9 +863,9 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("linear(Tensor input, Tensor weight, Tensor bias, Tensor q_scale, Tensor q_mode) -> Tensor");
   m.def("quantize(Tensor x, int bitwidth, int position, float scale=1.0) -> Tensor");
   m.def("quantize_dev(Tensor x, int bitwidth, Tensor position) -> Tensor");
-  m.def("quantize_nhwc(Tensor x, int bitwidth, int position, int cpad=0) -> Tensor");
+  m.def("quantize_nhwc(Tensor x, int bitwidth, int position, int cpad=0, float scale=1.0) -> Tensor");
   m.def("quantize_nhwc_frame(Tensor x, int bitwidth, int position, int cpad, int out_h, int out_w, int top, "
-        "int left) -> Tensor");
+        "int left, float scale=1.0) -> Tensor");
   m.def("quantize_param(Tensor x, int bitwidth, int mode) -> (Tensor, Tensor, Tensor)");
   m.def("quantize_per_channel(Tensor w, Tensor scales, int bitwidth) -> (Tensor, Tensor, Tensor)");
   m.def("dequantize(Tensor q, int position, float scale=1.0, bool half=False) -> Tensor");

@@ -35,9 +35,19 @@ def pos_from_scale(bw, scale):
     return p.value
 
 
+def quant_params(bw, scale):
+    """scale (= qmax / absmax) -> (position, fractional scale in [1, 2)): the general form
+    q = rne(x * scale_frac * 2^-position) whose step is absmax / qmax exactly
+    (setQuantizedParams, torch_mlu/csrc/jit/utils/utils.cpp:81-118 in the reference)"""
+    p, f, sf = ctypes.c_int(), ctypes.c_float(), ctypes.c_float()
+    _native.check(_native.kernel_lib().catchq_quant_params(int(bw), float(scale), ctypes.byref(p), ctypes.byref(f),
+                                                           ctypes.byref(sf)), "quant_params")
+    return p.value, f.value
+
+
 class _LayerQ(object):
     """decoded q-params and the quantized weight of one conv / fc layer"""
-    __slots__ = ("bw_x", "bw_w", "pos_x", "pos_w", "qw", "chan_div", "bias", "exp2", "cpad", "groups")
+    __slots__ = ("bw_x", "bw_w", "pos_x", "scale_x", "pos_w", "qw", "chan_div", "bias", "exp2", "cpad", "groups")
 
 
 def _pad16(c, bw=8):
@@ -60,10 +70,33 @@ def _act_bits(layer, sd):
     return int(sd[k + "scale"].detach().float().cpu()[0].item())
 
 
-def _decode(layer, sd, device, ci_dev, co_dev):
+def _quantize_weight_fractional(w, bw, scales):
+    """w [Co, ...] fp32 (dim 0 slowest in memory), scales: one (per tensor) or Co (per axis) values of
+    qmax / absmax.  Each channel is quantized with its own (position, fractional scale)
+    (setQuantizedParams / setQuantizedParamsPerAxis, jit/utils/utils.cpp:81-167 in the reference).
+    -> (q, P, div): integer weights, the largest position P, and div[c] = scale_c * 2^(P - position_c),
+    so that the real value of q[c, ...] is q * 2^P / div[c]."""
+    co = w.shape[0]
+    pf = [quant_params(bw, float(v)) for v in scales]
+    if len(pf) == 1:
+        q = torch.ops.torch_mlu.quantize(w, bw, pf[0][0], pf[0][1])
+        pf = pf * co
+    else:
+        rows = w.reshape(co, -1)
+        q = torch.stack([torch.ops.torch_mlu.quantize(rows[c], bw, pf[c][0], pf[c][1]) for c in range(co)])
+        q = q.reshape(w.shape)
+    top = max(p for p, _ in pf)
+    div = np.array([np.ldexp(np.float32(f), top - p) for p, f in pf], dtype=np.float32)
+    return q, top, div
+
+
+def _decode(layer, sd, device, ci_dev, co_dev, fractional=False):
     """ci_dev / co_dev: channel counts of the layer's input / output tensors as laid out on the
-    device (>= the real counts; extra channels are zeros: zero weights, zero bias, divisor 1)."""
+    device (>= the real counts; extra channels are zeros: zero weights, zero bias, divisor 1).
+    fractional: quantize with position *and* fractional scale (steps of exactly absmax / qmax) rather
+    than with the power-of-two step the eager ops use."""
     q = _LayerQ()
+    q.scale_x = 1.0
     k = _key(layer.name)
     w = sd[k + "weight"].to(device=device, dtype=torch.float32)
     scale = sd[k + "scale"].detach().float().cpu()
@@ -73,7 +106,20 @@ def _decode(layer, sd, device, ci_dev, co_dev):
     q.chan_div = None
     if layer.kind == "conv":
         w = w.contiguous(memory_format=torch.channels_last)  # memory [Co][kh][kw][Ci/g]
-    if mode.numel() == 1:
+    if fractional:
+        if mode.numel() != 1:
+            raise ValueError("%s: a checkpoint of bit widths and positions holds no fractional scales" % layer.name)
+        m = int(mode[0])
+        bw = 8 if m in (1, 3) else 16
+        q.bw_x = q.bw_w = bw
+        q.pos_x, q.scale_x = quant_params(bw, scale[0].item())
+        if layer.kind == "conv":  # [Co,kh,kw,Ci/g] contiguous: every channel is one run of memory
+            w = w.permute(0, 2, 3, 1).contiguous()
+        qw, q.pos_w, div = _quantize_weight_fractional(w, bw, scale[2:].tolist() if m > 2 else [scale[1].item()])
+        if layer.kind == "conv":
+            qw = qw.permute(0, 3, 1, 2)  # logical [Co,Ci/g,kh,kw] again, same memory
+        q.chan_div = torch.from_numpy(np.float32(q.scale_x) * div).to(device)
+    elif mode.numel() == 1:
         m = int(mode[0])
         bw = 8 if m in (1, 3) else 16
         q.bw_x = q.bw_w = bw
@@ -115,7 +161,11 @@ def _decode(layer, sd, device, ci_dev, co_dev):
 
 
 class FusedNet(object):
-    def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True):
+    def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True,
+                 fractional_scale=False):
+        """fractional_scale: quantize activations and weights with position and fractional scale -- the
+        general form the reference's fused (graph) mode hands to its backend per tensor / per axis
+        (jit/utils/utils.cpp:81-167) -- instead of the eager ops' power-of-two steps."""
         self.layers = list(layers)
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
@@ -135,7 +185,7 @@ class FusedNet(object):
                 self.chan[l.name] = self.cdev[l.name] = sum(self.chan[s_] for s_ in l.src)
             else:
                 self.chan[l.name], self.cdev[l.name] = self.chan[l.src], self.cdev[l.src]
-        self.q = {l.name: _decode(l, state_dict, self.device, self.cdev[l.src], self.cdev[l.name])
+        self.q = {l.name: _decode(l, state_dict, self.device, self.cdev[l.src], self.cdev[l.name], fractional_scale)
                   for l in self.layers if l.kind in ("conv", "fc")}
         self._plan_demands()
         self._graph = None
@@ -179,7 +229,7 @@ class FusedNet(object):
             return [0, 0]
         return [layer.pad, layer.pad]
 
-    # which forms of every tensor are needed: 'f' (fp32 NHWC) and/or quantized at (bitwidth, position)
+    # which forms of every tensor are needed: 'f' (fp32 NHWC) and/or quantized at (bitwidth, position, scale)
     def _plan_demands(self):
         names = ["input"] + [l.name for l in self.layers]
         self.q_demand = {n: [] for n in names}
@@ -194,7 +244,7 @@ class FusedNet(object):
         for l in reversed(self.layers):
             if l.kind in ("conv", "fc"):
                 lq = self.q[l.name]
-                want_q(l.src, (lq.bw_x, lq.pos_x))
+                want_q(l.src, (lq.bw_x, lq.pos_x, lq.scale_x))
                 if l.add:
                     self.f_demand[l.add] = True
             elif l.kind == "gap":
@@ -231,16 +281,16 @@ class FusedNet(object):
             if self.stem:
                 sp, h, w = self.stem["pad"], x.shape[2], x.shape[3]
                 env[("input",) + d] = ops.quantize_nhwc_frame(x, d[0], d[1], self.cdev["input"], h + 2 * sp,
-                                                              w + 2 * sp + self.stem["extra"], sp, sp)
+                                                              w + 2 * sp + self.stem["extra"], sp, sp, d[2])
             else:
-                env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"])
+                env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"], d[2])
         for l in self.layers:
             name = l.name
             if l.kind == "conv" and not tracing and name in self._fused_away:
                 continue
             if l.kind == "conv":
                 lq = self.q[name]
-                qx = env[(l.src, lq.bw_x, lq.pos_x)]
+                qx = env[(l.src, lq.bw_x, lq.pos_x, lq.scale_x)]
                 qd = self.q_demand[name][0] if self.q_demand[name] else None
                 want_y = self.f_demand[name] or tracing or qd is None
                 ds = None if tracing else self.shortcut_of.get(name)
@@ -248,10 +298,10 @@ class FusedNet(object):
                 if ds is not None:
                     dq = self.q[ds.name]
                     y, q = ops.qconv2d_shortcut(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias,
-                                                env[(ds.src, dq.bw_x, dq.pos_x)], dq.qw, ds.stride, dq.exp2,
+                                                env[(ds.src, dq.bw_x, dq.pos_x, dq.scale_x)], dq.qw, ds.stride, dq.exp2,
                                                 dq.chan_div, dq.bias, self.padding(l), [l.stride, l.stride], [1, 1],
                                                 _ACT_CODE[l.act], want_y, self.out_half and name in self.outputs,
-                                                qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
+                                                qd[0] if qd else 0, qd[1] if qd else 0, qd[2] if qd else 1.0, LEAKY_SLOPE,
                                                 bool(l.add_after))
                     acc = None
                 else:
@@ -259,7 +309,7 @@ class FusedNet(object):
                     y, q, acc = ops.qconv2d(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, self.padding(l),
                                             [l.stride, l.stride], [1, 1], lq.groups, _ACT_CODE[l.act], want_y,
                                             self.out_half and name in self.outputs, tracing,
-                                            qd[0] if qd else 0, qd[1] if qd else 0, 1.0, LEAKY_SLOPE,
+                                            qd[0] if qd else 0, qd[1] if qd else 0, qd[2] if qd else 1.0, LEAKY_SLOPE,
                                             bool(l.add_after))
                 tick(name)
                 if want_y:
@@ -267,7 +317,7 @@ class FusedNet(object):
                 if qd:
                     env[(name,) + qd] = q
                 for d in self.q_demand[name][1:]:
-                    env[(name,) + d] = ops.quantize(y, d[0], d[1])
+                    env[(name,) + d] = ops.quantize(y, d[0], d[1], d[2])
                 if tracing:
                     trace[name] = dict(qx=qx, acc=acc, y=y)
                     if self.stem and name == self.stem["name"]:  # the image inside the frame
@@ -276,7 +326,7 @@ class FusedNet(object):
                         trace[name]["qx"] = qx[:, sp:qx.shape[1] - sp, sp:qx.shape[2] - sp - self.stem["extra"]].contiguous()
             elif l.kind == "fc":
                 lq = self.q[name]
-                qx = env[(l.src, lq.bw_x, lq.pos_x)]
+                qx = env[(l.src, lq.bw_x, lq.pos_x, lq.scale_x)]
                 qx2 = qx.reshape(qx.shape[0], -1)
                 tick(name)
                 y, _, acc = ops.qlinear(qx2, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, tracing, 0, 0, 1.0)
@@ -291,7 +341,7 @@ class FusedNet(object):
                 g = ops.global_avgpool_nhwc(env[(l.src, "f")])
                 env[(name, "f")] = g.reshape(g.shape[0], 1, 1, g.shape[1])
                 for d in self.q_demand[name]:
-                    env[(name,) + d] = ops.quantize(env[(name, "f")], d[0], d[1])
+                    env[(name,) + d] = ops.quantize(env[(name, "f")], d[0], d[1], d[2])
             elif l.kind == "upsample":
                 for form in self._forms(name):
                     t = env[(l.src,) + form]

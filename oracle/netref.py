@@ -11,7 +11,7 @@ import numpy as np
 
 from . import (conv2d_nhwc, epilogue, gemm_nt, global_avgpool_nhwc, maxpool_nhwc, quantize,
                quantize_per_channel)
-from .ops import decode_qparams
+from .ops import decode_fractional, decode_qparams, quantize_weight_fractional
 
 _ACT = {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}
 LEAKY_SLOPE = 0.1
@@ -21,15 +21,21 @@ def _key(name):
     return "mods." + name.replace(".", "_") + "."
 
 
-def run(layers, sd, x_nchw, record=True):
+def run(layers, sd, x_nchw, record=True, fractional_scale=False):
     """sd: dict of numpy arrays (weight [Co,Ci/g,kh,kw] / [N,K], bias, scale, quantized_mode).
-    record=False keeps only the activations (no per-layer quantized inputs / integer sums)."""
+    record=False keeps only the activations (no per-layer quantized inputs / integer sums).
+    fractional_scale: quantize with position and fractional scale per tensor / per output channel
+    (ops.decode_fractional) instead of the eager ops' power-of-two steps."""
     t = {"input": np.ascontiguousarray(np.transpose(np.asarray(x_nchw, np.float32), (0, 2, 3, 1)))}
     rec = {}
     for l in layers:
         if l.kind in ("conv", "fc"):
             k = _key(l.name)
-            d = decode_qparams(sd[k + "scale"], sd[k + "quantized_mode"])
+            if fractional_scale:
+                fr = decode_fractional(sd[k + "scale"], sd[k + "quantized_mode"], np.shape(sd[k + "weight"])[0])
+                d = dict(bw_x=fr["bw"], pos_x=fr["pos_x"], pos_w=fr["exp2"] - fr["pos_x"], new_scale=fr["div"])
+            else:
+                d = decode_qparams(sd[k + "scale"], sd[k + "quantized_mode"])
             w = np.asarray(sd[k + "weight"], np.float32)
             b = sd.get(k + "bias")
             b = None if b is None else np.asarray(b, np.float32)
@@ -38,8 +44,13 @@ def run(layers, sd, x_nchw, record=True):
                 w = np.ascontiguousarray(np.transpose(w, (0, 2, 3, 1)))
             else:
                 x = x.reshape(x.shape[0], -1)
-            qx = quantize(x, d["bw_x"], d["pos_x"])
-            qw = quantize_per_channel(w, d["bw_w"], d["sf"]) if d["per_channel"] else quantize(w, d["bw_w"], d["pos_w"])
+            if fractional_scale:
+                qx = quantize(x, fr["bw"], fr["pos_x"], fr["scale_x"])
+                qw = quantize_weight_fractional(w, fr)
+            else:
+                qx = quantize(x, d["bw_x"], d["pos_x"])
+                qw = (quantize_per_channel(w, d["bw_w"], d["sf"]) if d["per_channel"]
+                      else quantize(w, d["bw_w"], d["pos_w"]))
             if l.kind == "conv":
                 acc, ovf = conv2d_nhwc(qx, qw, (l.pad, l.pad), (l.stride, l.stride), (1, 1), l.groups)
                 resid = t[l.add] if l.add else None

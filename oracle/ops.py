@@ -9,8 +9,8 @@ logical NCHW on input/output like the ops, NHWC inside.
 """
 import numpy as np
 
-from . import (conv2d_nhwc, conv_out_size, epilogue, gemm_nt, per_channel_params, pos_from_scale, quantize,
-               quantize_per_channel)
+from . import (conv2d_nhwc, conv_out_size, epilogue, gemm_nt, per_channel_params, pos_from_scale, quant_params,
+               quantize, quantize_per_channel)
 
 
 def decode_qparams(q_scale, q_mode):
@@ -36,6 +36,35 @@ def decode_qparams(q_scale, q_mode):
         return d
     return dict(bw_x=int(q_scale[0]), bw_w=int(q_scale[1]), per_channel=False, pos_x=int(q_mode[0]),
                 pos_w=int(q_mode[1]), new_scale=None, sf=None)
+
+
+def decode_fractional(q_scale, q_mode, co):
+    """Encoding A read the way the reference's graph mode reads it: every tensor (per-axis: every
+    output channel) gets position and fractional scale from its own scale = qmax / absmax
+    (setQuantizedParams / setQuantizedParamsPerAxis, torch_mlu/csrc/jit/utils/utils.cpp:81-167), so its
+    step is absmax / qmax rather than a power of two.
+    -> dict(bw, pos_x, scale_x, pos_c[], scale_c[], exp2, div[co]): a weight of channel c is
+    q * 2^pos_c / scale_c; with P = max pos_c, an integer sum dequantizes as
+    acc * 2^(pos_x + P) / div[c], div[c] = fp32(scale_x * scale_c * 2^(P - pos_c))."""
+    q_scale = np.asarray(q_scale, dtype=np.float32).reshape(-1)
+    mode = int(np.asarray(q_mode).reshape(-1)[0])
+    bw = 8 if mode in (1, 3) else 16
+    pos_x, scale_x, _ = quant_params(bw, q_scale[0])
+    per = [quant_params(bw, s) for s in (q_scale[2:] if mode > 2 else q_scale[1:2])]
+    pos_c = np.array([p for p, _, _ in per], np.int32)
+    scale_c = np.array([f for _, f, _ in per], np.float32)
+    top = int(pos_c.max())
+    div = np.float32(scale_x) * np.ldexp(scale_c, top - pos_c).astype(np.float32)
+    return dict(bw=bw, pos_x=pos_x, scale_x=scale_x, pos_c=pos_c, scale_c=scale_c, exp2=pos_x + top,
+                div=np.ascontiguousarray(np.broadcast_to(div.astype(np.float32), (co,))))
+
+
+def quantize_weight_fractional(w, d):
+    """w [Co, ...]; one (position, scale) for the tensor or one per output channel"""
+    if d["pos_c"].size == 1:
+        return quantize(w, d["bw"], int(d["pos_c"][0]), float(d["scale_c"][0]))
+    return np.stack([quantize(np.ascontiguousarray(w[c]), d["bw"], int(d["pos_c"][c]), float(d["scale_c"][c]))
+                     for c in range(w.shape[0])])
 
 
 def _quantize_weight(w, d):

@@ -412,11 +412,14 @@ EPILOGUE_SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("q_scale", [1.0, 1.3720703125, 1.9999998807907104])
 @pytest.mark.parametrize("shape", EPILOGUE_SHAPES)
-def test_specialised_epilogues(shape):
+def test_specialised_epilogues(shape, q_scale):
+    """every epilogue instance the kernels are compiled with, with a unit requantization scale (the eager ops'
+    power-of-two steps) and with fractional ones"""
     n, ci, h, w, co, k, pad, xbits = shape
     g = ci if (k == 3 and ci == co == 16) else 1
-    note("specialised epilogues", shape)
+    note("specialised epilogues", shape, q_scale)
     r = rng(sum(shape))
     x, wt = _ints(r, (n, h, w, ci), xbits), _ints(r, (co, k, k, ci // g), 8)
     acc, ovf = orc.conv2d_nhwc(x, wt, (pad, pad), (1, 1), (1, 1), g)
@@ -430,7 +433,7 @@ def test_specialised_epilogues(shape):
         out = cabi.conv2d_nhwc(xd, wd, (pad, pad), (1, 1), (1, 1), g, exp2=exp2,
                                chan_div=cabi.dev(div) if per_channel else None, bias=cabi.dev(bias),
                                resid=cabi.dev(resid) if res_mode else None, act=act, y_dtype=y_dtype, want_acc=False,
-                               q_bw=q_bw, q_pos=-3 if q_bw == 8 else -10,
+                               q_bw=q_bw, q_pos=-3 if q_bw == 8 else -10, q_scale=q_scale,
                                chan_rcp=cabi.dev(np.float32(1) / div) if per_channel else None, act_slope=0.1,
                                resid_after_act=res_mode == 2)
         y = orc.epilogue(acc, exp2, div if per_channel else None, bias, resid if res_mode else None, act,
@@ -440,7 +443,7 @@ def test_specialised_epilogues(shape):
             want = y.astype(np.float16) if y_dtype == torch.float16 else y
             assert same_bits(want, out["y"].cpu().numpy()), row
         if q_bw:
-            assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10), out["q"].cpu().numpy()), row
+            assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10, q_scale), out["q"].cpu().numpy()), row
 
 
 @pytest.mark.parametrize("shape", [EPILOGUE_SHAPES[0], EPILOGUE_SHAPES[2], EPILOGUE_SHAPES[4]])
@@ -459,16 +462,19 @@ def test_relu_folded_into_requantization_handles_non_finite_values(shape, act):
     bias = r.standard_normal(co).astype(np.float32)
     bias[0], bias[1], bias[2] = np.nan, np.inf, -np.inf
     resid = r.standard_normal(acc.shape).astype(np.float32)
-    for q_pos, exp2, with_res in ((-3, -10, False), (-6, -10, False), (-4, -9, True)):
+    for q_pos, exp2, with_res, q_scale in ((-3, -10, False, 1.0), (-6, -10, False, 1.0), (-4, -9, True, 1.0),
+                                           (-3, -10, False, 1.37), (-4, -10, True, 1.77), (-5, -10, False, 1.12)):
         out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), (pad, pad), (1, 1), (1, 1), g, exp2=exp2, chan_div=cabi.dev(div),
                                bias=cabi.dev(bias), resid=cabi.dev(resid) if with_res else None, act=act, y_dtype=None,
-                               want_acc=False, q_bw=8, q_pos=q_pos, chan_rcp=cabi.dev(np.float32(1) / div))
+                               want_acc=False, q_bw=8, q_pos=q_pos, q_scale=q_scale,
+                               chan_rcp=cabi.dev(np.float32(1) / div))
         y = orc.epilogue(acc, exp2, div, bias, resid if with_res else None, act)
-        want = orc.quantize(y, 8, q_pos)
+        want = orc.quantize(y, 8, q_pos, q_scale)
         got = out["q"].cpu().numpy()
-        assert same_bits(want, got), (q_pos, exp2, with_res)
+        assert same_bits(want, got), (q_pos, exp2, with_res, q_scale)
         assert not got[..., 0].any() and not got[..., 2].any()
-        assert (got[..., 1] == min(127, int(6 * 2 ** -q_pos) if act == 2 else 127)).all()
+        six = np.rint(np.float32(6) * np.float32(q_scale) * np.float32(2.0 ** -q_pos))
+        assert (got[..., 1] == min(127, int(six) if act == 2 else 127)).all()
 
 
 SHORTCUT_CASES = [

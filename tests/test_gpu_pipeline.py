@@ -29,8 +29,8 @@ def np_sd(sd):
     return {k: v.detach().cpu().numpy() for k, v in sd.items()}
 
 
-def check_against_oracle(layers, sd, x, fused):
-    t, rec = netref.run(layers, np_sd(sd), x.numpy())
+def check_against_oracle(layers, sd, x, fused, fractional_scale=False):
+    t, rec = netref.run(layers, np_sd(sd), x.numpy(), fractional_scale=fractional_scale)
     trace = {}
     out = fused.forward(x.cuda(), trace=trace)
     torch.cuda.synchronize()
@@ -73,6 +73,38 @@ def test_resnet18_bs1(per_channel):
     sd = pipeline.calibrate(net, x, "int8", per_channel)
     fused = pipeline.FusedNet(layers, sd)
     check_against_oracle(layers, sd, x, fused)
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_resnet18_bs1_position_and_fractional_scale(per_channel):
+    """The same network quantized the general way: position from max-abs plus a fractional scale per tensor
+    (per output channel for per-axis weights), so that every step is absmax / qmax exactly."""
+    note("resnet18 fractional scale", per_channel)
+    layers = nets.resnet(18)
+    net = nets.FloatNet(layers, seed=0).eval()
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(1))
+    sd = pipeline.calibrate(net, x, "int8", per_channel)
+    fused = pipeline.FusedNet(layers, sd, fractional_scale=True)
+    assert 1.0 < fused.q["conv1"].scale_x < 2.0 and fused.shortcut_of
+    (logits,) = check_against_oracle(layers, sd, x, fused, fractional_scale=True)
+    # the fractional scale uses the whole integer range: the largest input value maps to +-127
+    trace = {}
+    fused.forward(x.cuda(), trace=trace)
+    assert int(trace["conv1"]["qx"].abs().max()) == 127
+    # and it is a different quantization from the power-of-two one
+    (pow2,) = check_against_oracle(layers, sd, x, pipeline.FusedNet(layers, sd))
+    assert not torch.equal(pow2, logits)
+    _, replay = fused.capture(x.cuda())
+    assert torch.equal(replay(), logits)
+
+
+def test_fractional_scale_rejects_position_checkpoints():
+    layers = nets.resnet(18)
+    net = nets.FloatNet(layers, seed=0).eval()
+    x = torch.randn(1, 3, 64, 64, generator=torch.Generator().manual_seed(1))
+    sd = pipeline.to_position_encoding(pipeline.calibrate(net, x, "int8", False), 8, 8)
+    with pytest.raises(ValueError, match="fractional"):
+        pipeline.FusedNet(layers, sd, fractional_scale=True)
 
 
 def test_resnet50_small_batch_and_graph_replay():

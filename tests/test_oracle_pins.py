@@ -408,3 +408,46 @@ def test_conv3d_vs_torch_float64(case, xbits):
     np.testing.assert_allclose(r["y"], want, rtol=1e-6, atol=1e-6)
     ref = F.conv3d(torch.from_numpy(x), torch.from_numpy(wt), torch.from_numpy(bias), stride, pad, dil, g).numpy()
     assert _rel_rms(ref, r["y"]) <= 0.03
+
+
+# ---------------------------------------------------------------- position + fractional scale per tensor / per axis
+@pytest.mark.parametrize("per_axis", [False, True])
+@pytest.mark.parametrize("bw", [8, 16])
+def test_decode_fractional_is_the_exact_step_quantization(per_axis, bw):
+    """decode_fractional restates setQuantizedParams / ...PerAxis (jit/utils/utils.cpp:81-167): what fixes it is
+    that position and fractional scale together give a step of absmax / qmax -- the extreme element maps to
+    +-qmax, every element is within half a step, and acc * 2^exp2 / div[c] is the real-valued product."""
+    qmax = 127.0 if bw == 8 else 32767.0
+    co = 6
+    w = (rng.standard_normal((co, 3, 3, 5)) * np.exp(rng.uniform(-3, 3, (co, 1, 1, 1)))).astype(np.float32)
+    x = (rng.standard_normal((2, 7, 7, 5)) * 3.7).astype(np.float32)
+    s_in = np.float32(qmax / np.abs(x).max())
+    if per_axis:
+        s_c = (qmax / np.abs(w).reshape(co, -1).max(1)).astype(np.float32)
+        q_scale, mode = np.concatenate(([s_in, 0.0], s_c)).astype(np.float32), (3 if bw == 8 else 4)
+    else:
+        s_c = np.full(co, qmax / np.abs(w).max(), np.float32)
+        q_scale, mode = np.array([s_in, s_c[0]], np.float32), (1 if bw == 8 else 2)
+    d = oops.decode_fractional(q_scale, [mode], co)
+    assert d["bw"] == bw and d["pos_c"].size == (co if per_axis else 1)
+    assert 1.0 <= d["scale_x"] < 2.0 + 1e-6 and ((1.0 <= d["scale_c"]) & (d["scale_c"] < 2.0 + 1e-6)).all()
+    qx = orc.quantize(x, bw, d["pos_x"], d["scale_x"])
+    qw = oops.quantize_weight_fractional(w, d)
+    assert np.abs(qx).max() == qmax
+    step_x = 1.0 / float(s_in)
+    assert np.abs(qx * step_x - x).max() <= 0.5 * step_x * (1 + 1e-4)
+    for c in range(co):
+        step = 1.0 / float(s_c[c])
+        if per_axis:
+            assert np.abs(qw[c]).max() == qmax
+        assert np.abs(qw[c] * step - w[c]).max() <= 0.5 * step * (1 + 1e-4)
+        # dequantization constant: 2^exp2 / div[c] = step_x * step_c
+        assert math.isclose(2.0 ** d["exp2"] / float(d["div"][c]), step_x * step, rel_tol=1e-5)
+    if not per_axis:
+        assert np.abs(qw).max() == qmax
+    # against the float convolution: finer than the power-of-two quantization of the same tensors can be
+    acc, _ = orc.conv2d_nhwc(qx, qw, (1, 1), (1, 1), (1, 1), 1)
+    y = orc.epilogue(acc, d["exp2"], d["div"], None, None, 0, np.float32)
+    ref = F.conv2d(torch.from_numpy(np.transpose(x, (0, 3, 1, 2)).astype(np.float64)),
+                   torch.from_numpy(np.transpose(w, (0, 3, 1, 2)).astype(np.float64)), None, 1, 1).numpy()
+    assert _rel_rms(np.transpose(ref, (0, 2, 3, 1)), y) <= (0.03 if bw == 8 else 2e-4)
