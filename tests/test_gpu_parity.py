@@ -175,6 +175,49 @@ def test_gemm_i8_acc_and_epilogue(m, n, k):
     assert same_bits(orc.quantize(y, 8, -2), out["q"].cpu().numpy())
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_gemm_random_sweep(seed):
+    """15 random products per seed over all three operand widths, ragged in every dimension (rows up to 7000 so that
+    the streaming kernel is drawn, K from 1), each with a random epilogue: bit-exact against the oracle."""
+    r = rng(2000 + seed)
+    for i in range(15):
+        bits = [(8, 8), (8, 8), (16, 8), (16, 16)][int(r.integers(0, 4))]
+        m = int(r.choice([r.integers(1, 70), r.integers(70, 700), r.integers(4000, 7000)]))
+        n = int(r.choice([r.integers(1, 40), r.integers(40, 400), 16 * r.integers(1, 11)]))
+        k = int(r.choice([r.integers(1, 100), r.integers(100, 900), 16 * r.integers(1, 7)]))
+        a, b = _ints(r, (m, k), bits[0]), _ints(r, (n, k), bits[1])
+        use_div, use_rcp, use_bias = r.random() < 0.6, r.random() < 0.7, r.random() < 0.7
+        act = int(r.integers(0, 3))
+        y_dtype = [None, torch.float32, torch.float32, torch.float16][int(r.integers(0, 4))]
+        q_bw = int(r.choice([0, 8, 8, 16]))
+        want_acc = bits != (16, 16) and r.random() < 0.3
+        if y_dtype is None and not q_bw and not want_acc:
+            y_dtype = torch.float32
+        q_scale = 1.0 if r.random() < 0.5 else float(np.float32(r.uniform(1.0, 2.0)))
+        exp2 = {(8, 8): -10, (16, 8): -18, (16, 16): -26}[bits] + int(r.integers(-2, 3))
+        q_pos = int(r.integers(-5, 0)) if q_bw == 8 else int(r.integers(-12, -6))
+        case = dict(seed=seed, i=i, mnk=(m, n, k), bits=bits, route=cabi.lib().catchq_gemm_route(bits[0], bits[1], m, n, k),
+                    div=use_div, rcp=use_rcp, bias=use_bias, act=act, y=y_dtype, q_bw=q_bw, q_scale=q_scale, q_pos=q_pos,
+                    exp2=exp2, acc=want_acc)
+        note("gemm sweep", case)
+        acc, ovf = orc.gemm_nt(a, b)
+        div = r.uniform(0.6, 3.5, n).astype(np.float32) if use_div else None
+        bias = r.standard_normal(n).astype(np.float32) if use_bias else None
+        out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=exp2, chan_div=cabi.dev(div) if use_div else None,
+                           bias=cabi.dev(bias) if use_bias else None, act=act, y_dtype=y_dtype, want_acc=want_acc,
+                           q_bw=q_bw, q_pos=q_pos, q_scale=q_scale,
+                           chan_rcp=cabi.dev(np.float32(1) / div) if use_div and use_rcp else None)
+        torch.cuda.synchronize()
+        y = orc.epilogue(acc, exp2, div, bias, None, act)
+        if want_acc:
+            assert ovf == 0 and same_bits(acc.astype(np.int32), out["acc"].cpu().numpy()), case
+        if y_dtype is not None:
+            want = y.astype(np.float16) if y_dtype == torch.float16 else y
+            assert same_bits(want, out["y"].cpu().numpy()), case
+        if q_bw:
+            assert same_bits(orc.quantize(y, q_bw, q_pos, q_scale), out["q"].cpu().numpy()), case
+
+
 def test_division_by_reciprocal_is_exact():
     """v/d evaluated as q=v*r, e=fma(-q,d,v), fma(e,r,q) with r = RN(1/d) must equal IEEE division bit
     for bit: adversarial divisor significands x a wide set of dividends x several exponents."""
@@ -444,6 +487,83 @@ def test_specialised_epilogues(shape, q_scale):
             assert same_bits(want, out["y"].cpu().numpy()), row
         if q_bw:
             assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10, q_scale), out["q"].cpu().numpy()), row
+
+
+def _random_conv_case(r):
+    """a convolution problem drawn so that every kernel family turns up: few / odd / multiple-of-16 channel
+    counts, depthwise and grouped, 1x1 to 7x7 filters, strides, dilations, padding"""
+    kh, kw = (int(v) for v in r.choice([1, 1, 2, 3, 3, 5, 7], 2))
+    if r.random() < 0.6:
+        kw = kh
+    dil = (int(r.choice([1, 1, 1, 2])), int(r.choice([1, 1, 1, 2])))
+    stride = (int(r.choice([1, 1, 2, 3])), int(r.choice([1, 1, 2, 3])))
+    pad = (int(r.integers(0, kh // 2 + 2)), int(r.integers(0, kw // 2 + 2)))
+    h = int(r.integers(max(1, dil[0] * (kh - 1) + 1 - 2 * pad[0]), 40))
+    w = int(r.integers(max(1, dil[1] * (kw - 1) + 1 - 2 * pad[1]), 40))
+    kind = r.choice(["dense", "dense", "dense", "depthwise", "grouped", "pointwise_long"])
+    ci = int(r.choice([1, 3, 4, 8, 16, 16, 24, 32, 32, 48, 64, 96, 130, 256]))
+    co = int(r.choice([1, 4, 5, 8, 16, 24, 32, 36, 64, 64, 100, 128, 160, 255]))
+    g = 1
+    if kind == "depthwise":
+        ci = co = g = int(r.choice([4, 6, 8, 16, 24, 32, 96]))
+    elif kind == "grouped":
+        g = int(r.choice([2, 4]))
+        ci, co = g * int(r.choice([1, 3, 4, 8])), g * int(r.choice([1, 2, 4, 6]))
+    elif kind == "pointwise_long":  # many pixels, short K: the streaming kernels' territory
+        kh = kw = 1
+        pad, dil = (0, 0), (1, 1)
+        h, w = int(r.integers(40, 90)), int(r.integers(40, 90))
+        ci, co = int(r.choice([16, 32, 48, 64, 96])), int(r.choice([16, 24, 32, 64, 96, 144, 160]))
+    n = int(r.integers(1, 4))
+    bits = [(8, 8), (8, 8), (16, 8), (16, 16)][int(r.integers(0, 4))]
+    return n, ci, h, w, co, kh, kw, pad, stride, dil, g, bits
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_conv_random_sweep(seed):
+    """20 random problems per seed, each with a random epilogue (divisor in reciprocal or true-division form, bias,
+    residual before / after the activation, all four activations, fp32 / fp16 / no float output, int8 / int16 / no
+    requantization at unit and fractional scale, integer sums): everything bit-exact against the oracle."""
+    r = rng(1000 + seed)
+    for i in range(20):
+        n, ci, h, w, co, kh, kw, pad, stride, dil, g, bits = _random_conv_case(r)
+        route = cabi.conv_route(bits[0], bits[1], (n, h, w, ci), (co, kh, kw, ci // g), pad, stride, dil, g)
+        x, wt = _ints(r, (n, h, w, ci), bits[0]), _ints(r, (co, kh, kw, ci // g), bits[1])
+        use_div, use_rcp = r.random() < 0.6, r.random() < 0.7
+        use_bias, res_mode = r.random() < 0.7, int(r.choice([0, 0, 1, 2]))
+        act = int(r.integers(0, 4))
+        y_dtype = [None, torch.float32, torch.float32, torch.float16][int(r.integers(0, 4))]
+        q_bw = int(r.choice([0, 8, 8, 16]))
+        want_acc = bits != (16, 16) and r.random() < 0.3
+        if y_dtype is None and not q_bw and not want_acc:
+            y_dtype = torch.float32
+        q_scale = 1.0 if r.random() < 0.5 else float(np.float32(r.uniform(1.0, 2.0)))
+        exp2 = {(8, 8): -10, (16, 8): -18, (16, 16): -26}[bits] + int(r.integers(-2, 3))
+        q_pos = int(r.integers(-5, 0)) if q_bw == 8 else int(r.integers(-12, -6))
+        case = dict(seed=seed, i=i, shape=(n, ci, h, w, co, kh, kw), pad=pad, stride=stride, dil=dil, groups=g, bits=bits,
+                    route=route, div=use_div, rcp=use_rcp, bias=use_bias, res=res_mode, act=act, y=y_dtype, q_bw=q_bw,
+                    q_scale=q_scale, q_pos=q_pos, exp2=exp2, acc=want_acc)
+        note("sweep", case)
+        acc, ovf = orc.conv2d_nhwc(x, wt, pad, stride, dil, g)
+        assert acc.size > 0
+        div = r.uniform(0.6, 3.5, co).astype(np.float32) if use_div else None
+        bias = r.standard_normal(co).astype(np.float32) if use_bias else None
+        resid = r.standard_normal(acc.shape).astype(np.float32) if res_mode else None
+        out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), pad, stride, dil, g, exp2=exp2,
+                               chan_div=cabi.dev(div) if use_div else None, bias=cabi.dev(bias) if use_bias else None,
+                               resid=cabi.dev(resid) if res_mode else None, act=act, y_dtype=y_dtype, want_acc=want_acc,
+                               q_bw=q_bw, q_pos=q_pos, q_scale=q_scale,
+                               chan_rcp=cabi.dev(np.float32(1) / div) if use_div and use_rcp else None, act_slope=0.1,
+                               resid_after_act=res_mode == 2)
+        torch.cuda.synchronize()
+        y = orc.epilogue(acc, exp2, div, bias, resid, act, act_slope=0.1, resid_after_act=res_mode == 2)
+        if want_acc:
+            assert ovf == 0 and same_bits(acc.astype(np.int32), out["acc"].cpu().numpy()), case
+        if y_dtype is not None:
+            want = y.astype(np.float16) if y_dtype == torch.float16 else y
+            assert same_bits(want, out["y"].cpu().numpy()), case
+        if q_bw:
+            assert same_bits(orc.quantize(y, q_bw, q_pos, q_scale), out["q"].cpu().numpy()), case
 
 
 @pytest.mark.parametrize("shape", [EPILOGUE_SHAPES[0], EPILOGUE_SHAPES[2], EPILOGUE_SHAPES[4]])
