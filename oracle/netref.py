@@ -60,7 +60,7 @@ def run(layers, sd, x_nchw, record=True, fractional_scale=False):
             y = epilogue(acc, d["pos_x"] + d["pos_w"], d["new_scale"], b, resid, _ACT[l.act], act_slope=LEAKY_SLOPE,
                          resid_after_act=bool(l.add_after))
             if record:
-                rec[l.name] = dict(qx=qx, acc=acc, y=y, overflow=ovf, pos_x=d["pos_x"], pos_w=d["pos_w"])
+                rec[l.name] = dict(qx=qx, qw=qw, acc=acc, y=y, overflow=ovf, pos_x=d["pos_x"], pos_w=d["pos_w"])
             t[l.name] = y
         elif l.kind == "maxpool":
             t[l.name] = maxpool_nhwc(t[l.src], l.k, l.stride, l.pad)

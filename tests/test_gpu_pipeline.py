@@ -46,6 +46,11 @@ def check_against_oracle(layers, sd, x, fused, fractional_scale=False):
                 t = t[..., :want.shape[-1]]
             return t.reshape(want.shape)
         assert np.array_equal(r["qx"], real(g["qx"], r["qx"])), "quantized input of " + l.name
+        # the quantized weight as the plan holds it: the oracle's, plus zero padding (channels, taps of the stem's rows)
+        qw = fused.q[l.name].qw.cpu().numpy()
+        inner = tuple(slice(0, e) for e in r["qw"].shape)
+        assert qw.dtype == r["qw"].dtype and np.array_equal(qw[inner], r["qw"]), "quantized weight of " + l.name
+        assert np.count_nonzero(qw) == np.count_nonzero(r["qw"]), "weight padding of %s is not zero" % l.name
         assert np.array_equal(r["acc"].astype(np.int32), real(g["acc"], r["acc"])), "accumulators of " + l.name
         assert np.array_equal(r["y"], real(g["y"].float(), r["y"])), "output of " + l.name
     outs = out if isinstance(out, tuple) else (out,)
