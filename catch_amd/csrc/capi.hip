@@ -98,7 +98,7 @@ CATCHQ_API int catchq_gemm_nt(const void *a, int a_bits, const void *b, int b_bi
   if (st != CATCHQ_OK) return st;
   if (m == 0 || n == 0) return CATCHQ_OK;
   if (k > 0 && (!a || !b)) return CATCHQ_ERR_ARG;
-  const EpiDev e = make_epi(epilogue);
+  const EpiDev e = make_epi(epilogue, m * n);
   hipStream_t s = as_stream(stream);
   const Route route = gemm_route(a_bits, b_bits, m, n, k, a, b);
   if (route == kMfma) return gemm_nt_mfma_i8(a, b, m, n, k, e, s);
@@ -120,7 +120,7 @@ CATCHQ_API int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int 
   if (st != CATCHQ_OK) return st;
   if (desc->n == 0) return CATCHQ_OK;
   if (!x || !w) return CATCHQ_ERR_ARG;
-  const EpiDev e = make_epi(epilogue);
+  const EpiDev e = make_epi(epilogue, (int64_t)desc->n * ho * wo * desc->co);
   hipStream_t s = as_stream(stream);
   const catchq_conv_desc_t &d = *desc;
   switch (conv_route(x_bits, w_bits, desc, x, w)) {
@@ -192,7 +192,7 @@ CATCHQ_API int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void
   const catchq_conv_desc_t &d = *desc;
   const catchq_shortcut_t &sc = *shortcut;
   if (shortcut_fusable(x_bits, w_bits, desc, shortcut) && !epilogue->exp2_dev[0] && !epilogue->exp2_dev[1]) {
-    EpiDev e = make_epi(epilogue);
+    EpiDev e = make_epi(epilogue, (int64_t)d.n * ho * wo * d.co);
     e.resid_after = epilogue->resid_after_act ? 1 : 0;
     ShortcutDev sd;
     sd.exp2 = sc.exp2;

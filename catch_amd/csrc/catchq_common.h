@@ -94,6 +94,9 @@ struct EpiDev {
   float act_slope;
   int resid_after;
   const int *exp2_a, *exp2_b;  // device-resident positions added to exp2 (resolve_exp2)
+  // the floating output / the residual is too large to stay cached until it is next used: written / read with
+  // the non-temporal hint so that it does not push the operands and the int8 output out of the caches
+  int y_stream, resid_stream;
 };
 
 // The second operand pair of a two-branch launch: the projection shortcut of a residual block.  Its
@@ -104,8 +107,12 @@ struct ShortcutDev {
   const float *chan_div, *chan_rcp, *bias;
 };
 
-inline EpiDev make_epi(const catchq_epilogue_t *e) {
+// out_elems: elements of the output tensor (0: unknown, nothing is streamed)
+inline EpiDev make_epi(const catchq_epilogue_t *e, int64_t out_elems = 0) {
   EpiDev d;
+  constexpr int64_t kStreamBytes = 64ll << 20;  // a quarter of the 256 MB last-level cache
+  d.y_stream = (e->y && out_elems * (e->y_dtype == CATCHQ_F16 ? 2 : 4) >= kStreamBytes) ? 1 : 0;
+  d.resid_stream = (e->resid && out_elems * 4 >= kStreamBytes) ? 1 : 0;
   d.exp2 = e->exp2;
   d.chan_div = e->chan_div;
   const bool dev_exp = e->exp2_dev[0] || e->exp2_dev[1];

@@ -189,6 +189,31 @@ struct EpiAtSplit {
   template <class T> __device__ __forceinline__ T *at(T *base) const { return (base + uni) + off; }
 };
 
+// A store / load with or without the non-temporal hint, chosen by a wave-uniform flag.  The empty volatile
+// statements keep the two branches apart: merged into one access, they would lose the hint.
+template <class T>
+__device__ __forceinline__ void store_stream(T *dst, const T v, bool stream) {
+  if (stream) {
+    asm volatile("");
+    __builtin_nontemporal_store(v, dst);
+    asm volatile("");
+  } else {
+    *dst = v;
+  }
+}
+template <class T>
+__device__ __forceinline__ T load_stream(const T *src, bool stream) {
+  T v;
+  if (stream) {
+    asm volatile("");
+    v = __builtin_nontemporal_load(src);
+    asm volatile("");
+  } else {
+    v = *src;
+  }
+  return v;
+}
+
 // four integer sums of one pixel (channels n..n+3 at `where`) -> all requested outputs
 template <class S, class At>
 __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLane &L, const At where, const EpiDev &e) {
@@ -209,10 +234,11 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
   if (S::y16(e)) {
     __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
                     __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
-    *reinterpret_cast<v2i *>(where.at(reinterpret_cast<__half *>(e.y))) = *reinterpret_cast<v2i *>(h);
+    store_stream(reinterpret_cast<v2i *>(where.at(reinterpret_cast<__half *>(e.y))), *reinterpret_cast<v2i *>(h),
+                 e.y_stream != 0);
   } else if (S::y32(e)) {
     v4f o = {v[0], v[1], v[2], v[3]};
-    *reinterpret_cast<v4f *>(where.at(reinterpret_cast<float *>(e.y))) = o;
+    store_stream(reinterpret_cast<v4f *>(where.at(reinterpret_cast<float *>(e.y))), o, e.y_stream != 0);
   }
   if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
     // values are >= 0 and never NaN here (or, with the activation folded in, are made so by the median:
@@ -315,7 +341,7 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
         for (int it = 0; it < NIT; ++it) {
           resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
           if (FULL || (n_ok && it * RPI + rsub < rows))
-            resv[it] = *reinterpret_cast<const v4f *>((e.resid + uni) + (lane_off + it * it_step));
+            resv[it] = load_stream(reinterpret_cast<const v4f *>((e.resid + uni) + (lane_off + it * it_step)), e.resid_stream != 0);
         }
       }
       // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
