@@ -111,11 +111,12 @@ template <> struct EpiOf<EPI_LK_Y_Q16> { typedef EpiSpec<0, 1, 0, CATCHQ_ACT_LEA
 template <> struct EpiOf<EPI_LK_RESA_Q16> { typedef EpiSpec<0, 1, 2, CATCHQ_ACT_LEAKY, 0, 16, 0> type; };
 template <> struct EpiOf<EPI_LK_RESA_Y_Q16> { typedef EpiSpec<0, 1, 2, CATCHQ_ACT_LEAKY, 1, 16, 0> type; };
 
-// which variant serves this launch; a kernel family that has no instance of the variant returned uses
-// the generic EPI_VECTOR
+// which variant serves this launch (the specialised ones also need a unit requantization scale: a
+// fractional one costs them 2-4 % end to end even when it is not used, measured); a kernel family
+// that has no instance of the variant returned uses the generic EPI_VECTOR
 inline int pick_epilogue(int N, const EpiDev &e) {
   if (!vec_epilogue_ok(N, e)) return EPI_SCALAR;
-  if (e.acc_out || (e.chan_div && !e.chan_rcp)) return EPI_VECTOR;
+  if (e.acc_out || (e.q && e.q_scale != 1.0f) || (e.chan_div && !e.chan_rcp)) return EPI_VECTOR;
   const int div = e.chan_rcp ? 1 : 0, bias = e.bias ? 1 : 0;
   const int res = !e.resid ? 0 : (e.resid_after ? 2 : 1);
   const int ym = !e.y ? 0 : (e.y_f16 ? 2 : 1);
@@ -147,7 +148,7 @@ __device__ __forceinline__ EpiLane epi_lane_setup(int n, bool n_ok, const EpiDev
   L.use_rcp = S::rcp(e); L.use_div = S::truediv(e); L.use_bias = S::bias(e); L.use_res = S::resid(e);
   L.res_after = S::resid_after(e);
   L.act = S::act(e);
-  L.unit_q = e.q_scale == 1.0f;
+  L.unit_q = S::kGeneric ? (e.q_scale == 1.0f) : true;
   // Reciprocal form with the power of two folded in:
   //   v = (f*2^e)/d  ==  q = f*(r*2^e); err = fma(-q, d*2^-e, f); fma(err, r*2^e, q)
   // (scaling by 2^e is exact, so every intermediate is the scaled image of the unfolded one)
@@ -242,24 +243,15 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
   }
   if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
     // values are >= 0 and never NaN here (or, with the activation folded in, are made so by the median:
-    // for a NaN operand it returns the smallest of the other two, 0, which is what ReLU makes of a NaN).
-    // With s the requantization scale and x = fl(v * s) (a wave-uniform branch skips the multiply for s = 1):
+    // for a NaN operand it returns the smallest of the other two, 0, which is what ReLU makes of a NaN);
+    // the requantization scale is 1:
     //   sat(rne(x * 2^-pos)) = low byte of the float  fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23)
     // (the product is exact, so the fma rounds once, to an integer, ties to even; clamping before
-    // the rounding equals clamping after it because the bound is an integer multiple of 2^pos).  A folded
-    // activation commutes with the multiply, which is monotonic and keeps zero and the sign:
-    // fl(max(v, 0) * s) = max(fl(v * s), 0) and fl(min(v, 6) * s) = min(fl(v * s), fl(6 * s)), so the
-    // ReLU6 bound joins the clamp: min(min(x, fl(6 s)), hi) = min(x, min(fl(6 s), hi)).
+    // the rounding equals clamping after it because the bound is an integer multiple of 2^pos; a ReLU6
+    // bound of 6 below that one takes its place: min(min(x, 6), hi) = min(x, min(6, hi)))
     float hi = __builtin_ldexpf(127.0f, -e.q_neg_pos);
     const float sc = __builtin_ldexpf(1.0f, e.q_neg_pos);
-    if constexpr (S::kFoldAct && S::kAct == CATCHQ_ACT_RELU6) {
-      const float six = 6.0f * e.q_scale;
-      hi = (hi < six) ? hi : six;
-    }
-    if (!L.unit_q) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) v[t] = v[t] * e.q_scale;
-    }
+    if constexpr (S::kFoldAct && S::kAct == CATCHQ_ACT_RELU6) hi = (hi < 6.0f) ? hi : 6.0f;
     unsigned b[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
