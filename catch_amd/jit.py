@@ -219,9 +219,13 @@ def graph_to_layers(graph):
     return layers, sd, outs
 
 
-def lower(module, example_input, device="cuda", out_half=False):
+def lower(module, example_input, device="cuda", out_half=False, fractional_scale=False):
     """module: an nn.Module whose quantized layers call torch_mlu::conv2d / linear (as prepared by
     ``quantize_dynamic_mlu`` and moved to the device), or an already traced ScriptModule.
+    fractional_scale: give every tensor (every output channel of per-axis weights) position *and*
+    fractional scale, the form in which the reference's converters hand the ranges to their backend
+    (setQuantizedParams / setQuantizedParamsPerAxis, torch_mlu/csrc/jit/utils/utils.cpp:81-167);
+    the default keeps the eager ops' power-of-two steps, so that the plan equals the traced module.
     Returns (FusedNet, layers).  The FusedNet's outputs come in the order of the traced outputs."""
     if not isinstance(module, torch.jit.ScriptModule):
         with torch.no_grad():
@@ -229,7 +233,7 @@ def lower(module, example_input, device="cuda", out_half=False):
     frozen = torch.jit.freeze(module.eval())
     graph = frozen.inlined_graph
     layers, sd, outs = graph_to_layers(graph)
-    fused = FusedNet(layers, sd, device=device, out_half=out_half)
+    fused = FusedNet(layers, sd, device=device, out_half=out_half, fractional_scale=fractional_scale)
     if list(fused.outputs) != outs:
         if sorted(fused.outputs) != sorted(outs):
             raise LoweringError("graph outputs %s do not match the plan's terminal tensors %s" % (outs, fused.outputs))

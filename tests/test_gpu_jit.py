@@ -31,6 +31,29 @@ def dropin_model(layers, x, seed, weight_std, per_channel=True):
     return net, qnet.to("cuda").eval()
 
 
+def test_lowering_with_fractional_scales():
+    """the converters' general form (position + fractional scale per tensor / per axis): the lowered plan equals
+    the plan built directly from the checkpoint in that mode, and over the 21 int8 layers of the network it stays
+    closer to the float result than the power-of-two plan (relative RMS, the reference's own error measure,
+    test/common_utils.py:514-522 there)"""
+    note("jit lowering, fractional scales")
+    layers = nets.NETS["resnet18"]()
+    x = torch.rand(2, 3, 64, 64, generator=torch.Generator().manual_seed(3))
+    net, qnet = dropin_model(layers, x, 9, 0.05)
+    fused, _ = jit.lower(qnet, x.cuda(), fractional_scale=True)
+    pow2, _ = jit.lower(qnet, x.cuda())
+    direct = pipeline.FusedNet(layers, pipeline.calibrate(net, x, "int8", True), fractional_scale=True)
+    got = fused.forward(x.cuda())
+    assert torch.equal(got, direct.forward(x.cuda()))
+    ref = net(x).cuda()
+
+    def rel_rms(a, b):
+        return ((a - b).pow(2).sum().sqrt() / b.pow(2).sum().sqrt()).item()
+    e_frac, e_pow2 = rel_rms(got, ref), rel_rms(pow2.forward(x.cuda()), ref)
+    note("relative RMS vs float: fractional %.4f, power of two %.4f" % (e_frac, e_pow2))
+    assert e_frac < e_pow2 <= 0.05
+
+
 @pytest.mark.parametrize("arch,size,std", [("resnet18", 64, 0.05), ("mobilenet_v2", 64, 0.2),
                                            ("darknet53_yolov3", 64, "he")])
 def test_lowered_trace_equals_direct_plan(arch, size, std):
