@@ -28,6 +28,11 @@
  *   NaN -> 0 in quantize      PARITY UNPINNED (vendor behaviour not stated anywhere)
  *   float order of dequant+bias inside the vendor conv/matmul: PARITY UNPINNED;
  *                             fixed here as cvt(acc) * 2^e [/ new_scale_c] [+ bias] in fp32.
+ *   position + fractional scale per tensor / per axis (oracle/ops.py decode_fractional, the
+ *                             composition of orc_quant_params and orc_quantize_* with scale != 1):
+ *                             parameters pinned (the step is absmax/qmax: extreme element -> +-qmax,
+ *                             error <= half a step); what the reference's graph backend computes
+ *                             from them is in a closed library: PARITY UNPINNED.
  */
 #include <math.h>
 #include <stdint.h>

@@ -45,7 +45,10 @@ def decode_fractional(q_scale, q_mode, co):
     step is absmax / qmax rather than a power of two.
     -> dict(bw, pos_x, scale_x, pos_c[], scale_c[], exp2, div[co]): a weight of channel c is
     q * 2^pos_c / scale_c; with P = max pos_c, an integer sum dequantizes as
-    acc * 2^(pos_x + P) / div[c], div[c] = fp32(scale_x * scale_c * 2^(P - pos_c))."""
+    acc * 2^(pos_x + P) / div[c], div[c] = fp32(scale_x * scale_c * 2^(P - pos_c)).
+    Parity unpinned beyond the parameters themselves: what the reference's graph backend computes from
+    them bit by bit is inside a closed library; this applies the eager quantizer's stated formula
+    q = sat(rne(x * scale * 2^-position)) with scale != 1 and the eager epilogue's order of operations."""
     q_scale = np.asarray(q_scale, dtype=np.float32).reshape(-1)
     mode = int(np.asarray(q_mode).reshape(-1)[0])
     bw = 8 if mode in (1, 3) else 16
