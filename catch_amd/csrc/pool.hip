@@ -22,8 +22,11 @@ struct Lowest<float> {
   static __device__ float value() { return -__builtin_inff(); }
 };
 
-// one thread = one output pixel x VEC consecutive channels (VEC * sizeof(T) = 16 bytes, or VEC = 1)
-template <typename T, int VEC>
+// one thread = one output pixel x VEC consecutive channels (VEC * sizeof(T) = 16 bytes, or VEC = 1).
+// K > 0: the window size is known, every load of the window is requested before the first comparison
+// (taps outside the image read the centre tap again, which is always inside and changes nothing);
+// K = 0: any window, tap by tap.
+template <typename T, int VEC, int K>
 __global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const T *__restrict__ x, T *__restrict__ y, int N, int H,
                                                           int W, int C, int k, int stride, int pad, int Ho,
                                                           int Wo) {
@@ -40,18 +43,48 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const T *__restrict__
     T m[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) m[j] = Lowest<T>::value();
-    for (int r = 0; r < k; ++r) {
-      const int hi = ho * stride - pad + r;
-      if ((unsigned)hi >= (unsigned)H) continue;
-      for (int q = 0; q < k; ++q) {
-        const int wi = wo * stride - pad + q;
-        if ((unsigned)wi >= (unsigned)W) continue;
-        const T *src = x + (((int64_t)n * H + hi) * W + wi) * C + c;
-        T v[VEC];
-        if constexpr (VEC == 1) v[0] = src[0];
-        else *reinterpret_cast<v4i *>(v) = *reinterpret_cast<const v4i *>(src);
+    const T *img = x + (int64_t)n * H * W * C + c;
+    if constexpr (K > 0) {
+      // a window of K x K with pad <= K/2 always contains the pixel (ho*stride, wo*stride) clamped into the image
+      const int hc = min(ho * stride, H - 1), wc = min(wo * stride, W - 1);
+      v4i raw[K * K];
+      T one[K * K];
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) m[j] = (v[j] > m[j]) ? v[j] : m[j];
+      for (int r = 0; r < K; ++r)
+#pragma unroll
+        for (int q = 0; q < K; ++q) {
+          int hi = ho * stride - pad + r, wi = wo * stride - pad + q;
+          const bool in = (unsigned)hi < (unsigned)H && (unsigned)wi < (unsigned)W;
+          hi = in ? hi : hc;
+          wi = in ? wi : wc;
+          const T *src = img + ((int64_t)hi * W + wi) * C;
+          if constexpr (VEC == 1) one[r * K + q] = src[0];
+          else raw[r * K + q] = *reinterpret_cast<const v4i *>(src);
+        }
+#pragma unroll
+      for (int t = 0; t < K * K; ++t) {
+        if constexpr (VEC == 1) m[0] = (one[t] > m[0]) ? one[t] : m[0];
+        else {
+          T v[VEC];
+          *reinterpret_cast<v4i *>(v) = raw[t];
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) m[j] = (v[j] > m[j]) ? v[j] : m[j];
+        }
+      }
+    } else {
+      for (int r = 0; r < k; ++r) {
+        const int hi = ho * stride - pad + r;
+        if ((unsigned)hi >= (unsigned)H) continue;
+        for (int q = 0; q < k; ++q) {
+          const int wi = wo * stride - pad + q;
+          if ((unsigned)wi >= (unsigned)W) continue;
+          const T *src = img + ((int64_t)hi * W + wi) * C;
+          T v[VEC];
+          if constexpr (VEC == 1) v[0] = src[0];
+          else *reinterpret_cast<v4i *>(v) = *reinterpret_cast<const v4i *>(src);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) m[j] = (v[j] > m[j]) ? v[j] : m[j];
+        }
       }
     }
     T *dst = y + (((int64_t)n * Ho + ho) * Wo + wo) * C + c;
@@ -69,10 +102,16 @@ static int launch_maxpool(const void *x, void *y, int N, int H, int W, int C, in
   int64_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   if (blocks < 1) blocks = 1;
-  if (vec)
-    maxpool_nhwc_kernel<T, VEC><<<(int)blocks, 256, 0, s>>>((const T *)x, (T *)y, N, H, W, C, k, stride, pad, Ho, Wo);
-  else
-    maxpool_nhwc_kernel<T, 1><<<(int)blocks, 256, 0, s>>>((const T *)x, (T *)y, N, H, W, C, k, stride, pad, Ho, Wo);
+#define CATCHQ_POOL(V, K) \
+  maxpool_nhwc_kernel<T, V, K><<<(int)blocks, 256, 0, s>>>((const T *)x, (T *)y, N, H, W, C, k, stride, pad, Ho, Wo)
+  // the unrolled windows rely on the clamped corner pixel lying inside the window: pad <= k/2 and a window
+  // that starts inside the image
+  const bool corner_ok = 2 * pad <= k && (int64_t)(Ho - 1) * stride - pad < H && (int64_t)(Wo - 1) * stride - pad < W;
+  if (vec && k == 3 && corner_ok) CATCHQ_POOL(VEC, 3);
+  else if (vec && k == 2 && corner_ok) CATCHQ_POOL(VEC, 2);
+  else if (vec) CATCHQ_POOL(VEC, 0);
+  else CATCHQ_POOL(1, 0);
+#undef CATCHQ_POOL
   return launch_status();
 }
 

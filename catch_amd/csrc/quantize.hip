@@ -158,28 +158,43 @@ __global__ __launch_bounds__(kThreads) void quantize_nchw_nhwc_frame_kernel(cons
                                                                            int n, int c, int h, int w, int oh, int ow,
                                                                            int top, int left, int pos, float scale) {
   typedef typename QRange<BW>::type TQ;
-  // blockIdx.y walks the output rows (image, oy), threads the pixels of a row: the row's coordinates are
-  // scalar arithmetic, a pixel costs no division
+  // A block is 64 lanes along a row x 4 rows; a lane owns PX pixels of its row, 64 apart (so that every load
+  // and store instruction of the wave covers consecutive pixels), all of whose loads (PX pixels x c channel
+  // planes) are requested before the first conversion.  The rows' coordinates are computed once per row: a
+  // pixel costs no division.
+  constexpr int PX = 4;
   const int64_t hw = (int64_t)h * w, rows = (int64_t)n * oh;
-  for (int64_t row = blockIdx.y; row < rows; row += gridDim.y) {
+  const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
+  for (int64_t row = (int64_t)blockIdx.y * 4 + ly; row < rows; row += (int64_t)gridDim.y * 4) {
     const int64_t img = row / oh;
     const int oy = (int)(row - img * oh), iy = oy - top;
     const bool row_inside = (unsigned)iy < (unsigned)h;
     const TIn *src = x + img * c * hw + (int64_t)iy * w;
     TQ *dst = q + row * ow * CPAD;
-    for (int ox = blockIdx.x * kThreads + threadIdx.x; ox < ow; ox += gridDim.x * kThreads) {
-      const int ix = ox - left;
-      const bool inside = row_inside && (unsigned)ix < (unsigned)w;
-      TQ out[CPAD];
+    for (int ox0 = blockIdx.x * 64 * PX + lx; ox0 < ow; ox0 += gridDim.x * 64 * PX) {
+      float v[PX][CPAD];
 #pragma unroll
-      for (int ch = 0; ch < CPAD; ++ch) {
-        out[ch] = 0;
-        if (inside && ch < c) out[ch] = (TQ)quant1<BW>(ld_f(src, ch * hw + ix), scale, -pos);
+      for (int px = 0; px < PX; ++px) {
+        const int ix = ox0 + px * 64 - left;
+        const bool inside = row_inside && (unsigned)ix < (unsigned)w;
+#pragma unroll
+        for (int ch = 0; ch < CPAD; ++ch) {
+          v[px][ch] = 0.0f;
+          if (inside && ch < c) v[px][ch] = ld_f(src, ch * hw + ix);
+        }
       }
-      constexpr int BYTES = CPAD * sizeof(TQ);
-      if constexpr (BYTES == 4) *reinterpret_cast<int *>(dst + ox * CPAD) = *reinterpret_cast<int *>(out);
-      else if constexpr (BYTES == 8) *reinterpret_cast<v2i *>(dst + ox * CPAD) = *reinterpret_cast<v2i *>(out);
-      else *reinterpret_cast<v4i *>(dst + ox * CPAD) = *reinterpret_cast<v4i *>(out);
+#pragma unroll
+      for (int px = 0; px < PX; ++px) {
+        if (ox0 + px * 64 >= ow) break;
+        TQ out[CPAD];
+#pragma unroll
+        for (int ch = 0; ch < CPAD; ++ch) out[ch] = (TQ)quant1<BW>(v[px][ch], scale, -pos);  // 0 -> 0
+        constexpr int BYTES = CPAD * sizeof(TQ);
+        TQ *o = dst + (ox0 + px * 64) * CPAD;
+        if constexpr (BYTES == 4) *reinterpret_cast<int *>(o) = *reinterpret_cast<int *>(out);
+        else if constexpr (BYTES == 8) *reinterpret_cast<v2i *>(o) = *reinterpret_cast<v2i *>(out);
+        else *reinterpret_cast<v4i *>(o) = *reinterpret_cast<v4i *>(out);
+      }
     }
   }
 }
@@ -377,7 +392,8 @@ static int launch_frame(const void *x, void *q, int n, int c, int h, int w, int 
                         float scale, hipStream_t s) {
   typedef typename QRange<BW>::type TQ;
   const int64_t rows = (int64_t)n * oh;
-  const dim3 grid((unsigned)((ow + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+  const int64_t row_groups = (rows + 3) / 4;  // a block takes 4 rows x 256 pixels
+  const dim3 grid((unsigned)((ow + 255) / 256), (unsigned)(row_groups < 65535 ? row_groups : 65535));
   quantize_nchw_nhwc_frame_kernel<TIn, BW, CPAD><<<grid, kThreads, 0, s>>>((const TIn *)x, (TQ *)q, n, c, h, w, oh, ow,
                                                                           top, left, pos, scale);
   return launch_status();
