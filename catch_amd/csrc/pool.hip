@@ -61,6 +61,28 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_kernel(const T *__restrict__
           if constexpr (VEC == 1) one[r * K + q] = src[0];
           else raw[r * K + q] = *reinterpret_cast<const v4i *>(src);
         }
+      if constexpr (VEC == 16) {
+        // sixteen int8 per tap, four to a dword: flipping the sign bits turns the signed order into the unsigned
+        // one, and the even / odd bytes of a dword, each alone in a 16-bit half, compare as 16-bit unsigned
+        // numbers -- two packed 16-bit maxima per dword instead of four extract-and-compare pairs
+        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+        u16x2 even[4], odd[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) even[d] = odd[d] = u16x2{0, 0};
+#pragma unroll
+        for (int t = 0; t < K * K; ++t)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const unsigned u = (unsigned)raw[t][d] ^ 0x80808080u;
+            even[d] = __builtin_elementwise_max(even[d], __builtin_bit_cast(u16x2, u & 0x00ff00ffu));
+            odd[d] = __builtin_elementwise_max(odd[d], __builtin_bit_cast(u16x2, u & 0xff00ff00u));
+          }
+        v4i packed;
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          packed[d] = (int)((__builtin_bit_cast(unsigned, even[d]) | __builtin_bit_cast(unsigned, odd[d])) ^ 0x80808080u);
+        *reinterpret_cast<v4i *>(m) = packed;
+      } else
 #pragma unroll
       for (int t = 0; t < K * K; ++t) {
         if constexpr (VEC == 1) m[0] = (one[t] > m[0]) ? one[t] : m[0];

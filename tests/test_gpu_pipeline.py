@@ -218,6 +218,15 @@ def test_pool_kernels():
         q16 = orc.quantize(x, 16, -12)
         gq16 = torch.ops.torch_mlu.maxpool_nhwc(torch.from_numpy(q16).cuda(), k, s, p).cpu().numpy()
         assert np.array_equal(orc.quantize(want, 16, -12), gq16)
+    # the whole int8 / int16 range (the int8 kernel compares packed bytes), windows hanging over every border
+    for shape, k, s, p in (((2, 13, 10, 32), 3, 2, 1), ((1, 9, 12, 32), 2, 2, 0), ((2, 5, 6, 16), 3, 1, 0),
+                           ((1, 11, 11, 48), 5, 2, 2), ((1, 4, 4, 16), 2, 1, 1), ((3, 1, 1, 16), 3, 2, 1)):
+        for bits, dt in ((8, np.int8), (16, np.int16)):
+            q = g.integers(-2 ** (bits - 1), 2 ** (bits - 1), shape).astype(dt)
+            q[0, 0, 0, :4] = (-2 ** (bits - 1), 2 ** (bits - 1) - 1, -1, 0)
+            want = orc.maxpool_nhwc(q.astype(np.float32), k, s, p).astype(dt)
+            got = torch.ops.torch_mlu.maxpool_nhwc(torch.from_numpy(q).cuda(), k, s, p).cpu().numpy()
+            assert np.array_equal(want, got), (shape, k, s, p, bits)
     x = (g.standard_normal((3, 7, 7, 130)) * 100).astype(np.float32)
     got = torch.ops.torch_mlu.global_avgpool_nhwc(torch.from_numpy(x).cuda()).cpu().numpy()
     assert np.array_equal(orc.global_avgpool_nhwc(x), got)
