@@ -489,6 +489,51 @@ def test_specialised_epilogues(shape, q_scale):
             assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10, q_scale), out["q"].cpu().numpy()), row
 
 
+def test_conv_streamed_output_and_residual():
+    """an fp32 output of 64 MiB: the library writes it, and reads a residual of that size, with non-temporal hints
+    (a different store / load instruction in every epilogue); results must not depend on that"""
+    n, h, w, ci, co = 8, 128, 128, 16, 128
+    assert n * h * w * co * 4 >= 64 << 20
+    note("streamed output", (n, h, w, ci, co))
+    r = rng(77)
+    x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, 1, 1, ci), 8)
+    acc, _ = orc.conv2d_nhwc(x, wt, (0, 0), (1, 1), (1, 1), 1)
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = r.standard_normal(co).astype(np.float32)
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    for per_channel, use_res, act, y_dtype, q_bw in ((True, True, 1, torch.float32, 8), (True, False, 0, torch.float32, 0),
+                                                     (False, True, 3, torch.float32, 16), (True, True, 2, torch.float32, 0)):
+        out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), exp2=-9, chan_div=cabi.dev(div) if per_channel else None,
+                               bias=cabi.dev(bias), resid=cabi.dev(resid) if use_res else None, act=act, y_dtype=y_dtype,
+                               want_acc=False, q_bw=q_bw, q_pos=-3 if q_bw == 8 else -10,
+                               chan_rcp=cabi.dev(np.float32(1) / div) if per_channel else None, act_slope=0.1)
+        y = orc.epilogue(acc, -9, div if per_channel else None, bias, resid if use_res else None, act, act_slope=0.1)
+        assert same_bits(y, out["y"].cpu().numpy()), (per_channel, use_res, act)
+        if q_bw:
+            assert same_bits(orc.quantize(y, q_bw, -3 if q_bw == 8 else -10), out["q"].cpu().numpy())
+    # the LDS-ring kernel (K = 128) and the two-branch kernel at the same output size
+    x2, w2 = _ints(r, (n, h, w, 128), 8), _ints(r, (co, 1, 1, 128), 8)
+    acc2, _ = orc.conv2d_nhwc(x2, w2, (0, 0), (1, 1), (1, 1), 1)
+    assert cabi.conv_route(8, 8, x2.shape, w2.shape) == "mfma"
+    out = cabi.conv2d_nhwc(cabi.dev(x2), cabi.dev(w2), exp2=-12, chan_div=cabi.dev(div), bias=cabi.dev(bias),
+                           resid=cabi.dev(resid), act=1, want_acc=False, q_bw=8, q_pos=-3,
+                           chan_rcp=cabi.dev(np.float32(1) / div))
+    y2 = orc.epilogue(acc2, -12, div, bias, resid, 1)
+    assert same_bits(y2, out["y"].cpu().numpy()) and same_bits(orc.quantize(y2, 8, -3), out["q"].cpu().numpy())
+    sdiv = r.uniform(0.6, 3.5, co).astype(np.float32)
+    out, ws = cabi.conv2d_shortcut_nhwc(cabi.dev(x2), cabi.dev(w2), cabi.dev(x), cabi.dev(wt), 1, -9, cabi.dev(sdiv), cabi.dev(bias),
+                                        cabi.dev(np.float32(1) / sdiv), exp2=-12, chan_div=cabi.dev(div), bias=cabi.dev(bias),
+                                        act=1, q_bw=8, q_pos=-3, chan_rcp=cabi.dev(np.float32(1) / div))
+    assert ws == 0  # served by the two-branch kernel
+    y3 = orc.epilogue(acc2, -12, div, bias, orc.epilogue(acc, -9, sdiv, bias, None, 0), 1)
+    assert same_bits(y3, out["y"].cpu().numpy()) and same_bits(orc.quantize(y3, 8, -3), out["q"].cpu().numpy())
+    # the same through the GEMM entry point
+    a, b = x.reshape(-1, ci), wt.reshape(co, ci)
+    out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=-9, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=1,
+                       want_acc=False, chan_rcp=cabi.dev(np.float32(1) / div))
+    assert same_bits(orc.epilogue(acc.reshape(-1, co), -9, div, bias, None, 1), out["y"].cpu().numpy())
+
+
 def _random_conv_case(r):
     """a convolution problem drawn so that every kernel family turns up: few / odd / multiple-of-16 channel
     counts, depthwise and grouped, 1x1 to 7x7 filters, strides, dilations, padding"""
