@@ -268,7 +268,7 @@ static int launch_a16(const void *a, const void *b, IgemmParams p, const EpiDev 
   const int epi = pick_epilogue(p.N, e);
   if (epi == EPI_SCALAR)
     return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_SCALAR>(a, b, p, e, a_bytes, b_bytes, s);
-  if constexpr (BM == 64 && BN == 64) {  // the tile of every detector layer: leaky ReLU, int16 requantization
+  if constexpr (BM == 64) {  // the tiles of the detector layers: leaky ReLU, int16 requantization
     switch (epi) {
       case EPI_LK_Q16: return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_LK_Q16>(a, b, p, e, a_bytes, b_bytes, s);
       case EPI_LK_Y_Q16: return launch_a16_epi<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI_LK_Y_Q16>(a, b, p, e, a_bytes, b_bytes, s);
@@ -287,11 +287,19 @@ static int pick_a16_tile(const void *a, const void *b, const IgemmParams &p, con
   constexpr int64_t kCUs = 256;
   int tile = forced_tile();
   if (!tile) {
-    // Measured on every Darknet-53 layer (bs16, 416x416): the 64x64 tile wins or ties everywhere -- two
-    // accumulator sets and the digit split keep a wave busy enough, and small tiles mean more resident
-    // blocks per CU.  Only GEMMs far beyond those sizes take the wide tile.
+    // Measured on every Darknet-53 layer (bs16, 416x416): the 64x64 tile is the default -- two accumulator
+    // sets and the digit split keep a wave busy enough, and small tiles mean more resident blocks per CU.
+    // Only GEMMs far beyond those sizes take the widest tile.
     if (p.N >= 256 && p.K >= 256 && (int64_t)p.M * p.N * p.K >= (1ll << 34)) tile = 128256;
-    else tile = 64064;
+    else {
+      tile = 64064;
+      // Twice the columns per block halve the fetches of the int16 operand.  It pays where the epilogue is light
+      // enough for three waves per SIMD (leaky ReLU -> int16, no residual) and the launch still has two blocks
+      // per CU: the downsampling and head convolutions and the 1x1 layers of the detector gain 15-25 %; with the
+      // residual epilogue (two waves per SIMD) or fewer blocks the same tile loses a few percent (all measured).
+      const int epi = pick_epilogue(p.N, e);
+      if ((epi == EPI_LK_Q16 || epi == EPI_LK_Y_Q16) && p.N % 128 == 0 && blocks(64, 128) >= 2 * kCUs) tile = 64128;
+    }
   }
   switch (tile) {
     case 128256: return launch_a16<128, 256, 2, 4, 4, LOAD>(a, b, p, e, a_bytes, b_bytes, s);
