@@ -230,7 +230,9 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
         acc_lo[i][j][r] = (int)(((unsigned)acc_hi[i][j][r] << 8) + (unsigned)acc_lo[i][j][r] + ws);
   }
   int *stage = reinterpret_cast<int *>(lds_dyn) + wave * 32 * EPI_STRIDE;
-  igemm_epilogue<TM, TN, EPI>(acc_lo, stage, m0 + wave_m * WM, n0 + wave_n * WN, lane, p, e);
+  // the residual epilogues of the wide tile in two passes: 104 registers or fewer keep three waves per SIMD
+  constexpr int EPI_PASSES = (WN == 64 && (EPI == EPI_LK_RESA_Q16 || EPI == EPI_LK_RESA_Y_Q16)) ? 2 : 1;
+  igemm_epilogue<TM, TN, EPI, EPI_PASSES>(acc_lo, stage, m0 + wave_m * WM, n0 + wave_n * WN, lane, p, e);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int LOAD, int EPI>
@@ -293,12 +295,14 @@ static int pick_a16_tile(const void *a, const void *b, const IgemmParams &p, con
     if (p.N >= 256 && p.K >= 256 && (int64_t)p.M * p.N * p.K >= (1ll << 34)) tile = 128256;
     else {
       tile = 64064;
-      // Twice the columns per block halve the fetches of the int16 operand.  It pays where the epilogue is light
-      // enough for three waves per SIMD (leaky ReLU -> int16, no residual) and the launch still has two blocks
-      // per CU: the downsampling and head convolutions and the 1x1 layers of the detector gain 15-25 %; with the
-      // residual epilogue (two waves per SIMD) or fewer blocks the same tile loses a few percent (all measured).
+      // Twice the columns per block halve the fetches of the int16 operand.  It pays where the launch still has
+      // two blocks per CU and the kernel keeps three waves per SIMD, which the detector's epilogue instances do
+      // (the residual ones by working through a staged block in two passes): the 3x3 and 1x1 layers of
+      // Darknet-53 with 128 or more output channels gain 5-25 %, 7.6 % end to end; with fewer blocks or narrower
+      // outputs the same tile loses a few percent (all measured).
       const int epi = pick_epilogue(p.N, e);
-      if ((epi == EPI_LK_Q16 || epi == EPI_LK_Y_Q16) && p.N % 128 == 0 && blocks(64, 128) >= 2 * kCUs) tile = 64128;
+      const bool detector = epi == EPI_LK_Q16 || epi == EPI_LK_Y_Q16 || epi == EPI_LK_RESA_Q16 || epi == EPI_LK_RESA_Y_Q16;
+      if (detector && p.N % 128 == 0 && blocks(64, 128) >= 2 * kCUs) tile = 64128;
     }
   }
   switch (tile) {

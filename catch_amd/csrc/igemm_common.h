@@ -300,7 +300,10 @@ __device__ __forceinline__ int epi_lane_channel(int n_w, int lane) { return n_w 
 // 32-bit per-lane rest, and a wave whose tile lies wholly inside the matrix (the usual case) runs
 // without any per-lane bounds checks (FAST_PATH = false leaves that copy of the code out: kernels that
 // unroll the epilogue several times over cannot afford the registers its free scheduling takes).
-template <int TM, int TN, int EPI, bool FAST_PATH = true>
+// BATCHES > 1 handles the 32 rows of a staged block in that many passes (residual loads, staged reads and
+// arithmetic of one pass before the next): fewer values live at once, for instances that would otherwise lose a
+// wave per SIMD to their register count.
+template <int TM, int TN, int EPI, bool FAST_PATH = true, int BATCHES = 1>
 __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
                                                    const IgemmParams &p, const EpiDev &e, const EpiLane &L) {
   typedef typename EpiOf<EPI>::type S;
@@ -326,31 +329,40 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
       // offsets (loop invariants) in registers across the whole loop; recomputing them costs one add each.
       unsigned lane_off = lane_off0;
       asm volatile("" : "+v"(lane_off));
-      // residual rows of this 32-row block: all loads in flight before the staging below
-      v4f resv[NIT];
-      if (use_res) {
+      constexpr int NB = NIT / BATCHES;
+      static_assert(NIT % BATCHES == 0, "the passes must divide the iterations");
+      v4f resv[NB];
+      auto load_resid = [&](int b) {
 #pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          resv[it] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < NB; ++k) {
+          const int it = b * NB + k;
+          resv[k] = v4f{0.f, 0.f, 0.f, 0.f};
           if (FULL || (n_ok && it * RPI + rsub < rows))
-            resv[it] = load_stream(reinterpret_cast<const v4f *>((e.resid + uni) + (lane_off + it * it_step)), e.resid_stream != 0);
+            resv[k] = load_stream(reinterpret_cast<const v4f *>((e.resid + uni) + (lane_off + it * it_step)), e.resid_stream != 0);
         }
-      }
+      };
+      // residual rows of this 32-row block (of its first pass): all loads in flight before the staging below
+      if (use_res) load_resid(0);
       // wave-private staging: stores then loads of the same wave, ordered by the LDS counter
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
-      // all reads first: one LDS latency per 32 rows instead of one per iteration
-      v4i av[NIT];
 #pragma unroll
-      for (int it = 0; it < NIT; ++it)
-        av[it] = *reinterpret_cast<const v4i *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
+      for (int b = 0; b < BATCHES; ++b) {
+        if (b > 0 && use_res) load_resid(b);
+        // all reads first: one LDS latency per pass instead of one per iteration
+        v4i av[NB];
 #pragma unroll
-      for (int it = 0; it < NIT; ++it) {
-        if (!FULL && !(n_ok && it * RPI + rsub < rows)) continue;
-        epi_vec4<S>(av[it], use_res ? resv[it] : v4f{0.f, 0.f, 0.f, 0.f}, L, EpiAtSplit{uni, lane_off + it * it_step}, e);
+        for (int k = 0; k < NB; ++k)
+          av[k] = *reinterpret_cast<const v4i *>(stage + ((b * NB + k) * RPI + rsub) * EPI_STRIDE + cg * 4);
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+          const int it = b * NB + k;
+          if (!FULL && !(n_ok && it * RPI + rsub < rows)) continue;
+          epi_vec4<S>(av[k], use_res ? resv[k] : v4f{0.f, 0.f, 0.f, 0.f}, L, EpiAtSplit{uni, lane_off + it * it_step}, e);
+        }
       }
     }
   };
@@ -421,7 +433,7 @@ __device__ __forceinline__ void igemm_epilogue_dual(v16i (&acc)[TM][TN], v16i (&
 
 // Epilogue of one wave.  acc[i][j] is the 32x32 accumulator of rows m_w + i*32 .., columns
 // n_w + j*32 ..; stage is this wave's private LDS area of 32 * (TN*32 + 8) ints.
-template <int TM, int TN, int EPI>
+template <int TM, int TN, int EPI, int BATCHES = 1>
 __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, int64_t m_w, int n_w, int lane,
                                                const IgemmParams &p, const EpiDev &e) {
   typedef typename EpiOf<EPI>::type S;
@@ -447,7 +459,7 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
   } else {
     const int n = epi_lane_channel<TN>(n_w, lane);
     const EpiLane L = epi_lane_setup<S>(n, n < p.N, e);
-    igemm_epilogue_vec<TM, TN, EPI>(acc, stage, m_w, n_w, lane, p, e, L);
+    igemm_epilogue_vec<TM, TN, EPI, true, BATCHES>(acc, stage, m_w, n_w, lane, p, e, L);
   }
 }
 
