@@ -368,20 +368,43 @@ class FusedNet(object):
         return forms
 
     # ------------------------------------------------------------------------------------------
-    def capture(self, example):
+    def capture(self, example, streams=1):
         """Record one forward pass into a HIP graph; returns (static_input, replay) where replay()
-        re-runs the whole network on whatever static_input holds and returns the static output(s)."""
+        re-runs the whole network on whatever static_input holds and returns the static output(s).
+
+        streams > 1 splits the batch into that many parts, each recorded on a stream of its own (all of
+        default priority) between a fork and a join: the images are independent, so the results are the
+        same tensors, and the launches of one part fill the compute units that the other part's launches
+        leave idle while they start up and drain."""
         static_in = example.clone()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(2):
-                self.forward(static_in)
-        torch.cuda.current_stream().wait_stream(side)
+        parts = max(1, min(int(streams), static_in.shape[0]))
+        chunks = list(static_in.chunk(parts))
+        side = [torch.cuda.Stream() for _ in chunks]
+        for st, c in zip(side, chunks):  # warm-up outside the capture, on the streams the graph will use
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                for _ in range(2):
+                    self.forward(c)
+        for st in side:
+            torch.cuda.current_stream().wait_stream(st)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            static_out = self.forward(static_in)
+            if len(chunks) == 1:
+                static_out = self.forward(static_in)
+            else:
+                cur = torch.cuda.current_stream()
+                outs = []
+                for st, c in zip(side, chunks):
+                    st.wait_stream(cur)
+                    with torch.cuda.stream(st):
+                        outs.append(self.forward(c))
+                for st in side:
+                    cur.wait_stream(st)
+                if isinstance(outs[0], tuple):
+                    static_out = tuple(torch.cat([o[i] for o in outs]) for i in range(len(outs[0])))
+                else:
+                    static_out = torch.cat(outs)
         self._graph = graph
 
         def replay():

@@ -131,6 +131,37 @@ def test_resnet50_small_batch_and_graph_replay():
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("arch,batch,streams", [("resnet50", 5, 2), ("resnet50", 4, 3), ("darknet53_yolov3", 3, 2),
+                                                ("resnet18", 2, 4)])
+def test_graph_with_the_batch_on_parallel_streams(arch, batch, streams):
+    """the batch split into parts that run on streams of their own inside one HIP graph (uneven parts, more
+    streams than images, several outputs): every replay equals the single eager pass, new inputs included"""
+    note("parallel streams", arch, batch, streams)
+    layers = nets.NETS[arch]()
+    det = arch.startswith("darknet")
+    net = nets.FloatNet(layers, seed=0, weight_std="he" if det else 0.05).eval()
+    g = torch.Generator().manual_seed(11)
+    x = torch.rand(batch, 3, 64, 64, generator=g) if det else torch.randn(batch, 3, 64, 64, generator=g)
+    sd = pipeline.calibrate(net, x, "int16" if det else "int8", not det)
+    if det:
+        sd = pipeline.to_position_encoding(sd, 16, 8)
+    fused = pipeline.FusedNet(layers, sd, out_half=det)
+    static_in, replay = fused.capture(x.cuda(), streams=streams)
+    for i in range(4):
+        xi = x.cuda() if i % 2 == 0 else (x.cuda() * 0.5 + 0.1)
+        want = fused.forward(xi)
+        static_in.copy_(xi)
+        got = replay()
+        torch.cuda.synchronize()
+        want = want if isinstance(want, tuple) else (want,)
+        got = got if isinstance(got, tuple) else (got,)
+        assert len(want) == len(got)
+        for a, b in zip(want, got):
+            assert a.shape == b.shape and torch.equal(a, b), "replay %d" % i
+        _ = fused.forward(torch.randn(batch, 3, 64, 64, device="cuda"))  # eager work between the replays
+        torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("depth,expect", [(18, ["l2.0.c2", "l3.0.c2", "l4.0.c2"]),
                                           (50, ["l1.0.c3", "l2.0.c3", "l3.0.c3", "l4.0.c3"])])
 def test_projection_shortcuts_fused_into_block_end(depth, expect):
