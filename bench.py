@@ -191,6 +191,8 @@ def main():
     # The launches measured are the ones the graph holds: with the batch in `streams` parts, every layer is
     # launched once per part, on that part's images.
     parts = list(xg.chunk(args.streams))
+    from catch_amd import _native
+    _native.kernel_lib().catchq_set_launch_sharing(args.streams)  # the tile shapes the graph's launches were given
     rows = layer_profile(fused, parts[0])
     # Launch durations in their real sequence: HIP events around every conv/fc launch of eager forward
     # passes on the stream the kernels run on (no graph: a captured launch cannot be bracketed; one part
@@ -202,6 +204,7 @@ def main():
         for part in parts:
             fused.forward(part, timers=t_)
     torch.cuda.synchronize()
+    _native.kernel_lib().catchq_set_launch_sharing(1)
     seq = {}
     for name, evs in timers.items():
         pairs = [(evs[i], evs[i + 1]) for i in range(0, len(evs), 2)]

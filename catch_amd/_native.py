@@ -43,6 +43,7 @@ class Shortcut(ctypes.Structure):
 _I, _I64, _F, _P, _SZ = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 SIGNATURES = {
     "catchq_version": (_I, []),
+    "catchq_set_launch_sharing": (_I, [_I]),
     "catchq_status_string": (ctypes.c_char_p, [_I]),
     "catchq_pos_from_scale": (_I, [_I, _F, ctypes.POINTER(_I)]),
     "catchq_quant_params": (_I, [_I, _F, ctypes.POINTER(_I), ctypes.POINTER(_F), ctypes.POINTER(_F)]),

@@ -19,6 +19,10 @@ inline hipStream_t as_stream(catchq_stream_t s) { return reinterpret_cast<hipStr
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? CATCHQ_OK : CATCHQ_ERR_LAUNCH; }
 
+// compute units one launch should plan its tile shapes for: the device's 256, divided by the number of
+// launches the caller says share the device (catchq_set_launch_sharing)
+int planned_cus();
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- the quantize rule: q = sat(rne(x * scale * 2^-pos)), NaN -> 0 -------------------------

@@ -380,6 +380,15 @@ class FusedNet(object):
         parts = max(1, min(int(streams), static_in.shape[0]))
         chunks = list(static_in.chunk(parts))
         side = [torch.cuda.Stream() for _ in chunks]
+        # the launches recorded below will share the device: their tile shapes are chosen for a part of it
+        lib = _native.kernel_lib()
+        before = lib.catchq_set_launch_sharing(len(chunks))
+        try:
+            return self._capture(static_in, chunks, side)
+        finally:
+            lib.catchq_set_launch_sharing(max(before, 1))
+
+    def _capture(self, static_in, chunks, side):
         for st, c in zip(side, chunks):  # warm-up outside the capture, on the streams the graph will use
             st.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(st):

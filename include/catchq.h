@@ -47,6 +47,13 @@ enum { CATCHQ_QUANTIZE_POSITION = 0, CATCHQ_QUANTIZE_POSITION_SCALE = 1, CATCHQ_
 int catchq_version(void);
 const char *catchq_status_string(int status);
 
+/* Planning hint: `launches` launches of this library are expected to run on the device at the same time
+ * (e.g. the parts of a batch on parallel streams), so each one's tile shapes are chosen for 1/launches of the
+ * compute units.  Affects speed only, never a result.  Process-wide, default 1; returns the previous value,
+ * or -CATCHQ_ERR_ARG for launches < 1.  (The reference plans per handle, one handle per device re-bound to
+ * the calling thread's queue: torch_mlu/csrc/aten/cnnl/cnnlHandle.cpp:41-55; it has no such hint.) */
+int catchq_set_launch_sharing(int launches);
+
 /* ------------------------------------------------------------------ host q-param math */
 
 /* get_pos_from_scale_data(bitwidth, scale_data)            cnnl/cnnl_util.cpp:337-347 */

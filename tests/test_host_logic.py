@@ -37,6 +37,16 @@ def test_library_exports_every_declared_symbol(lib):
     assert lib.catchq_status_string(2) == b"quantify only support input float/half"
 
 
+def test_launch_sharing_hint(lib):
+    """process-wide planning hint: returns the previous value, rejects counts below one, changes the tile a route
+    reports nothing about (results never depend on it: the GPU suite runs graphs recorded with 1, 2, 3 and 4)"""
+    assert lib.catchq_set_launch_sharing(1) >= 1
+    assert lib.catchq_set_launch_sharing(4) == 1
+    assert lib.catchq_set_launch_sharing(2) == 4
+    assert lib.catchq_set_launch_sharing(0) < 0 and lib.catchq_set_launch_sharing(-3) < 0
+    assert lib.catchq_set_launch_sharing(1) == 2  # the rejected calls left it alone
+
+
 def test_torch_ops_are_registered():
     import catch_amd  # noqa: F401
     for name in ("conv2d", "linear", "quantize", "quantize_per_channel", "quantize_param", "mm_q", "qconv2d",
