@@ -114,7 +114,8 @@ struct ShortcutDev {
 // out_elems: elements of the output tensor (0: unknown, nothing is streamed)
 inline EpiDev make_epi(const catchq_epilogue_t *e, int64_t out_elems = 0) {
   EpiDev d;
-  constexpr int64_t kStreamBytes = 64ll << 20;  // a quarter of the 256 MB last-level cache
+  // a quarter of the 256 MB last-level cache, of this launch's share of it
+  const int64_t kStreamBytes = (64ll << 20) * planned_cus() / 256;
   d.y_stream = (e->y && out_elems * (e->y_dtype == CATCHQ_F16 ? 2 : 4) >= kStreamBytes) ? 1 : 0;
   d.resid_stream = (e->resid && out_elems * 4 >= kStreamBytes) ? 1 : 0;
   d.exp2 = e->exp2;
