@@ -205,10 +205,20 @@ def main():
             fused.forward(part, timers=t_)
     torch.cuda.synchronize()
     _native.kernel_lib().catchq_set_launch_sharing(1)
+    # what a pair of events reads with nothing between them (the command processor's time per marker): part of
+    # every bracketed duration, none of the kernel's
+    empty = []
+    for _ in range(200):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        b.record()
+        empty.append((a, b))
+    torch.cuda.synchronize()
+    empty_s = sorted(a.elapsed_time(b) for a, b in empty)[len(empty) // 2] * 1e-3
     seq = {}
     for name, evs in timers.items():
         pairs = [(evs[i], evs[i + 1]) for i in range(0, len(evs), 2)]
-        seq[name] = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs) * 1e-3
+        seq[name] = max(sum(a.elapsed_time(b) for a, b in pairs) / len(pairs) * 1e-3 - empty_s, 1e-7)
     for r in rows:
         r["t_seq"] = seq[r["name"]]
     conv_rows = [r for r in rows if r["route"].startswith("mfma")]
@@ -232,7 +242,9 @@ def main():
                 "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, batch, n_parts)),
                 "avg_launch_us": round(t_conv / max(n_parts * len(conv_rows), 1) * 1e6, 2),
-                "timing": "HIP events around each launch of eager forward passes over the parts, in sequence (%d passes)" % args.seq_passes,
+                "timing": "HIP events around each launch of eager forward passes over the parts, in sequence (%d passes), "
+                          "minus what an empty pair of events reads in the same run (%.2f us)" % (args.seq_passes, empty_s * 1e6),
+                "event_pair_overhead_us": round(empty_s * 1e6, 2),
                 "achieved_repeated_launches": round(b_conv / t_conv_hot / 1e9, 1),
                 "algorithmic_bytes_per_step": b_conv, "int8_tops": round(o_conv / t_conv / 1e12, 1),
                 "mfma_frac": round(o_conv / t_conv / 1e12 / INT8_PEAK_TOPS, 4),
