@@ -205,16 +205,26 @@ def main():
             fused.forward(part, timers=t_)
     torch.cuda.synchronize()
     _native.kernel_lib().catchq_set_launch_sharing(1)
-    # what a pair of events reads with nothing between them (the command processor's time per marker): part of
-    # every bracketed duration, none of the kernel's
-    empty = []
-    for _ in range(200):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        b.record()
-        empty.append((a, b))
-    torch.cuda.synchronize()
-    empty_s = sorted(a.elapsed_time(b) for a, b in empty)[len(empty) // 2] * 1e-3
+    # The part of a bracketed duration that is the bracket's, not the kernel's: a pair of events around one small
+    # kernel reads T1, around two of them T2; T2 - T1 is one kernel (and the gap before it), so 2*T1 - T2 is what
+    # does not grow with the kernels in between.  (An empty pair reads more, 5.1 us: the markers' own processing
+    # partly hides behind a kernel when there is one.)
+    probe = torch.zeros(1 << 20, device="cuda")
+
+    def bracket(n_kernels, reps=200):
+        evs = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(n_kernels):
+                probe.add_(1.0)
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) for a, b in evs)[reps // 2] * 1e-3
+    bracket(1, 20)
+    t1, t2 = bracket(1), bracket(2)
+    empty_s = min(max(2 * t1 - t2, 0.0), t1)
     seq = {}
     for name, evs in timers.items():
         pairs = [(evs[i], evs[i + 1]) for i in range(0, len(evs), 2)]
@@ -243,7 +253,8 @@ def main():
                 "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, batch, n_parts)),
                 "avg_launch_us": round(t_conv / max(n_parts * len(conv_rows), 1) * 1e6, 2),
                 "timing": "HIP events around each launch of eager forward passes over the parts, in sequence (%d passes), "
-                          "minus what an empty pair of events reads in the same run (%.2f us)" % (args.seq_passes, empty_s * 1e6),
+                          "minus the bracket's own share, 2*T(pair around one small kernel) - T(pair around two), "
+                          "measured in the same run (%.2f us)" % (args.seq_passes, empty_s * 1e6),
                 "event_pair_overhead_us": round(empty_s * 1e6, 2),
                 "achieved_repeated_launches": round(b_conv / t_conv_hot / 1e9, 1),
                 "algorithmic_bytes_per_step": b_conv, "int8_tops": round(o_conv / t_conv / 1e12, 1),
