@@ -415,6 +415,10 @@ class FusedNet(object):
                 else:
                     static_out = torch.cat(outs)
         self._graph = graph
+        # the first replays of a new graph are slower (the executable graph is uploaded on first use): take them here
+        for _ in range(8):
+            graph.replay()
+        torch.cuda.synchronize()
 
         def replay():
             graph.replay()
