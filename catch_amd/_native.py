@@ -61,6 +61,7 @@ SIGNATURES = {
     "catchq_conv2d_nhwc": (_I, [_P, _I, _P, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Epilogue), _P]),
     "catchq_maxpool_nhwc": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "catchq_global_avgpool_nhwc": (_I, [_P, _P, _I, _I, _I, _P]),
+    "catchq_global_avgpool_quantize_nhwc": (_I, [_P, _P, _I, _I, _I, _I, _I, _F, _P]),
     "catchq_quantize_conv2d_workspace_size": (_I, [ctypes.POINTER(ConvDesc), _I, _I, ctypes.POINTER(_SZ)]),
     "catchq_quantize_conv2d_nhwc": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, ctypes.POINTER(ConvDesc), _P, _P, _I, _P, _SZ, _P]),
     "catchq_conv2d_shortcut_workspace_size": (_I, [_I, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Shortcut),

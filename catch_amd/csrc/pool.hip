@@ -137,8 +137,10 @@ static int launch_maxpool(const void *x, void *y, int N, int H, int W, int C, in
   return launch_status();
 }
 
-__global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const float *__restrict__ x, float *__restrict__ y,
-                                                                 int N, int HW, int C) {
+// QBW = 0: the fp32 mean; 8 / 16: the mean quantized at (position, scale)
+template <int QBW>
+__global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const float *__restrict__ x, void *__restrict__ yv,
+                                                                 int N, int HW, int C, int neg_pos, float scale) {
   const int64_t total = (int64_t)N * C;
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (int64_t)gridDim.x * blockDim.x) {
@@ -157,7 +159,10 @@ __global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const float *_
       for (int u = 0; u < 8; ++u) s = s + v[u];
     }
     for (; p < HW; ++p) s = s + src[(int64_t)p * C];
-    y[idx] = s / (float)HW;
+    const float mean = s / (float)HW;
+    if constexpr (QBW == 0) reinterpret_cast<float *>(yv)[idx] = mean;
+    else if constexpr (QBW == 8) reinterpret_cast<int8_t *>(yv)[idx] = (int8_t)quant1<8>(mean, scale, neg_pos);
+    else reinterpret_cast<int16_t *>(yv)[idx] = (int16_t)quant1<16>(mean, scale, neg_pos);
   }
 }
 
@@ -188,6 +193,21 @@ CATCHQ_API int catchq_global_avgpool_nhwc(const float *x, float *y, int n, int h
   const int64_t total = (int64_t)n * c;
   int blocks = (int)((total + 255) / 256);
   if (blocks > 65536) blocks = 65536;
-  global_avgpool_nhwc_kernel<<<blocks, 256, 0, as_stream(stream)>>>(x, y, n, hw, c);
+  global_avgpool_nhwc_kernel<0><<<blocks, 256, 0, as_stream(stream)>>>(x, y, n, hw, c, 0, 1.0f);
+  return launch_status();
+}
+
+CATCHQ_API int catchq_global_avgpool_quantize_nhwc(const float *x, void *q, int bitwidth, int n, int hw, int c,
+                                                   int position, float scale, catchq_stream_t stream) {
+  if (n < 0 || hw <= 0 || c <= 0) return CATCHQ_ERR_SHAPE;
+  if (bitwidth != 8 && bitwidth != 16) return CATCHQ_ERR_BITWIDTH;
+  if (position < -126 || position > 126) return CATCHQ_ERR_ARG;
+  if (n == 0) return CATCHQ_OK;
+  if (!x || !q) return CATCHQ_ERR_ARG;
+  const int64_t total = (int64_t)n * c;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 65536) blocks = 65536;
+  if (bitwidth == 8) global_avgpool_nhwc_kernel<8><<<blocks, 256, 0, as_stream(stream)>>>(x, q, n, hw, c, -position, scale);
+  else global_avgpool_nhwc_kernel<16><<<blocks, 256, 0, as_stream(stream)>>>(x, q, n, hw, c, -position, scale);
   return launch_status();
 }

@@ -830,11 +830,21 @@ Tensor maxpool_nhwc_op(const Tensor &x, int64_t k, int64_t stride, int64_t pad) 
   return y;
 }
 
-// x [N,H,W,C] contiguous fp32 -> [N,C]
-Tensor global_avgpool_nhwc_op(const Tensor &x) {
+// x [N,H,W,C] contiguous fp32 -> [N,C]: the fp32 means, or (q_bitwidth 8 / 16) the means quantized at
+// (q_position, q_scale) in the same launch
+Tensor global_avgpool_nhwc_op(const Tensor &x, int64_t q_bitwidth, int64_t q_position, double q_scale) {
   TORCH_CHECK(x.dim() == 4 && x.is_contiguous() && x.scalar_type() == at::kFloat,
               "global_avgpool_nhwc expects a contiguous fp32 [N,H,W,C] tensor");
   c10::DeviceGuard guard(x.device());
+  if (q_bitwidth != 0) {
+    TORCH_CHECK(q_bitwidth == 8 || q_bitwidth == 16, "bitwidth not support");
+    Tensor q = at::empty({x.size(0), x.size(3)}, x.options().dtype(int_type((int)q_bitwidth)));
+    check_status(catchq_global_avgpool_quantize_nhwc(x.data_ptr<float>(), q.data_ptr(), (int)q_bitwidth, (int)x.size(0),
+                                                     (int)(x.size(1) * x.size(2)), (int)x.size(3), (int)q_position,
+                                                     (float)q_scale, current_stream()),
+                 "torch_mlu::global_avgpool_nhwc");
+    return q;
+  }
   Tensor y = at::empty({x.size(0), x.size(3)}, x.options());
   check_status(catchq_global_avgpool_nhwc(x.data_ptr<float>(), y.data_ptr<float>(), (int)x.size(0),
                                           (int)(x.size(1) * x.size(2)), (int)x.size(3), current_stream()),
@@ -884,7 +894,7 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("quantize_conv2d(Tensor input, Tensor input_position, Tensor weight, Tensor weight_position, Tensor bias, "
         "int[] padding, int[] stride, int[] dilation, int groups, int input_bitwidth=8, int weight_bitwidth=8) -> Tensor");
   m.def("maxpool_nhwc(Tensor x, int k, int stride, int pad) -> Tensor");
-  m.def("global_avgpool_nhwc(Tensor x) -> Tensor");
+  m.def("global_avgpool_nhwc(Tensor x, int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> Tensor");
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
         "int[] dilation, int groups) -> str", &conv2d_route_op);

@@ -338,10 +338,15 @@ class FusedNet(object):
                 for form in self._forms(name):
                     env[(name,) + form] = ops.maxpool_nhwc(env[(l.src,) + form], l.k, l.stride, l.pad)
             elif l.kind == "gap":
-                g = ops.global_avgpool_nhwc(env[(l.src, "f")])
-                env[(name, "f")] = g.reshape(g.shape[0], 1, 1, g.shape[1])
-                for d in self.q_demand[name]:
-                    env[(name,) + d] = ops.quantize(env[(name, "f")], d[0], d[1], d[2])
+                if self.f_demand[name] or tracing or not self.q_demand[name]:
+                    g = ops.global_avgpool_nhwc(env[(l.src, "f")])
+                    env[(name, "f")] = g.reshape(g.shape[0], 1, 1, g.shape[1])
+                    for d in self.q_demand[name]:
+                        env[(name,) + d] = ops.quantize(env[(name, "f")], d[0], d[1], d[2])
+                else:  # only quantized forms are read: pooled and quantized in one launch each
+                    for d in self.q_demand[name]:
+                        g = ops.global_avgpool_nhwc(env[(l.src, "f")], d[0], d[1], d[2])
+                        env[(name,) + d] = g.reshape(g.shape[0], 1, 1, g.shape[1])
             elif l.kind == "upsample":
                 for form in self._forms(name):
                     t = env[(l.src,) + form]
@@ -389,31 +394,38 @@ class FusedNet(object):
             lib.catchq_set_launch_sharing(max(before, 1))
 
     def _capture(self, static_in, chunks, side):
+        sample = None
         for st, c in zip(side, chunks):  # warm-up outside the capture, on the streams the graph will use
             st.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(st):
                 for _ in range(2):
-                    self.forward(c)
+                    sample = self.forward(c)
         for st in side:
             torch.cuda.current_stream().wait_stream(st)
         torch.cuda.synchronize()
+        # the whole batch's outputs, allocated outside the graph; every part fills its rows
+        sample_outs = sample if isinstance(sample, tuple) else (sample,)
+        whole = [torch.empty((static_in.shape[0],) + tuple(o.shape[1:]), dtype=o.dtype, device=o.device,
+                             memory_format=torch.channels_last if o.dim() == 4 else torch.contiguous_format)
+                 for o in sample_outs]  # feature maps stay NHWC in memory, like the parts' own outputs
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             if len(chunks) == 1:
                 static_out = self.forward(static_in)
             else:
+                # every part copies its outputs into its rows of the whole batch's outputs on its own stream
                 cur = torch.cuda.current_stream()
-                outs = []
+                row = 0
                 for st, c in zip(side, chunks):
                     st.wait_stream(cur)
                     with torch.cuda.stream(st):
-                        outs.append(self.forward(c))
+                        out = self.forward(c)
+                        for w_, o in zip(whole, out if isinstance(out, tuple) else (out,)):
+                            w_[row:row + c.shape[0]].copy_(o)
+                    row += c.shape[0]
                 for st in side:
                     cur.wait_stream(st)
-                if isinstance(outs[0], tuple):
-                    static_out = tuple(torch.cat([o[i] for o in outs]) for i in range(len(outs[0])))
-                else:
-                    static_out = torch.cat(outs)
+                static_out = tuple(whole) if isinstance(sample, tuple) else whole[0]
         self._graph = graph
         # the first replays of a new graph are slower (the executable graph is uploaded on first use): take them here
         for _ in range(8):

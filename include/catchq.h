@@ -241,6 +241,13 @@ int catchq_maxpool_nhwc(const void *x, void *y, int elem_bits, int n, int h, int
  * models, operators/cnnl/pooling.cpp). */
 int catchq_global_avgpool_nhwc(const float *x, float *y, int n, int hw, int c, catchq_stream_t stream);
 
+/* The same pooling followed by the quantizer of the layer that consumes it, in one launch:
+ * q[n, c] = sat(rne(mean * scale * 2^-position)), int8 / int16 (bitwidth 8 / 16) -- the values
+ * catchq_global_avgpool_nhwc then catchq_quantize produce (adaptive_avg_pool2d, operators/cnnl/pooling.cpp,
+ * followed by cnnl_quantify_offline_internal, operators/cnnl/internal/quantify.cpp:69-101, in the reference). */
+int catchq_global_avgpool_quantize_nhwc(const float *x, void *q, int bitwidth, int n, int hw, int c, int position,
+                                        float scale, catchq_stream_t stream);
+
 /* Name of the kernel family catchq_conv2d_nhwc / catchq_gemm_nt would use ("mfma", "direct",
  * "depthwise", ...): for logs and tests; not part of the arithmetic. */
 const char *catchq_conv2d_route(int x_bits, int w_bits, const catchq_conv_desc_t *desc);

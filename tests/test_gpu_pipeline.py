@@ -261,3 +261,16 @@ def test_pool_kernels():
     x = (g.standard_normal((3, 7, 7, 130)) * 100).astype(np.float32)
     got = torch.ops.torch_mlu.global_avgpool_nhwc(torch.from_numpy(x).cuda()).cpu().numpy()
     assert np.array_equal(orc.global_avgpool_nhwc(x), got)
+
+
+def test_global_avgpool_with_fused_quantizer():
+    """the pooled-and-quantized launch equals pooling then quantizing, at unit and fractional scale, int8 and int16"""
+    import oracle as orc
+    g = np.random.default_rng(5)
+    x = (g.standard_normal((3, 7, 7, 130)) * 40).astype(np.float32)
+    mean = orc.global_avgpool_nhwc(x)
+    for bw, pos, scale in ((8, -1, 1.0), (8, 0, 1.3720703125), (16, -9, 1.0), (16, -8, 1.9990234375)):
+        got = torch.ops.torch_mlu.global_avgpool_nhwc(torch.from_numpy(x).cuda(), bw, pos, scale).cpu().numpy()
+        assert np.array_equal(orc.quantize(mean, bw, pos, scale), got), (bw, pos, scale)
+    with pytest.raises(RuntimeError, match="bitwidth not support"):
+        torch.ops.torch_mlu.global_avgpool_nhwc(torch.from_numpy(x).cuda(), 12, 0, 1.0)
