@@ -148,15 +148,17 @@ __global__ __launch_bounds__(256) void global_avgpool_nhwc_kernel(const float *_
     const int64_t n = idx / C;
     const float *src = x + n * HW * C + c;
     // the sum runs over the pixels in order (one fp32 addition each: the order is part of the result);
-    // eight loads are requested before their additions so that the thread has more than one in flight
+    // 25 loads are requested before their additions (a 7x7 map is two such batches): with one wave per SIMD the
+    // kernel's time is the number of memory round trips a thread makes
     float s = 0.0f;
     int p = 0;
-    for (; p + 8 <= HW; p += 8) {
-      float v[8];
+    constexpr int U = 25;
+    for (; p + U <= HW; p += U) {
+      float v[U];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(p + u) * C];
+      for (int u = 0; u < U; ++u) v[u] = src[(int64_t)(p + u) * C];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) s = s + v[u];
+      for (int u = 0; u < U; ++u) s = s + v[u];
     }
     for (; p < HW; ++p) s = s + src[(int64_t)p * C];
     const float mean = s / (float)HW;
