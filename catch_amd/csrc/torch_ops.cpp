@@ -299,6 +299,7 @@ EpiOut qconv2d_impl(const Tensor &qx, const Tensor &qw, at::IntArrayRef padding,
   catchq_epilogue_t e;
   std::vector<Tensor> keep;
   EpiOut o = prepare_epilogue(a, {d.n, ho, wo, d.co}, d.co, qx.options(), &e, &keep);
+  if (d.n == 0 || d.co == 0) return o;  // nothing to compute: the empty outputs are the result
   check_status(catchq_conv2d_nhwc(qx.data_ptr(), bits_of(qx), qw.data_ptr(), bits_of(qw), &d, &e, current_stream()),
                "torch_mlu::conv2d");
   return o;
@@ -347,6 +348,7 @@ EpiOut qconv2d_shortcut_impl(const Tensor &qx, const Tensor &qw, at::IntArrayRef
     if (rcp.defined()) { sc.chan_rcp = rcp.data_ptr<float>(); keep.push_back(rcp); }
   }
   if (bs.defined()) { sc.bias = bs.data_ptr<float>(); keep.push_back(bs); }
+  if (d.n == 0) return o;  // nothing to compute
   size_t ws_bytes = 0;
   check_status(catchq_conv2d_shortcut_workspace_size(bits_of(qx), bits_of(qw), &d, &sc, &ws_bytes),
                "torch_mlu::qconv2d_shortcut");
@@ -363,6 +365,7 @@ EpiOut qlinear_impl(const Tensor &qx, const Tensor &qw, const EpiArgs &a) {
   catchq_epilogue_t e;
   std::vector<Tensor> keep;
   EpiOut o = prepare_epilogue(a, {qx.size(0), qw.size(0)}, qw.size(0), qx.options(), &e, &keep);
+  if (qx.size(0) == 0 || qw.size(0) == 0) return o;  // nothing to compute
   check_status(catchq_gemm_nt(qx.data_ptr(), bits_of(qx), qw.data_ptr(), bits_of(qw), qx.size(0), qw.size(0),
                               qx.size(1), &e, current_stream()),
                "torch_mlu::linear");

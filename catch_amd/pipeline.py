@@ -327,7 +327,7 @@ class FusedNet(object):
             elif l.kind == "fc":
                 lq = self.q[name]
                 qx = env[(l.src, lq.bw_x, lq.pos_x, lq.scale_x)]
-                qx2 = qx.reshape(qx.shape[0], -1)
+                qx2 = qx.reshape(qx.shape[0], lq.qw.shape[1])  # not -1: an empty batch leaves it ambiguous
                 tick(name)
                 y, _, acc = ops.qlinear(qx2, lq.qw, lq.exp2, lq.chan_div, lq.bias, 0, True, False, tracing, 0, 0, 1.0)
                 tick(name)

@@ -401,3 +401,48 @@ def test_conv2d_first_qint(k, co, h, w):
     ref = oops.conv2d(x_norm.cpu().numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
                       (2, 2), (1, 4), (1, 1), 1, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
     assert same_bits(ref["y"], got.cpu().numpy())
+
+
+def test_empty_batches():
+    """zero images / zero rows: the ops return empty tensors of the right shape and dtype, nothing is launched"""
+    note("empty batches")
+    w = torch.randn(8, 4, 3, 3)
+    q_scale = torch.tensor([20.0, 30.0])
+    q_mode = torch.tensor([1], dtype=torch.int32)
+    for dt in (torch.float32, torch.float16):
+        x = torch.zeros(0, 4, 9, 9, dtype=dt, device="cuda")
+        y = torch.ops.torch_mlu.conv2d(x, w.cuda().to(dt), torch.zeros(8, device="cuda", dtype=dt), [1, 1], [2, 2], [1, 1], 1,
+                                       q_scale.cuda(), q_mode.cuda())
+        assert tuple(y.shape) == (0, 8, 5, 5) and y.dtype == dt
+    xl = torch.zeros(0, 16, device="cuda")
+    yl = torch.ops.torch_mlu.linear(xl, torch.randn(5, 16, device="cuda"), torch.zeros(5, device="cuda"), q_scale.cuda(),
+                                    q_mode.cuda())
+    assert tuple(yl.shape) == (0, 5)
+    yl = torch.ops.torch_mlu.linear(torch.zeros(3, 0, 16, device="cuda"), torch.randn(5, 16, device="cuda"),
+                                    torch.zeros(5, device="cuda"), q_scale.cuda(), q_mode.cuda())
+    assert tuple(yl.shape) == (3, 0, 5)
+    q = torch.ops.torch_mlu.quantize(torch.zeros(0, 7, device="cuda"), 8, -3)
+    assert tuple(q.shape) == (0, 7) and q.dtype == torch.int8
+    p = torch.ops.torch_mlu.maxpool_nhwc(torch.zeros(0, 8, 8, 16, dtype=torch.int8, device="cuda"), 3, 2, 1)
+    assert tuple(p.shape) == (0, 4, 4, 16)
+    g = torch.ops.torch_mlu.global_avgpool_nhwc(torch.zeros(0, 7, 7, 32, device="cuda"))
+    assert tuple(g.shape) == (0, 32)
+    y1 = torch.ops.torch_mlu.conv1d(torch.zeros(0, 4, 20, device="cuda"), torch.randn(6, 4, 3, device="cuda"),
+                                    torch.zeros(6, device="cuda"), [1], [1], [1], 1, q_scale.cuda(), q_mode.cuda())
+    assert tuple(y1.shape) == (0, 6, 20)
+    y3 = torch.ops.torch_mlu.conv3d(torch.zeros(0, 4, 5, 6, 6, device="cuda"), torch.randn(6, 4, 3, 3, 3, device="cuda"),
+                                    torch.zeros(6, device="cuda"), [1, 1, 1], [1, 1, 1], [1, 1, 1], 1, q_scale.cuda(),
+                                    q_mode.cuda())
+    assert tuple(y3.shape) == (0, 6, 5, 6, 6)
+    m = torch.ops.torch_mlu.mm_q(torch.zeros(0, 16, dtype=torch.int8, device="cuda"), -3,
+                                 torch.zeros(5, 16, dtype=torch.int8, device="cuda"), -4)
+    assert tuple(m.shape) == (0, 5)
+    # the fused plan on an empty batch
+    from catch_amd import nets, pipeline
+    layers = nets.resnet(18)
+    net = nets.FloatNet(layers, seed=0).eval()
+    xc = torch.randn(1, 3, 64, 64, generator=torch.Generator().manual_seed(1))
+    fused = pipeline.FusedNet(layers, pipeline.calibrate(net, xc, "int8", True))
+    out = fused.forward(torch.zeros(0, 3, 64, 64, device="cuda"))
+    assert tuple(out.shape) == (0, 1000)
+    torch.cuda.synchronize()
