@@ -725,3 +725,78 @@ def test_error_statuses():
     with pytest.raises(Exception):
         cabi.conv2d_nhwc(torch.zeros((1, 2, 2, 4), dtype=torch.int8, device="cuda"),
                          torch.zeros((4, 3, 3, 4), dtype=torch.int8, device="cuda"))  # output extent <= 0
+
+
+# ------------------------------------------------------------------------------ operands of 2 GiB and more
+def _sample_rows(total, block, r):
+    """row blocks at the start, around the 2^31-byte marks and at the end"""
+    starts = {0, total - block}
+    for frac in (0.25, 0.5, 0.75):
+        starts.add(int(total * frac) // 32 * 32)
+    starts.update(int(v) for v in r.integers(0, total - block, 3))
+    return sorted(starts)
+
+
+def test_quantize_more_than_2g_elements():
+    """2^31 + 37 elements: indices beyond 32 bits in the streaming quantizer (fp16 in, int8 out)"""
+    n = 2 ** 31 + 37
+    note("quantize", n)
+    x = torch.empty(n, dtype=torch.float16, device="cuda")
+    x.normal_(0.0, 3.0)
+    q = cabi.quantize(x, 8, -4)
+    torch.cuda.synchronize()
+    r = rng(5)
+    for s in _sample_rows(n, 4096, r) + [n - 4096 - 37, n - 64]:
+        e = min(s + 4096, n)
+        assert same_bits(orc.quantize(x[s:e].cpu().numpy(), 8, -4), q[s:e].cpu().numpy()), s
+    del x, q
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("m,n,k", [(2 ** 25, 16, 64),      # A operand of exactly 2 GiB: beyond the 32-bit buffer offsets
+                                   (2 ** 25 + 40, 160, 16),  # 5.4 G output elements: element indices beyond 32 bits
+                                   (2 ** 22 + 3, 64, 512)])  # 2 GiB A operand with long K: the LDS ring is not eligible
+def test_gemm_operands_beyond_32_bit_offsets(m, n, k):
+    route = cabi.lib().catchq_gemm_route(8, 8, m, n, k)
+    note("gemm beyond 32 bits", m, n, k, route)
+    a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
+    b = torch.randint(-128, 128, (n, k), dtype=torch.int8, device="cuda")
+    r = rng(m % 1000 + n + k)
+    div = r.uniform(0.6, 3.5, n).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    out = cabi.gemm_nt(a, b, exp2=-8, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=1, y_dtype=None, want_acc=False,
+                       q_bw=8, q_pos=-2, chan_rcp=cabi.dev(np.float32(1) / div))
+    torch.cuda.synchronize()
+    bh = b.cpu().numpy()
+    for s in _sample_rows(m, 256, r):  # the rows of a product are independent: check blocks of them
+        acc, _ = orc.gemm_nt(a[s:s + 256].cpu().numpy(), bh)
+        want = orc.quantize(orc.epilogue(acc, -8, div, bias, None, 1), 8, -2)
+        assert same_bits(want, out["q"][s:s + 256].cpu().numpy()), (s, route)
+    del a, out
+    torch.cuda.empty_cache()
+
+
+def test_conv_input_beyond_32_bit_offsets():
+    """a 2.1 GB input image pair: the convolution takes the kernel with 64-bit addressing; horizontal bands of
+    the output (which depend on their own input rows only) against the oracle"""
+    n, h, w, ci, co = 2, 4100, 4096, 64, 16
+    assert n * h * w * ci >= 2 ** 31
+    note("conv beyond 32 bits", (n, h, w, ci, co), cabi.conv_route(8, 8, (n, h, w, ci), (co, 3, 3, ci), (1, 1)))
+    x = torch.randint(-128, 128, (n, h, w, ci), dtype=torch.int8, device="cuda")
+    r = rng(9)
+    wt = _ints(r, (co, 3, 3, ci), 8)
+    bias = r.standard_normal(co).astype(np.float32)
+    out = cabi.conv2d_nhwc(x, cabi.dev(wt), (1, 1), (1, 1), (1, 1), 1, exp2=-12, bias=cabi.dev(bias), act=1, y_dtype=None,
+                           want_acc=False, q_bw=8, q_pos=-1)
+    torch.cuda.synchronize()
+    for img, h0 in ((0, 0), (0, 2047), (1, 1), (1, 2050), (1, h - 6)):
+        lo, hi = max(h0 - 1, 0), min(h0 + 7, h)          # input rows that output rows h0 .. h0+5 read
+        band = x[img:img + 1, lo:hi].cpu().numpy()
+        acc, _ = orc.conv2d_nhwc(band, wt, (1, 1), (1, 1), (1, 1), 1)  # its first / last rows see zero padding instead
+        want = orc.quantize(orc.epilogue(acc, -12, None, bias, None, 1), 8, -1)
+        first = 0 if lo == 0 else 1                        # of the band's output rows, the ones with true neighbours
+        last = want.shape[1] if hi == h else want.shape[1] - 1
+        got = out["q"][img:img + 1, lo + first:lo + last].cpu().numpy()
+        assert same_bits(want[:, first:last], got), (img, h0)
+    del x, out
+    torch.cuda.empty_cache()
