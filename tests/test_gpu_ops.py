@@ -446,3 +446,31 @@ def test_empty_batches():
     out = fused.forward(torch.zeros(0, 3, 64, 64, device="cuda"))
     assert tuple(out.shape) == (0, 1000)
     torch.cuda.synchronize()
+
+
+def test_strided_inputs_equal_their_contiguous_copies():
+    """sliced / transposed / expanded views as input, weight and bias: same results as dense copies"""
+    note("strided inputs")
+    g = torch.Generator().manual_seed(21)
+    big = torch.randn(3, 16, 12, 20, generator=g).cuda()
+    x = big[:, ::2, 1:11, ::2]                      # [3, 8, 10, 10], strided in every dimension
+    wbig = torch.randn(12, 8, 3, 6, generator=g).cuda() * 0.1
+    w = wbig[::2, :, :, ::2]                        # [6, 8, 3, 3]
+    bias = torch.randn(1, generator=g).cuda().expand(6)   # stride 0
+    q_scale = torch.tensor([127.0 / x.abs().max().item(), 127.0 / w.abs().max().item()]).cuda()
+    q_mode = torch.tensor([1], dtype=torch.int32).cuda()
+    args = ([1, 1], [1, 1], [1, 1], 1, q_scale, q_mode)
+    y = torch.ops.torch_mlu.conv2d(x, w, bias, *args)
+    y_ref = torch.ops.torch_mlu.conv2d(x.contiguous(), w.contiguous(), bias.contiguous(), *args)
+    assert torch.equal(y, y_ref)
+    y_cl = torch.ops.torch_mlu.conv2d(x.contiguous(memory_format=torch.channels_last), w.contiguous(), bias.contiguous(), *args)
+    assert torch.equal(y_cl, y_ref)
+    xl = torch.randn(40, 7, generator=g).cuda().t()          # [7, 40], column-major
+    wl = torch.randn(80, 5, generator=g).cuda().t()[:, ::2]  # [5, 40]
+    qs = torch.tensor([127.0 / xl.abs().max().item(), 127.0 / wl.abs().max().item()]).cuda()
+    yl = torch.ops.torch_mlu.linear(xl, wl, bias[:5], qs, q_mode)
+    assert torch.equal(yl, torch.ops.torch_mlu.linear(xl.contiguous(), wl.contiguous(), bias[:5].contiguous(), qs, q_mode))
+    # host-resident q-params are accepted like device-resident ones (the reference copies them to the host itself)
+    assert torch.equal(torch.ops.torch_mlu.linear(xl, wl, bias[:5], qs.cpu(), q_mode.cpu()), yl)
+    qq = torch.ops.torch_mlu.quantize(x, 8, -4)
+    assert torch.equal(qq, torch.ops.torch_mlu.quantize(x.contiguous(), 8, -4))
