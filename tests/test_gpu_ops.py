@@ -474,3 +474,48 @@ def test_strided_inputs_equal_their_contiguous_copies():
     assert torch.equal(torch.ops.torch_mlu.linear(xl, wl, bias[:5], qs.cpu(), q_mode.cpu()), yl)
     qq = torch.ops.torch_mlu.quantize(x, 8, -4)
     assert torch.equal(qq, torch.ops.torch_mlu.quantize(x.contiguous(), 8, -4))
+
+
+def test_ops_from_several_threads():
+    """the prepared-weight cache is shared by every thread of the process: four threads, each on a stream of its
+    own, run one shared and one private layer over and over; every result equals the single-threaded one"""
+    import threading
+    note("threads")
+    g = torch.Generator().manual_seed(33)
+    shared_w = (torch.randn(32, 16, 3, 3, generator=g) * 0.1).cuda()
+    shared_b = torch.randn(32, generator=g).cuda()
+    q_mode = torch.tensor([3], dtype=torch.int32).cuda()
+
+    def qscale(x, w):
+        s_c = 127.0 / w.reshape(w.shape[0], -1).abs().max(1)[0]
+        return torch.cat([torch.tensor([127.0 / x.abs().max().item(), 0.0], device="cuda"), s_c.cuda()])
+    jobs = []
+    for t in range(4):
+        x = torch.randn(2, 16, 20, 20, generator=g).cuda()
+        w = (torch.randn(24, 16, 3, 3, generator=g) * 0.1).cuda()
+        b = torch.randn(24, generator=g).cuda()
+        jobs.append((x, w, b, qscale(x, shared_w), qscale(x, w)))
+    conv = torch.ops.torch_mlu.conv2d
+    want = [(conv(x, shared_w, shared_b, [1, 1], [1, 1], [1, 1], 1, qs_s, q_mode),
+             conv(x, w, b, [1, 1], [2, 2], [1, 1], 1, qs_p, q_mode)) for x, w, b, qs_s, qs_p in jobs]
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(t):
+        x, w, b, qs_s, qs_p = jobs[t]
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for i in range(25):
+                    a = conv(x, shared_w, shared_b, [1, 1], [1, 1], [1, 1], 1, qs_s, q_mode)
+                    c = conv(x, w, b, [1, 1], [2, 2], [1, 1], 1, qs_p, q_mode)
+                    torch.cuda.current_stream().synchronize()
+                    if not (torch.equal(a, want[t][0]) and torch.equal(c, want[t][1])):
+                        errors.append((t, i))
+        except Exception as exc:  # noqa: BLE001
+            errors.append((t, repr(exc)))
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
