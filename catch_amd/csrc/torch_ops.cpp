@@ -11,6 +11,7 @@
 // Device tensors only: there is deliberately no CPU implementation behind these ops (the
 // reference's own CPU fall-back for them returns its input, operators/op_methods.cpp:1019-1035).
 #include <ATen/ATen.h>
+#include <ATen/hip/HIPEvent.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/core/DeviceGuard.h>
 #include <torch/library.h>
@@ -492,6 +493,9 @@ struct Prepared {
   int variant = 0;   // caller's layout choice for qw (part of the cache key)
   Tensor qw;         // conv: [Co,kh,kw,Ci/g]; linear: [N,K]
   Tensor new_scale;  // device fp32 [Co] when per_channel
+  // recorded on the stream that quantized the weight, behind those kernels: a later call on another stream
+  // (another thread's, a side stream) waits for it before it reads qw / new_scale
+  at::cuda::CUDAEvent ready;
   Prepared() : w_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)),
                s_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)),
                m_impl(c10::weak_intrusive_ptr<c10::TensorImpl>::reclaim(nullptr)) {}
@@ -591,12 +595,17 @@ std::shared_ptr<Prepared> prepared_for(const Tensor &weight, const Tensor &q_sca
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
     if (it != g_cache.end()) {
-      if (it->second->variant == variant && still_valid(*it->second, weight, q_scale, q_mode)) return it->second;
+      if (it->second->variant == variant && still_valid(*it->second, weight, q_scale, q_mode)) {
+        if (!it->second->ready.query())  // still in flight on the stream that prepared it
+          it->second->ready.block(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+        return it->second;
+      }
       g_cache.erase(it);
     }
   }
   auto p = prepare(make_dense, weight, q_scale, q_mode);
   p->variant = variant;
+  p->ready.record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
   if (use_cache) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     if (g_cache.size() > 4096) {  // drop entries whose weight is gone

@@ -519,3 +519,41 @@ def test_ops_from_several_threads():
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+def test_first_use_of_a_weight_from_several_streams():
+    """the cache entry of a weight is created by whichever thread comes first, on its stream; the others wait for
+    that stream's quantization kernels before they read the entry"""
+    import threading
+    note("first use from several streams")
+    g = torch.Generator().manual_seed(35)
+    conv = torch.ops.torch_mlu.conv2d
+    q_mode = torch.tensor([3], dtype=torch.int32).cuda()
+    for rep in range(6):
+        w = (torch.randn(512, 256, 3, 3, generator=g) * 0.05).cuda()   # a fresh tensor: nothing cached for it
+        b = torch.randn(512, generator=g).cuda()
+        x = torch.randn(1, 256, 6, 6, generator=g).cuda()
+        s_c = 127.0 / w.reshape(512, -1).abs().max(1)[0]
+        qs = torch.cat([torch.tensor([127.0 / x.abs().max().item(), 0.0], device="cuda"), s_c])
+        torch.cuda.synchronize()
+        outs, errors = [None] * 4, []
+        gate = threading.Barrier(4)
+
+        def work(t):
+            try:
+                with torch.cuda.stream(torch.cuda.Stream()):
+                    gate.wait()
+                    outs[t] = conv(x, w, b, [1, 1], [1, 1], [1, 1], 1, qs, q_mode)
+                    torch.cuda.current_stream().synchronize()
+            except Exception as exc:  # noqa: BLE001
+                errors.append(repr(exc))
+        threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join()
+        assert not errors, errors
+        torch.ops.torch_mlu.clear_weight_cache()
+        want = conv(x, w, b, [1, 1], [1, 1], [1, 1], 1, qs, q_mode)
+        for t in range(4):
+            assert torch.equal(outs[t], want), (rep, t)
