@@ -168,8 +168,10 @@ def main():
         what += ", position + fractional scale"
     fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale)
     xg = x.cuda()
-    if args.streams < 1 or batch % args.streams:
-        sys.exit("--streams must divide the batch (%d)" % batch)
+    if args.streams < 1:
+        sys.exit("--streams must be at least 1")
+    while batch % args.streams:  # the largest number of equal parts not above what was asked for
+        args.streams -= 1
     static_in, replay = fused.capture(xg, streams=args.streams)
     static_in.copy_(xg)
     for _ in range(args.warmup):
