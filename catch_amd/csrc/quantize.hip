@@ -345,7 +345,8 @@ __global__ __launch_bounds__(kThreads) void absmax_finalize_kernel(const float *
     if (absmax > 0.0f && absmax < __builtin_inff()) {
       // floor(log2(absmax)) from the exponent: exact, no transcendental
       pos = ilogbf(absmax) - (bw - 2);
-      scale = __builtin_ldexpf(qmax, pos) / absmax;
+      // absmax * 2^-pos is exact (also for a denormal absmax), so the quotient is rounded once
+      scale = qmax / __builtin_ldexpf(absmax, -pos);
     }
     if (absmax_out) *absmax_out = absmax;
     if (pos_out) *pos_out = pos;

@@ -23,8 +23,15 @@
  *   orc_gemm_nt / orc_conv2d  torch int64 matmul / F.conv2d on int64 (textbook)
  *   orc_epilogue_*            numpy float32 evaluation of the same expression order
  *   orc_f32_to_f16 / f16_to_f32  numpy float16 (exhaustive one way, ties the other)
- *   orc_quantize_param        PARITY UNPINNED: cnnlQuantizeParam's formula is not in
- *                             the tree (internal/quantize_param.cpp:85-94 only calls it)
+ *   orc_quantize_param        cnnlQuantizeParam's own formula is not in the tree
+ *                             (internal/quantize_param.cpp:85-94 only calls it); defined as the
+ *                             position rule of cnnl_util.cpp:337-347 and the scale of
+ *                             jit/utils/utils.cpp:97-100; pinned by frexp (position), the exact
+ *                             rational 2^pos*qmax/absmax rounded once (scale), agreement with
+ *                             orc_quant_params, absmax -> +-qmax, zero / inf / NaN / denormals
+ *   orc_maxpool_nhwc_f32      torch.nn.functional.max_pool2d over (k, stride, pad) grids
+ *   orc_global_avgpool_nhwc_f32  numpy's sequential fp32 cumsum; float64 mean bound; an input on
+ *                             which sequential, pairwise and reversed sums differ
  *   NaN -> 0 in quantize      PARITY UNPINNED (vendor behaviour not stated anywhere)
  *   float order of dequant+bias inside the vendor conv/matmul: PARITY UNPINNED;
  *                             fixed here as cvt(acc) * 2^e [/ new_scale_c] [+ bias] in fp32.
@@ -210,10 +217,12 @@ ORC_API void orc_per_channel_params(int bw, const float *s, int co, int *new_pos
 
 /* position (+scale) from a tensor's max-abs: the role of cnnlQuantizeParam
  * (torch_mlu/csrc/aten/operators/cnnl/internal/quantize_param.cpp:39-96).
- * PARITY UNPINNED: the vendor formula is not in the tree.  Defined here as the
- * exact-exponent form of the position rule above:
+ * The vendor's own formula is not in the tree; defined here by the two formulas the tree does
+ * state for the same quantities (cnnl_util.cpp:337-347; jit/utils/utils.cpp:97-100), in their
+ * exact-exponent form:
  *   pos = floor(log2(absmax)) - (n-2) with floor(log2) taken from the exponent,
- *   scale = 2^pos * qmax / absmax (fp32), offset = 0.   absmax==0 -> pos 0, scale 1. */
+ *   scale = 2^pos * qmax / absmax rounded once to fp32, offset = 0.
+ *   absmax 0, inf or NaN -> pos 0, scale 1. */
 ORC_API void orc_quantize_param(float absmax, int bw, int *pos, float *scale, float *offset) {
   float qmax = (bw == 16) ? 32767.0f : 127.0f;
   int n = (bw == 16) ? 16 : 8;
@@ -223,7 +232,9 @@ ORC_API void orc_quantize_param(float absmax, int bw, int *pos, float *scale, fl
   }
   int p = ilogbf(absmax) - (n - 2);
   *pos = p;
-  *scale = ldexpf(qmax, p) / absmax;
+  /* absmax * 2^-p lies in [2^(n-2), 2^(n-1)): the scaling is exact even for a denormal absmax, so the
+   * quotient is rounded once (2^p * qmax would underflow first for the smallest inputs) */
+  *scale = qmax / ldexpf(absmax, -p);
   *offset = 0.0f;
 }
 

@@ -112,6 +112,14 @@ def test_quantize_param(dtype, n):
     z = torch.zeros(100, device="cuda")
     absmax, pos, scale, _ = cabi.quantize_param(z, 8)
     assert (absmax.item(), pos.item(), scale.item()) == (0.0, 0, 1.0)
+    if dtype is np.float32 and n == 7:
+        # magnitudes at both ends of fp32 (denormals included) and exact powers of two
+        for mag in (1.4e-45, 1e-40, 2.0 ** -126, 2.0 ** -20, 1.0, 2.0 ** 20, 3.0e38, np.inf):
+            t = np.array([0.0, -mag, mag / 2], np.float32)
+            for bw in (8, 16):
+                absmax, pos, scale, _ = cabi.quantize_param(cabi.dev(t), bw)
+                p, s, _ = orc.quantize_param(orc.absmax(t), bw)
+                assert (pos.item(), np.float32(scale.item())) == (p, s), (mag, bw)
 
 
 @pytest.mark.parametrize("bw", [8, 16])

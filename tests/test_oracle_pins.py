@@ -451,3 +451,112 @@ def test_decode_fractional_is_the_exact_step_quantization(per_axis, bw):
     ref = F.conv2d(torch.from_numpy(np.transpose(x, (0, 3, 1, 2)).astype(np.float64)),
                    torch.from_numpy(np.transpose(w, (0, 3, 1, 2)).astype(np.float64)), None, 1, 1).numpy()
     assert _rel_rms(np.transpose(ref, (0, 2, 3, 1)), y) <= (0.03 if bw == 8 else 2e-4)
+
+
+# ---------------------------------------------------------------- position (+ scale) from a tensor's max-abs (A6)
+@pytest.mark.parametrize("bw", [8, 16])
+def test_quantize_param_position_is_the_exponent_and_scale_the_exact_quotient(bw):
+    """What fixes position and scale without the vendor library: the position is the one of
+    get_pos_from_scale_data (cnnl_util.cpp:337-347: floor(log2 absmax) - (n-2), here from frexp, which is
+    exact where the float logarithm is not), and position + scale together map absmax onto qmax
+    (setQuantizedParams, jit/utils/utils.cpp:97-100: scale = 2^pos * qmax / absmax), evaluated in exact
+    rational arithmetic and rounded once to fp32."""
+    from fractions import Fraction
+    qmax = 127 if bw == 8 else 32767
+    n = bw
+    vals = np.concatenate([np.exp(rng.uniform(-30, 30, 3000)),
+                           2.0 ** np.arange(-40, 41),                       # exact powers of two
+                           np.nextafter(np.float32(2.0) ** np.arange(-20, 21, dtype=np.float32), np.float32(0)),
+                           [1e-40, 1.4e-45, 3.0e-39, 3.4e38, 1.0, 127.0, 32767.0]]).astype(np.float32)
+    for a in vals:
+        pos, scale, off = orc.quantize_param(a, bw)
+        m, e = math.frexp(float(a))          # a = m * 2^e, m in [0.5, 1)
+        assert pos == e - 1 - (n - 2), a
+        assert off == 0.0
+        exact = Fraction(2) ** pos * qmax / Fraction(float(a))
+        if exact > Fraction(3.4e38):
+            continue                          # the quotient leaves fp32 (denormal absmax): no finite scale to pin
+        want = np.float32(float(exact)) if exact < Fraction(2) ** 1000 else np.float32(np.inf)
+        # float(Fraction) rounds once to double; the fp32 quotient of two fp32-exact numbers is the
+        # correctly rounded result, which the double detour reproduces except on a double-rounding tie
+        assert abs(float(scale) - float(exact)) <= float(np.spacing(np.float32(float(exact)))) / 2 * (1 + 1e-9), a
+        # scale in (qmax / 2^(n-1), qmax / 2^(n-2)]: the tensor's extreme element lands on +-qmax exactly
+        assert qmax / 2.0 ** (n - 1) * (1 - 1e-6) <= scale <= qmax / 2.0 ** (n - 2) * (1 + 1e-6)
+        assert abs(int(orc.quantize(np.array([a, -a], np.float32), bw, pos, scale)[0])) == qmax
+        # position alone (the eager quantizer's scale = 1) uses at least half of the range
+        q = orc.quantize(np.array([a], np.float32), bw, pos)[0]
+        assert 2 ** (n - 2) <= int(q) <= qmax
+
+
+@pytest.mark.parametrize("bw", [8, 16])
+def test_quantize_param_agrees_with_the_scale_route(bw):
+    """absmax -> (position, scale) must be the same numbers the reference derives from the calibration
+    scale qmax / absmax (orc_quant_params, pinned above), away from exact powers of two where the
+    float logarithm of that route may fall either side."""
+    qmax = 127.0 if bw == 8 else 32767.0
+    for a in np.exp(rng.uniform(-8, 8, 2000)).astype(np.float32):
+        if not 0.5 + 1e-4 < math.frexp(float(a))[0] < 1 - 1e-4:
+            continue
+        pos, scale, _ = orc.quantize_param(a, bw)
+        p2, frac, _ = orc.quant_params(bw, np.float32(qmax) / a)
+        assert pos == p2
+        assert math.isclose(float(scale), float(frac), rel_tol=3e-7)
+
+
+def test_quantize_param_degenerate_inputs():
+    for bw in (8, 16):
+        assert orc.quantize_param(0.0, bw) == (0, 1.0, 0.0)
+        assert orc.quantize_param(np.inf, bw) == (0, 1.0, 0.0)
+        assert orc.quantize_param(np.nan, bw) == (0, 1.0, 0.0)
+    # smallest denormal: exponent -149
+    assert orc.quantize_param(1.4e-45, 8)[0] == -149 - 6
+    assert orc.absmax(np.array([1.0, -3.5, np.nan, 2.0], np.float32)) == 3.5   # NaN is skipped
+    assert orc.absmax(np.zeros(0, np.float32)) == 0.0
+
+
+# ---------------------------------------------------------------- pooling between the quantized ops
+@pytest.mark.parametrize("k,stride,pad", [(2, 2, 0), (3, 2, 1), (3, 1, 1), (2, 1, 1), (5, 1, 2), (3, 3, 0), (4, 2, 2),
+                                          (1, 1, 0), (13, 1, 6), (3, 2, 0)])
+@pytest.mark.parametrize("hw", [(7, 9), (12, 12), (5, 6)])
+def test_maxpool_vs_torch(k, stride, pad, hw):
+    """F.max_pool2d (floor mode, -inf padding) over windows that hang over every border"""
+    h, w = hw
+    if h + 2 * pad < k or w + 2 * pad < k:
+        pytest.skip("window larger than the padded image")
+    x = rng.standard_normal((2, h, w, 5)).astype(np.float32)
+    x[0, 0, 0, :] = 1e30       # corners and edges carry the extreme values
+    x[1, -1, -1, :] = 1e30
+    x[1, 0, -1, 2] = -1e30
+    want = F.max_pool2d(torch.from_numpy(np.transpose(x, (0, 3, 1, 2))), k, stride, pad).numpy()
+    got = orc.maxpool_nhwc(x, k, stride, pad)
+    assert np.array_equal(np.transpose(want, (0, 2, 3, 1)), got)
+    neg = -np.abs(x)            # all-negative input: a zero-valued padding would win, -inf never does
+    want = F.max_pool2d(torch.from_numpy(np.transpose(neg, (0, 3, 1, 2))), k, stride, pad).numpy()
+    assert np.array_equal(np.transpose(want, (0, 2, 3, 1)), orc.maxpool_nhwc(neg, k, stride, pad))
+
+
+def test_global_avgpool_is_the_sequential_fp32_sum():
+    """np.cumsum over fp32 is a sequential left-to-right sum by construction: its last element over the
+    pixel axis, divided once by the pixel count, is the definition; a float64 mean bounds it; and an input
+    built so that sequential, pairwise and reversed summation give three different fp32 results tells
+    the order apart."""
+    x = (rng.standard_normal((3, 7, 7, 11)) * 10).astype(np.float32)
+    got = orc.global_avgpool_nhwc(x)
+    flat = x.reshape(3, 49, 11)
+    want = np.cumsum(flat, axis=1, dtype=np.float32)[:, -1, :] / np.float32(49)
+    assert np.array_equal(want, got)
+    mean64 = flat.astype(np.float64).mean(1)
+    bound = 49 * 2.0 ** -24 * np.abs(flat).astype(np.float64).sum(1) / 49 + 2.0 ** -24 * np.abs(mean64)
+    assert np.all(np.abs(got - mean64) <= bound)
+    # 2^24, 1, 1, 1: left to right every +1 is a tie that rounds back to 2^24 -> 2^24; pairwise
+    # (2^24 + 1) + (1 + 1) -> 2^24 + 2; right to left 1+1+1 = 3, + 2^24 -> 2^24 + 4 (tie to even)
+    c = np.array([2.0 ** 24, 1, 1, 1], np.float32).reshape(1, 2, 2, 1)
+    assert orc.global_avgpool_nhwc(c)[0, 0] == np.float32(2.0 ** 24) / np.float32(4)
+    pair = (c[0, 0, 0, 0] + c[0, 0, 1, 0]) + (c[0, 1, 0, 0] + c[0, 1, 1, 0])
+    rev = ((c[0, 1, 1, 0] + c[0, 1, 0, 0]) + c[0, 0, 1, 0]) + c[0, 0, 0, 0]
+    assert pair == np.float32(2.0 ** 24 + 2) and rev == np.float32(2.0 ** 24 + 4)
+    # one pixel, and the division is a true division (49 is not a power of two)
+    one = rng.standard_normal((2, 1, 1, 4)).astype(np.float32)
+    assert np.array_equal(orc.global_avgpool_nhwc(one), one.reshape(2, 4))
+    t = np.full((1, 7, 7, 1), 0.1, np.float32)
+    assert orc.global_avgpool_nhwc(t)[0, 0] == np.cumsum(t.reshape(-1), dtype=np.float32)[-1] / np.float32(49)
