@@ -53,6 +53,7 @@ CATCHQ_API const char *catchq_status_string(int status) {
     case CATCHQ_ERR_SHAPE: return "inconsistent shapes";
     case CATCHQ_ERR_LAUNCH: return "kernel launch failed";
     case CATCHQ_ERR_UNSUPPORTED: return "combination not supported";
+    case CATCHQ_ERR_TOO_LARGE: return "input larger than the fixed scratch memory of this entry point serves";
     default: return "unknown status";
   }
 }

@@ -1,5 +1,7 @@
 // Streaming quantize / dequantize / max-abs kernels: HBM-bound, 16-byte loads per lane,
 // lane-contiguous so every wave instruction touches whole cache lines.
+#include <mutex>
+
 #include "catchq_common.h"
 
 namespace catchq {
@@ -449,6 +451,46 @@ CATCHQ_API int catchq_quantize_param(const void *x, int x_dtype, int64_t n, int 
                                                mode >= CATCHQ_QUANTIZE_POSITION_SCALE ? scale_dev : nullptr,
                                                mode >= CATCHQ_QUANTIZE_POSITION_SCALE_OFFSET ? offset_dev : nullptr);
   return launch_status();
+}
+
+// ---- the same reduction for callers that cannot allocate ---------------------------------------------------
+// The per-block partial maxima live in a file-scope device array instead of a caller's workspace.  Each
+// device holds its own copy of the array at its own address; host code never uses the array's name as a
+// pointer, only the address hipGetSymbolAddress reports for the current device, looked up once per device.
+static __device__ __align__(256) float scratch[kMaxBlocks];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static float *scratch_ptr[kMaxDevices];  // guarded by scratch_mutex
+
+static int scratch_for_current_device(float **out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return CATCHQ_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return CATCHQ_ERR_LAUNCH;
+    }
+    scratch_ptr[dev] = static_cast<float *>(p);
+  }
+  *out = scratch_ptr[dev];
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_quantize_param_noalloc(const void *x, int x_dtype, int64_t n, int bitwidth, int mode,
+                                             float *absmax_dev, int32_t *position_dev, float *scale_dev,
+                                             float *offset_dev, catchq_stream_t stream) {
+  if (n < 0 || (n > 0 && !x)) return CATCHQ_ERR_ARG;
+  if (n > CATCHQ_QUANTIZE_PARAM_NOALLOC_MAX_N) return CATCHQ_ERR_TOO_LARGE;
+  float *partial = nullptr;
+  const int st = scratch_for_current_device(&partial);
+  if (st != CATCHQ_OK) return st;
+  // every block writes its own slot before the finalize kernel reads exactly those slots: nothing of an
+  // earlier call's contents is ever read, so nothing needs clearing
+  return catchq_quantize_param(x, x_dtype, n, bitwidth, mode, partial, sizeof(float) * (size_t)kMaxBlocks,
+                               absmax_dev, position_dev, scale_dev, offset_dev, stream);
 }
 
 CATCHQ_API int catchq_quantize_per_channel(const void *w, int w_dtype, void *q, int bitwidth, int co,

@@ -10,7 +10,10 @@
  *   - plain pointers and sizes only; every device buffer (inputs, outputs,
  *     workspace) is owned by the caller; nothing here allocates or frees;
  *   - all device entry points are asynchronous on `stream` (a hipStream_t passed
- *     as void*; NULL = the null stream) and keep no mutable global state;
+ *     as void*; NULL = the null stream).  They are re-entrant and keep no state from call to
+ *     call, with two documented exceptions: the planning hint catchq_set_launch_sharing
+ *     (process-wide, affects speed only) and the fixed scratch memory of
+ *     catchq_quantize_param_noalloc (per device, calls on one device must not overlap);
  *   - the return value is a status (0 = CATCHQ_OK); no exception crosses the
  *     boundary; catchq_status_string() names a status;
  *   - activations are NHWC, convolution weights [Co][kh][kw][Ci/groups]
@@ -36,7 +39,8 @@ enum {
   CATCHQ_ERR_BITWIDTH = 3,    /* "bitwidth not support" (operators/cnnl/internal/quantify.cpp:63) */
   CATCHQ_ERR_SHAPE = 4,       /* inconsistent shapes (groups, output extent <= 0, ...) */
   CATCHQ_ERR_LAUNCH = 5,      /* the HIP runtime refused the launch */
-  CATCHQ_ERR_UNSUPPORTED = 6  /* combination not implemented */
+  CATCHQ_ERR_UNSUPPORTED = 6, /* combination not implemented */
+  CATCHQ_ERR_TOO_LARGE = 7    /* input larger than the fixed scratch memory of a *_noalloc entry point serves */
 };
 
 enum { CATCHQ_F32 = 0, CATCHQ_F16 = 1 };
@@ -106,6 +110,21 @@ int catchq_quantize_param_workspace_size(int64_t n, size_t *bytes);
 int catchq_quantize_param(const void *x, int x_dtype, int64_t n, int bitwidth, int mode, void *workspace,
                           size_t workspace_bytes, float *absmax_dev, int32_t *position_dev,
                           float *scale_dev, float *offset_dev, catchq_stream_t stream);
+
+/* catchq_quantize_param for callers that cannot allocate device memory or bring a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference, whose wrapper allocates the vendor workspace on every call (operators/cnnl/internal/quantize_param.cpp:67-83).
+ * Same kernels, same results bit for bit; the per-block partial maxima go to a fixed 16 KiB array in
+ * device memory that every device the library runs on holds until the process ends.  The call allocates
+ * and frees nothing.  n above CATCHQ_QUANTIZE_PARAM_NOALLOC_MAX_N returns CATCHQ_ERR_TOO_LARGE.  All
+ * calls on one device share that array: two calls whose kernels may run at the same time on one device
+ * (different streams, different threads) race; calls on one stream are ordered and safe.  Nothing of an
+ * earlier call's contents is read, so no clearing happens between calls.  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress); make that call outside a stream capture. */
+#define CATCHQ_QUANTIZE_PARAM_NOALLOC_MAX_N (INT64_C(1) << 40)
+int catchq_quantize_param_noalloc(const void *x, int x_dtype, int64_t n, int bitwidth, int mode,
+                                  float *absmax_dev, int32_t *position_dev, float *scale_dev,
+                                  float *offset_dev, catchq_stream_t stream);
 
 /* the elementwise part of cnnl_quantify_per_channel        operators/cnnl/quantify.cpp:100-112
  * q[c, i] = sat(rne(w[c, i] / scale_factor[c])), w [co, inner] fp32/fp16, scale_factor on the device. */
