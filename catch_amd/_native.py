@@ -56,6 +56,8 @@ SIGNATURES = {
     "catchq_quantize_param": (_I, [_P, _I, _I64, _I, _I, _P, _SZ, _P, _P, _P, _P, _P]),
     "catchq_quantize_param_noalloc": (_I, [_P, _I, _I64, _I, _I, _P, _P, _P, _P, _P]),
     "catchq_quantize_per_channel": (_I, [_P, _I, _P, _I, _I, _I64, _P, _P]),
+    "catchq_quantize_per_channel_f16": (_I, [_P, _P, _I, _I, _I64, _P, _P]),
+    "catchq_per_channel_params_f16": (_I, [_I, _P, _I, ctypes.POINTER(_I), _P, _P]),
     "catchq_dequantize": (_I, [_P, _I, _P, _I, _I64, _I, _F, _P]),
     "catchq_gemm_nt": (_I, [_P, _I, _P, _I, _I64, _I64, _I64, ctypes.POINTER(Epilogue), _P]),
     "catchq_conv_out_size": (_I, [_I] * 5),

@@ -125,12 +125,18 @@ class MLUConvNd(torch.nn.Module, MLUModel):
                ", scale={}, quantized_mode={}".format(self.scale, self.quantized_mode)
 
     def _apply(self, fn, recurse=True):
-        # q_scale stays fp32 under .half(): int16 scales (32767/absmax) overflow fp16
+        # The reference has no override: .half() turns the q-params into half tensors, and its per-channel
+        # derivation then runs in half as well.  That is followed for int8, where half holds every number of
+        # that derivation.  int16 q-params stay fp32: 32767 / absmax exceeds the largest half for absmax < 0.5,
+        # and half holds neither 32767 nor the integers above 2048.
         kept = None if self.scale is None else self.scale.detach().clone()
         super()._apply(fn)
         if kept is not None and self.scale is not None and self.scale.dtype != torch.float32:
-            self.scale = Parameter(kept.detach().to(device=self.scale.device, dtype=torch.float32),
-                                   requires_grad=False)
+            int8 = self.quantized_mode is not None and self.quantized_mode.numel() == 1 \
+                and int(self.quantized_mode.flatten()[0]) in (1, 3)
+            if not int8 or not bool(torch.isfinite(self.scale.float()).all()):
+                self.scale = Parameter(kept.detach().to(device=self.scale.device, dtype=torch.float32),
+                                       requires_grad=False)
         return self
 
     def _get_name(self):

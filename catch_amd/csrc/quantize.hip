@@ -272,6 +272,23 @@ __global__ __launch_bounds__(kThreads) void quantize_per_channel_kernel(const TI
   }
 }
 
+// the all-half form: weight, scale factor and their quotient are binary16 (the quotient of two halves,
+// evaluated in fp32 and rounded to binary16, is the correctly rounded half quotient), then round + clamp
+template <int BW>
+__global__ __launch_bounds__(kThreads) void quantize_per_channel_f16_kernel(const __half *__restrict__ w,
+                                                                           typename QRange<BW>::type *__restrict__ q,
+                                                                           int64_t total, int64_t inner,
+                                                                           const __half *__restrict__ sf) {
+  typedef typename QRange<BW>::type TQ;
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const float t = __half2float(__float2half_rn(__half2float(w[i]) / __half2float(sf[i / inner])));
+    float r = __builtin_rintf(t);
+    r = fminf(fmaxf(r, QRange<BW>::lo), QRange<BW>::hi);
+    q[i] = (t != t) ? (TQ)0 : (TQ)(int)r;
+  }
+}
+
 // ---- dequantize: y = q * 2^pos / scale ------------------------------------------------------------
 template <typename TQ, typename TOut>
 __global__ __launch_bounds__(kThreads) void dequantize_kernel(const TQ *__restrict__ q, TOut *__restrict__ y,
@@ -511,6 +528,24 @@ CATCHQ_API int catchq_quantize_per_channel(const void *w, int w_dtype, void *q, 
     if (bitwidth == 8) quantize_per_channel_kernel<__half, 8><<<g, kThreads, 0, s>>>((const __half *)w, (int8_t *)q, total, inner, scale_factor_dev);
     else quantize_per_channel_kernel<__half, 16><<<g, kThreads, 0, s>>>((const __half *)w, (int16_t *)q, total, inner, scale_factor_dev);
   }
+  return launch_status();
+}
+
+CATCHQ_API int catchq_quantize_per_channel_f16(const void *w, void *q, int bitwidth, int co, int64_t inner,
+                                               const void *scale_factor_dev, catchq_stream_t stream) {
+  if (co < 0 || inner < 0) return CATCHQ_ERR_SHAPE;
+  if (bitwidth != 8 && bitwidth != 16) return CATCHQ_ERR_BITWIDTH;
+  const int64_t total = (int64_t)co * inner;
+  if (total == 0) return CATCHQ_OK;
+  if (!w || !q || !scale_factor_dev) return CATCHQ_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const int g = grid_for(total, kThreads * 4);
+  if (bitwidth == 8)
+    quantize_per_channel_f16_kernel<8><<<g, kThreads, 0, s>>>((const __half *)w, (int8_t *)q, total, inner,
+                                                              (const __half *)scale_factor_dev);
+  else
+    quantize_per_channel_f16_kernel<16><<<g, kThreads, 0, s>>>((const __half *)w, (int16_t *)q, total, inner,
+                                                               (const __half *)scale_factor_dev);
   return launch_status();
 }
 

@@ -114,6 +114,7 @@ struct PerChannel {
   int new_pos = 0;
   Tensor new_scale;     // device fp32 [Co]
   Tensor scale_factor;  // device fp32 [Co]
+  Tensor scale_factor_h;  // device fp16 [Co]: set when the parameters were derived in binary16
 };
 
 PerChannel per_channel_params(const float *scales_host, int64_t co, int bw, const at::TensorOptions &dev_opts) {
@@ -127,10 +128,53 @@ PerChannel per_channel_params(const float *scales_host, int64_t co, int bw, cons
   return pc;
 }
 
+// scales: a half tensor (any device).  The reference derives the parameters in the dtype of the scales
+// (operators/cnnl/quantify.cpp:64-98), so a model converted with .half() gets them rounded to binary16 step
+// by step; new_scale and scale_factor come back as the fp32 images of those binary16 values.
+PerChannel per_channel_params_half(const Tensor &scales, int bw, const at::TensorOptions &dev_opts) {
+  Tensor s_host = scales.to(at::kCPU).contiguous();
+  const int64_t co = s_host.numel();
+  Tensor ns = at::empty({co}, at::TensorOptions().dtype(at::kHalf));
+  Tensor sf = at::empty({co}, at::TensorOptions().dtype(at::kHalf));
+  PerChannel pc;
+  const int st = catchq_per_channel_params_f16(bw, reinterpret_cast<const uint16_t *>(s_host.data_ptr<at::Half>()),
+                                               (int)co, &pc.new_pos,
+                                               reinterpret_cast<uint16_t *>(ns.data_ptr<at::Half>()),
+                                               reinterpret_cast<uint16_t *>(sf.data_ptr<at::Half>()));
+  TORCH_CHECK(st == CATCHQ_OK,
+              "per-channel scales held in half precision must be finite and positive there (an int", bw,
+              " scale ", bw == 16 ? "32767" : "127", "/absmax above 65504 is inf in half): keep q_scale in float");
+  pc.new_scale = ns.to(at::kFloat).to(dev_opts.device(), false);
+  pc.scale_factor = sf.to(at::kFloat).to(dev_opts.device(), false);
+  pc.scale_factor_h = sf.to(dev_opts.device(), false);
+  return pc;
+}
+
+// Whether the per-channel parameters are derived with half tensor ops like the reference does for a model
+// converted with .half().  int8 only: every constant of the chain (127, the quotients up to 127 in steps of
+// 1/16) is a half number.  For int16 half holds neither 32767 nor the integers above 2048, so what the
+// reference's half chain yields there depends on how the device clamps and casts 32768.0; those scales are
+// read as fp32 values and the derivation runs in fp32.  A half scale that is inf or NaN is refused either way.
+bool half_chain(const Tensor &scales, int bw) {
+  if (scales.scalar_type() != at::kHalf) return false;
+  TORCH_CHECK(at::isfinite(scales).all().item<bool>(),
+              "q_scale is held in half precision and is not finite there (an int16 scale 32767/absmax above 65504 "
+              "becomes inf in half): keep q_scale in float");
+  return bw == 8;
+}
+
 Tensor quantize_weight_per_channel(const Tensor &w_dense, const PerChannel &pc, int bw) {
   const int dt = fp_dtype(w_dense, "quantify only support input float/half");
   Tensor q = at::empty_like(w_dense, w_dense.options().dtype(int_type(bw)));
   const int64_t co = w_dense.size(0);
+  if (pc.scale_factor_h.defined() && dt == CATCHQ_F16) {
+    // half weight / half scale_factor: the quotient is a half tensor too (quantify.cpp:104)
+    check_status(catchq_quantize_per_channel_f16(w_dense.data_ptr(), q.data_ptr(), bw, (int)co,
+                                                 co ? w_dense.numel() / co : 0, pc.scale_factor_h.data_ptr(),
+                                                 current_stream()),
+                 "torch_mlu::quantize_per_channel");
+    return q;
+  }
   check_status(catchq_quantize_per_channel(w_dense.data_ptr(), dt, q.data_ptr(), bw, (int)co,
                                            co ? w_dense.numel() / co : 0, pc.scale_factor.data_ptr<float>(),
                                            current_stream()),
@@ -143,13 +187,19 @@ std::tuple<Tensor, Tensor, Tensor> quantize_per_channel_op(const Tensor &w, cons
   TORCH_CHECK(bitwidth == 8 || bitwidth == 16, "bitwidth not support");
   TORCH_CHECK(w.dim() >= 1 && scales.numel() == w.size(0), "one scale per output channel expected");
   c10::DeviceGuard guard(w.device());
-  Tensor s_host = scales.to(at::kCPU, at::kFloat).contiguous();
-  PerChannel pc = per_channel_params(s_host.data_ptr<float>(), s_host.numel(), (int)bitwidth, w.options());
+  PerChannel pc;
+  if (half_chain(scales, (int)bitwidth)) {
+    pc = per_channel_params_half(scales, (int)bitwidth, w.options());
+  } else {
+    Tensor s_host = scales.to(at::kCPU, at::kFloat).contiguous();
+    pc = per_channel_params(s_host.data_ptr<float>(), s_host.numel(), (int)bitwidth, w.options());
+  }
   // dim 0 must be the slowest-varying dimension of the memory: true for contiguous and channels-last
   Tensor wd = w.is_non_overlapping_and_dense() && w.stride(0) * w.size(0) == w.numel() ? w : w.contiguous();
   Tensor q = quantize_weight_per_channel(wd, pc, (int)bitwidth);
-  Tensor new_pos = at::full({1}, (double)pc.new_pos, w.options().dtype(at::kFloat));
-  return std::make_tuple(q, new_pos, pc.new_scale);
+  // new_position and new_scale in the dtype of the scales, as the reference's tensor ops leave them
+  Tensor new_pos = at::full({1}, (double)pc.new_pos, w.options().dtype(scales.scalar_type() == at::kHalf ? at::kHalf : at::kFloat));
+  return std::make_tuple(q, new_pos, scales.scalar_type() == at::kHalf ? pc.new_scale.to(at::kHalf) : pc.new_scale);
 }
 
 Tensor dequantize_op(const Tensor &q, int64_t position, double scale, bool half) {
@@ -564,7 +614,9 @@ std::shared_ptr<Prepared> prepare(MakeDense make_dense, const Tensor &weight, co
     } else {
       const int64_t co = w_dense.size(0);
       TORCH_CHECK(s_host.numel() == 2 + co, "per-channel q_scale must hold 2 + ", co, " values, got ", s_host.numel());
-      PerChannel pc = per_channel_params(s + 2, co, bw, w_dense.options());
+      PerChannel pc = half_chain(q_scale, bw)
+                          ? per_channel_params_half(q_scale.reshape({-1}).slice(0, 2), bw, w_dense.options())
+                          : per_channel_params(s + 2, co, bw, w_dense.options());
       p->pos_w = pc.new_pos;
       p->new_scale = pc.new_scale;
       p->qw = quantize_weight_per_channel(w_dense, pc, bw);

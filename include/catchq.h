@@ -72,6 +72,13 @@ int catchq_quant_params(int bitwidth, float scale, int *position, float *scale_f
 int catchq_per_channel_params(int bitwidth, const float *scales, int co, int *new_position,
                               float *new_scale, float *scale_factor);
 
+/* The same derivation for a model converted with .half(): scale_data is then a half tensor and every
+ * tensor op of operators/cnnl/quantify.cpp:64-98 rounds to binary16 (absmax, log2, position, scale, new_scale,
+ * scale_factor).  scales / new_scale / scale_factor hold binary16 bit patterns (host arrays).  A scale that is
+ * not finite in binary16 (an int16 scale 32767/absmax above 65504) returns CATCHQ_ERR_ARG. */
+int catchq_per_channel_params_f16(int bitwidth, const uint16_t *scales, int co, int *new_position,
+                                  uint16_t *new_scale, uint16_t *scale_factor);
+
 /* ------------------------------------------------------------------ quantize / dequantize */
 
 /* cnnl_quantify_offline_internal(input, bitwidth, int position) -> cnnlQuantizeV1
@@ -130,6 +137,12 @@ int catchq_quantize_param_noalloc(const void *x, int x_dtype, int64_t n, int bit
  * q[c, i] = sat(rne(w[c, i] / scale_factor[c])), w [co, inner] fp32/fp16, scale_factor on the device. */
 int catchq_quantize_per_channel(const void *w, int w_dtype, void *q, int bitwidth, int co, int64_t inner,
                                 const float *scale_factor_dev, catchq_stream_t stream);
+
+/* The same with half tensors on both sides (weight and scale_factor binary16, as after .half()): the quotient
+ * w / scale_factor is itself a half tensor in operators/cnnl/quantify.cpp:104, i.e. it is rounded to binary16
+ * before round() and clamp() see it.  scale_factor_dev holds binary16 values. */
+int catchq_quantize_per_channel_f16(const void *w, void *q, int bitwidth, int co, int64_t inner,
+                                    const void *scale_factor_dev, catchq_stream_t stream);
 
 /* explicit form of the dequantization the reference leaves to the vendor conv/matmul descriptors
  * (cnnl/cnnlTensorDescriptors.cpp:175-184) : y[i] = q[i] * 2^position / scale; q int8/int16/int32

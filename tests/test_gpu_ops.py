@@ -15,6 +15,7 @@ import torch.nn.functional as F
 
 import oracle as orc
 from oracle import ops as oops
+from oracle import ref_order
 
 pytestmark = pytest.mark.gpu
 
@@ -70,11 +71,25 @@ def test_conv2d_qint_grid(bias, bw, per_channel, half):
     assert got.shape == (3, 64, 10, 10) and got.dtype == xin.dtype
     assert got.is_contiguous(memory_format=torch.channels_last)
     b = conv.bias.detach().float().cpu().numpy()
-    ref = oops.conv2d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), b, (3, 3), (3, 3), (1, 1), 1,
-                      conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
-    if not half:  # a half model carries half weights: the oracle sees the same rounded values above
-        assert same_bits(ref["y"], got.cpu().numpy())
+    # .half() turns the q-params into half tensors too, as in the reference, unless half cannot hold them
+    # (int16 scales of weights below 0.5 are inf there: those stay fp32)
+    assert (conv.scale.dtype == torch.float16) == (half and bw == "int8")  # int16 q-params stay fp32
+    if half and per_channel and conv.scale.dtype == torch.float16:
+        # the reference's all-half order (quantify.cpp:55-114 and quantify_conv_forward.cpp:123-129 on half
+        # tensors): same integers bit for bit; the output, rounded once here and three times there, within
+        # 1e-3 of its range
+        r = ref_order.conv2d_per_channel(xin, conv.weight.detach().cpu(), conv.bias.detach().cpu(), (3, 3), (3, 3),
+                                         (1, 1), 1, conv.scale.detach().cpu(), conv.quantized_mode.cpu().numpy())
+        q, new_pos, new_scale = torch.ops.torch_mlu.quantize_per_channel(conv.weight.detach(), conv.scale.detach()[2:], 8)
+        assert same_bits(r["qw"], q.permute(0, 2, 3, 1).contiguous().cpu().numpy())
+        assert int(new_pos.item()) == r["new_pos"] and torch.equal(new_scale.cpu(), r["new_scale"])
+        want = r["y"].float().numpy()
+        err = np.abs(got.float().cpu().numpy() - want).max()
+        assert err <= 1e-3 * (want.max() - want.min()), err / (want.max() - want.min())
     else:
+        ref = oops.conv2d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), b, (3, 3), (3, 3), (1, 1), 1,
+                          conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
+        # a half model carries half weights: the oracle sees the same rounded values
         assert same_bits(ref["y"], got.cpu().numpy())
     assert rel_rms(want_float, got.float().cpu().numpy()) <= 0.02
 
@@ -97,10 +112,17 @@ def test_linear_qint_grid(bias, ni, ci, co):
         qmodel.to("cuda")
         got = qmodel(xin.to("cuda"))
         assert got.dtype == torch.float32 and got.shape == (ni, co)  # fp32 whatever the input type
-        ref = oops.linear(xin.numpy(), lin.weight.detach().float().cpu().numpy(),
-                          lin.bias.detach().float().cpu().numpy(), lin.scale.detach().float().cpu().numpy(),
-                          lin.quantized_mode.cpu().numpy())
-        assert same_bits(ref["y"], got.cpu().numpy()), (bw, per_channel, half)
+        if half and per_channel and lin.scale.dtype == torch.float16:
+            # all-half parameters and weight quotient, fp32 output arithmetic (linear.cpp:54-59 after matmul.cpp:72-74):
+            # nothing is left to tolerance
+            r = ref_order.linear_per_channel(xin, lin.weight.detach().cpu(), lin.bias.detach().cpu(),
+                                             lin.scale.detach().cpu(), lin.quantized_mode.cpu().numpy())
+            assert same_bits(r["y"].numpy(), got.cpu().numpy()), (bw, per_channel, half)
+        else:
+            ref = oops.linear(xin.numpy(), lin.weight.detach().float().cpu().numpy(),
+                              lin.bias.detach().float().cpu().numpy(), lin.scale.detach().float().cpu().numpy(),
+                              lin.quantized_mode.cpu().numpy())
+            assert same_bits(ref["y"], got.cpu().numpy()), (bw, per_channel, half)
         assert rel_rms(want_float, got.cpu().numpy()) <= 0.02, (bw, per_channel, half)
 
 
@@ -279,9 +301,18 @@ def test_conv1d_module_swap(bw, per_channel, half):
         qmodel.half()
     got = qmodel.to("cuda")(xin.to("cuda"))
     assert got.shape == want_float.shape and got.dtype == xin.dtype
-    ref = oops.conv1d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
-                      (3,), (2,), (2,), 2, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
-    assert same_bits(ref["y"], got.cpu().numpy())
+    if half and per_channel:
+        # all-half model: the reference's half tensor ops (the 1-d convolution as images of one row)
+        assert conv.scale.dtype == torch.float16
+        r = ref_order.conv2d_per_channel(xin[:, :, None, :], conv.weight.detach().cpu()[:, :, None, :],
+                                         conv.bias.detach().cpu(), (0, 3), (1, 2), (1, 2), 2, conv.scale.detach().cpu(),
+                                         conv.quantized_mode.cpu().numpy())
+        want = r["y"][:, :, 0, :].float().numpy()
+        assert np.abs(got.float().cpu().numpy() - want).max() <= 1e-3 * (want.max() - want.min())
+    else:
+        ref = oops.conv1d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
+                          (3,), (2,), (2,), 2, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
+        assert same_bits(ref["y"], got.cpu().numpy())
     assert rel_rms(want_float, got.float().cpu().numpy()) <= 0.02
 
 
@@ -398,9 +429,14 @@ def test_conv2d_first_qint(k, co, h, w):
     # exact: the oracle on the tensor the module hands to the op
     x_norm = ((raw.half().cuda() - conv.input_mean) / conv.input_std)
     assert x_norm.dtype == torch.float16
-    ref = oops.conv2d(x_norm.cpu().numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
-                      (2, 2), (1, 4), (1, 1), 1, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
-    assert same_bits(ref["y"], got.cpu().numpy())
+    # the all-half model against the reference's half tensor ops: same integers, output within 1e-3 of its range
+    assert conv.scale.dtype == torch.float16
+    r = ref_order.conv2d_per_channel(x_norm.cpu(), conv.weight.detach().cpu(), conv.bias.detach().cpu(), (2, 2), (1, 4),
+                                     (1, 1), 1, conv.scale.detach().cpu(), conv.quantized_mode.cpu().numpy())
+    q = torch.ops.torch_mlu.quantize_per_channel(conv.weight.detach(), conv.scale.detach()[2:], 8)[0]
+    assert same_bits(r["qw"], q.permute(0, 2, 3, 1).contiguous().cpu().numpy())
+    want = r["y"].float().numpy()
+    assert np.abs(got.float().cpu().numpy() - want).max() <= 1e-3 * (want.max() - want.min())
 
 
 def test_empty_batches():
@@ -557,3 +593,27 @@ def test_first_use_of_a_weight_from_several_streams():
         want = conv(x, w, b, [1, 1], [1, 1], [1, 1], 1, qs, q_mode)
         for t in range(4):
             assert torch.equal(outs[t], want), (rep, t)
+
+
+def test_half_q_scale_that_half_cannot_hold_is_refused():
+    """an int16 per-channel scale 32767 / absmax is inf in half for absmax < 0.5: the op says so instead of
+    deriving positions from inf (the module keeps such a q_scale in fp32 under .half())"""
+    note("half q_scale overflow")
+    torch.manual_seed(5)
+    x = torch.randn(2, 16, 8, 8).half().cuda()
+    w = (torch.randn(16, 16, 3, 3) * 0.05).half().cuda()
+    b = torch.zeros(16).half().cuda()
+    s_c = 32767.0 / w.float().reshape(16, -1).abs().max(1)[0]
+    q_scale = torch.cat([torch.tensor([32767.0 / 4.0, 0.0], device="cuda"), s_c]).half()
+    assert torch.isinf(q_scale).any()
+    with pytest.raises(RuntimeError, match="half"):
+        torch.ops.torch_mlu.conv2d(x, w, b, [1, 1], [1, 1], [1, 1], 1, q_scale, torch.tensor([4], dtype=torch.int32))
+    # weights of magnitude >= 0.5: every int16 scale fits half; int16 parameters are still derived in fp32, from
+    # the values the half tensor holds (half has neither 32767 nor the integers above 2048)
+    w2 = (torch.randn(16, 16, 3, 3) * 0.5).half().cuda()
+    s2 = torch.cat([torch.tensor([32767.0 / 4.0, 0.0], device="cuda"), 32767.0 / w2.float().reshape(16, -1).abs().max(1)[0]]).half()
+    assert torch.isfinite(s2).all()
+    got = torch.ops.torch_mlu.conv2d(x, w2, b, [1, 1], [1, 1], [1, 1], 1, s2, torch.tensor([4], dtype=torch.int32))
+    ref = oops.conv2d(x.cpu().numpy(), w2.float().cpu().numpy(), b.float().cpu().numpy(), (1, 1), (1, 1), (1, 1), 1,
+                      s2.float().cpu().numpy(), [4])
+    assert same_bits(ref["y"], got.cpu().numpy())

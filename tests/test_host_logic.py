@@ -261,3 +261,31 @@ def test_lrn_and_norm_observers():
     nr = sq.sum(1).sqrt() + 1e-10
     assert norm.boundary_1 == [sq.min().item(), sq.max().item()] and norm.boundary_2 == [nr.min().item(), nr.max().item()]
     assert norm.scale == [32767.0 / sq.max().item(), 32767.0 / nr.max().item()]
+
+
+def test_per_channel_params_in_half_follow_the_tensor_ops(lib):
+    """A .half() model derives the per-channel parameters with half tensors (quantify.cpp:64-98 in the dtype of
+    scale_data).  The shipped host routine rounds every step to binary16 by hand; torch's CPU half kernels,
+    applied expression by expression (oracle/ref_order.py), are the independent statement of the same chain."""
+    from oracle import ref_order
+    r = np.random.default_rng(5)
+    for bw in (8, 16):
+        qmax = 127.0 if bw == 8 else 32767.0
+        for co in (1, 7, 64, 513):
+            absmax = np.exp(r.uniform(np.log(0.6 if bw == 16 else 0.003), np.log(40.0), co))
+            s = torch.from_numpy((qmax / absmax).astype(np.float32)).half()
+            assert torch.isfinite(s).all()
+            sb = s.numpy().view(np.uint16).copy()
+            ns, sf = np.empty_like(sb), np.empty_like(sb)
+            p = ctypes.c_int()
+            assert lib.catchq_per_channel_params_f16(bw, sb.ctypes.data, co, ctypes.byref(p), ns.ctypes.data,
+                                                     sf.ctypes.data) == 0
+            w = torch.zeros(co, 2).half()
+            _, want_pos, want_ns = ref_order.quantify_per_channel(w, s, bw)
+            assert p.value == int(want_pos.float()[0])
+            assert np.array_equal(ns.view(np.float16), want_ns.numpy())
+    # a scale that half cannot hold is refused, not turned into garbage
+    bad = np.array([np.float16(np.inf)]).view(np.uint16)
+    out = np.empty(1, np.uint16)
+    p = ctypes.c_int()
+    assert lib.catchq_per_channel_params_f16(16, bad.ctypes.data, 1, ctypes.byref(p), out.ctypes.data, out.ctypes.data) == 1

@@ -560,3 +560,58 @@ def test_global_avgpool_is_the_sequential_fp32_sum():
     assert np.array_equal(orc.global_avgpool_nhwc(one), one.reshape(2, 4))
     t = np.full((1, 7, 7, 1), 0.1, np.float32)
     assert orc.global_avgpool_nhwc(t)[0, 0] == np.cumsum(t.reshape(-1), dtype=np.float32)[-1] / np.float32(49)
+
+
+# ---------------------------------------------------------------- the reference's tensor-op order, dtype by dtype
+@pytest.mark.parametrize("bw", [8, 16])
+def test_tensor_op_restatement_equals_the_c_oracle_in_fp32(bw):
+    """oracle/ref_order.py spells the per-channel branches out of torch tensor ops the way the reference does
+    (quantify.cpp:55-114; quantify_conv_forward.cpp:107-131; linear.cpp:40-70).  With fp32 tensors it must give
+    the numbers of the C restatement bit for bit -- two independent statements of the same lines."""
+    from oracle import ref_order
+    g = torch.Generator().manual_seed(3 + bw)
+    qmax = 127.0 if bw == 8 else 32767.0
+    x = torch.randn(3, 64, 24, 24, generator=g)
+    w = torch.randn(64, 64, 3, 3, generator=g) * 0.04 * (torch.rand(64, 1, 1, 1, generator=g) * 4 + 0.1)
+    b = torch.randn(64, generator=g)
+    q_scale = torch.cat([torch.tensor([qmax / x.abs().max().item(), 0.0]), qmax / w.reshape(64, -1).abs().max(1)[0]]).float()
+    mode = [3 if bw == 8 else 4]
+    r = ref_order.conv2d_per_channel(x, w, b, (3, 3), (3, 3), (1, 1), 1, q_scale, mode)
+    o = oops.conv2d(x.numpy(), w.numpy(), b.numpy(), (3, 3), (3, 3), (1, 1), 1, q_scale.numpy(), mode)
+    assert r["new_pos"] == o["pos_w"] and np.array_equal(r["new_scale"].numpy(), o["new_scale"])
+    assert np.array_equal(r["qw"], o["qw"]) and np.array_equal(r["qx"], o["qx"])
+    assert np.array_equal(r["y"].numpy(), o["y"])
+    xl, wl = torch.randn(20, 100, generator=g), torch.randn(125, 100, generator=g) * 0.1
+    bl = torch.randn(125, generator=g)
+    qs = torch.cat([torch.tensor([qmax / xl.abs().max().item(), 0.0]), qmax / wl.abs().max(1)[0]]).float()
+    rl = ref_order.linear_per_channel(xl, wl, bl, qs, mode)
+    ol = oops.linear(xl.numpy(), wl.numpy(), bl.numpy(), qs.numpy(), mode)
+    assert np.array_equal(rl["qw"], ol["qw"]) and np.array_equal(rl["y"].numpy(), ol["y"])
+
+
+def test_half_order_of_the_reference_what_it_changes():
+    """A .half() model rounds to half after every tensor op.  Measured against the single-rounding fp32
+    evaluation of the same half inputs: with the q-params kept in fp32 the integers are the same and the
+    output moves by a few 1e-4 of its range; with the q-params in half as well, the weight quotient's
+    rounding to half moves some weights by one step, which is quantization noise (1e-3 of the range)."""
+    from oracle import ref_order
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(3, 64, 24, 24, generator=g)
+    w = torch.randn(64, 64, 3, 3, generator=g) * 0.04
+    b = torch.randn(64, generator=g)
+    q_scale = torch.cat([torch.tensor([127.0 / x.abs().max().item(), 0.0]), 127.0 / w.reshape(64, -1).abs().max(1)[0]]).float()
+    args = ((3, 3), (3, 3), (1, 1), 1)
+    single = oops.conv2d(x.half().numpy(), w.half().numpy(), b.half().numpy(), *args, q_scale.numpy(), [3])
+    span = float(single["y"].astype(np.float32).max() - single["y"].astype(np.float32).min())
+    mixed = ref_order.conv2d_per_channel(x.half(), w.half(), b.half(), *args, q_scale, [3])
+    assert mixed["y"].dtype == torch.float32            # half / float promotes (output / new_scale, :127)
+    assert np.array_equal(mixed["qw"], single["qw"])
+    assert np.abs(mixed["y"].numpy() - single["y"].astype(np.float32)).max() <= 1e-3 * span
+    allhalf = ref_order.conv2d_per_channel(x.half(), w.half(), b.half(), *args, q_scale.half(), [3])
+    assert allhalf["y"].dtype == torch.float16 and torch.isfinite(allhalf["y"]).all()
+    moved = (allhalf["qw"] != single["qw"]).mean()
+    assert 0.005 < moved < 0.10
+    assert np.abs(allhalf["qw"].astype(np.int32) - single["qw"]).max() == 1
+    assert _rel_rms(F.conv2d(x, w, b, 3, 3).numpy().astype(np.float64), allhalf["y"].float().numpy().astype(np.float64)) <= 0.02
+    # int16: 32767 / absmax exceeds the largest half for absmax < 0.5 -> inf in the half q_scale
+    assert torch.isinf((32767.0 / w.reshape(64, -1).abs().max(1)[0]).half()).all()
