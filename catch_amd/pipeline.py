@@ -260,9 +260,12 @@ class FusedNet(object):
                 self.f_demand[l.name] = True
 
     # ------------------------------------------------------------------------------------------
-    def forward(self, x, trace=None, timers=None):
+    def forward(self, x, trace=None, timers=None, keep=None):
         """x: [N,3,H,W] fp32 (NCHW) on the device.  trace: optional dict filled with, per conv/fc
         layer, its quantized input, int32 accumulators and fp32 output (as NHWC tensors).
+        keep: optional dict that receives every tensor the plan itself produces, keyed (name, "f") for an
+        fp32 (or fp16 output) NHWC tensor and (name, bitwidth, position, scale) for a quantized one -- the
+        untraced plan's own launches, unlike trace, which asks every layer for extra outputs.
         timers: optional dict; every conv/fc launch is bracketed by a pair of events recorded on
         the current stream and the pair is appended to timers[layer name] (durations of the
         launches in their real sequence, caches as the previous layer left them)."""
@@ -356,6 +359,8 @@ class FusedNet(object):
                     env[(name,) + form] = torch.cat([env[(s,) + form] for s in l.src], 3)
             else:
                 raise ValueError(l.kind)
+        if keep is not None:
+            keep.update(env)
         outs = []
         for o in self.outputs:
             y = env[(o, "f")]

@@ -3,6 +3,7 @@ fused integer plan: the lowered network must reproduce, bit for bit, the plan bu
 the architecture description and the same checkpoint."""
 import sys
 
+import numpy as np
 import pytest
 import torch
 
@@ -45,6 +46,11 @@ def test_lowering_with_fractional_scales():
     direct = pipeline.FusedNet(layers, pipeline.calibrate(net, x, "int8", True), fractional_scale=True)
     got = fused.forward(x.cuda())
     assert torch.equal(got, direct.forward(x.cuda()))
+    from oracle import netref
+    sd = pipeline.calibrate(net, x, "int8", True)
+    t, _ = netref.run(layers, {k: v.detach().cpu().numpy() for k, v in sd.items()}, x.numpy(), record=False,
+                      fractional_scale=True)
+    assert np.array_equal(t[direct.outputs[0]].reshape(got.shape), got.cpu().numpy())
     ref = net(x).cuda()
 
     def rel_rms(a, b):
@@ -73,6 +79,17 @@ def test_lowered_trace_equals_direct_plan(arch, size, std):
     assert len(got) == len(want)
     for g, w in zip(got, want):
         assert torch.equal(g, w)
+    # against the oracle: the unfused network of the same checkpoint, run layer by layer on the CPU -- the lowered
+    # plan's outputs are the oracle's bit for bit (fractional mode: test_lowering_with_fractional_scales)
+    from oracle import netref
+    sd = pipeline.calibrate(net, x, "int8", True)
+    t, rec = netref.run(layers, {k: v.detach().cpu().numpy() for k, v in sd.items()}, x.numpy())
+    assert all(r["overflow"] == 0 for r in rec.values())
+    for name, g in zip(direct.outputs, got):  # the lowered plan names its tensors after the graph's nodes
+        o = t[name]
+        gn = g.cpu().numpy()
+        gn = np.transpose(gn, (0, 2, 3, 1)) if gn.ndim == 4 else gn.reshape(o.shape)
+        assert np.array_equal(o.reshape(gn.shape), gn), name
     # and the traced module itself (float tensors between the ops) agrees within the stated tolerance
     ref = qnet(x.cuda())
     ref = ref if isinstance(ref, tuple) else (ref,)
