@@ -27,6 +27,8 @@ KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "igemm_
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
              "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-I" + INCLUDE, "-I" + CSRC]
+# extra compiler flags for experiments, e.g. CATCHQ_EXTRA_HIPFLAGS=-DCATCHQ_TUNING (tile / load-path switches)
+HIP_FLAGS += os.environ.get("CATCHQ_EXTRA_HIPFLAGS", "").split()
 
 
 def _run(cmd):

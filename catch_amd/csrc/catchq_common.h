@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <cstdlib>
+
 #include "catchq.h"
 
 #define CATCHQ_API extern "C" __attribute__((visibility("default")))
@@ -22,6 +25,33 @@ inline int launch_status() { return hipGetLastError() == hipSuccess ? CATCHQ_OK 
 // compute units one launch should plan its tile shapes for: the device's 256, divided by the number of
 // launches the caller says share the device (catchq_set_launch_sharing)
 int planned_cus();
+
+// Allow `kern` more than the default 64 KiB of dynamic LDS: needed once per kernel and device.  `raised` is the
+// call site's own flag array (one per kernel instance); setting the attribute twice is harmless, so relaxed
+// atomics are all the synchronisation that concurrent first calls need.
+inline int raise_lds_limit(const void *kern, int bytes, std::atomic<bool> (&raised)[64]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CATCHQ_ERR_LAUNCH;
+  if (!raised[dev].load(std::memory_order_relaxed)) {
+    if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return CATCHQ_ERR_LAUNCH;
+    }
+    raised[dev].store(true, std::memory_order_relaxed);
+  }
+  return CATCHQ_OK;
+}
+
+// Tuning switches read from the environment exist only in builds made with -DCATCHQ_TUNING (A/B timing of tile
+// shapes and load paths); the shipped library reads no environment variable.
+inline const char *tuning_env(const char *name) {
+#ifdef CATCHQ_TUNING
+  return std::getenv(name);
+#else
+  (void)name;
+  return nullptr;
+#endif
+}
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

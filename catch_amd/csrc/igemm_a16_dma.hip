@@ -245,14 +245,8 @@ static int launch_a16_epi(const void *a, const void *b, const IgemmParams &p, co
   static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
   auto kern = igemm_a16_dma_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, LOAD, EPI>;
   if (LDS_BYTES > 64 * 1024) {
-    static bool raised[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CATCHQ_ERR_LAUNCH;
-    if (!raised[dev]) {
-      if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-        return CATCHQ_ERR_LAUNCH;
-      raised[dev] = true;
-    }
+    static std::atomic<bool> raised[64];
+    if (raise_lds_limit((const void *)kern, LDS_BYTES, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
   }
   kern<<<p.nblocks, 64 * NW, LDS_BYTES, s>>>((const int16_t *)a, (const int8_t *)b, p, e, (unsigned)a_bytes,
                                              (unsigned)b_bytes);

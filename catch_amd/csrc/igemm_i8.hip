@@ -289,7 +289,7 @@ static int pick_tile(const void *a, const void *b, const IgemmParams &p, const E
 // CATCHQ_NO_DMA=1 keeps every shape on the register-staged kernel (for A/B timing)
 static bool dma_enabled() {
   static const bool on = [] {
-    const char *v = getenv("CATCHQ_NO_DMA");
+    const char *v = tuning_env("CATCHQ_NO_DMA");
     return !(v && v[0] == '1');
   }();
   return on;

@@ -109,7 +109,7 @@ int conv2d_dual_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
   // (two accumulator sets leave a 128x128 tile a single block per CU); with short K the launch is all
   // epilogue and the wider tile's longer output rows help.
   int tile = (p.N >= 128 && p.K + ps.K <= 128) ? 64128 : 64064;
-  if (const char *t = getenv("CATCHQ_DUAL_TILE")) {  // tuning aid: BMxBN
+  if (const char *t = tuning_env("CATCHQ_DUAL_TILE")) {  // tuning aid: BMxBN
     int bm = 0, bn = 0;
     if (sscanf(t, "%dx%d", &bm, &bn) == 2) tile = bm * 1000 + bn;
   }

@@ -116,14 +116,8 @@ static int pw_launch(const void *a, const void *b, const IgemmParams &p, const E
   if (blocks > resident) blocks = resident;
   auto kern = pw_i8_kernel<KS, NF, EPI>;
   if (LDS_BYTES > 64 * 1024) {
-    static bool raised[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return CATCHQ_ERR_LAUNCH;
-    if (!raised[dev]) {
-      if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-        return CATCHQ_ERR_LAUNCH;
-      raised[dev] = true;
-    }
+    static std::atomic<bool> raised[64];
+    if (raise_lds_limit((const void *)kern, LDS_BYTES, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
   }
   kern<<<blocks, 256, LDS_BYTES, s>>>((const int8_t *)a, (const int8_t *)b, p, e, (int)ngroups);
   return launch_status();

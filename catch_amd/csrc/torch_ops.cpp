@@ -537,7 +537,9 @@ Tensor quantize_nhwc_frame_op(const Tensor &x, int64_t bitwidth, int64_t positio
 struct Prepared {
   c10::weak_intrusive_ptr<c10::TensorImpl> w_impl, s_impl, m_impl;
   uint32_t w_ver = 0, s_ver = 0, m_ver = 0;
-  const void *w_ptr = nullptr;
+  const void *w_ptr = nullptr, *s_ptr = nullptr, *m_ptr = nullptr;
+  Tensor s_host, m_host;  // the q-params as read when the entry was made (compared by content when they live on the host)
+  c10::StreamId made_on = 0;  // stream that allocated and filled qw / new_scale
   int bw_x = 8, bw_w = 8, pos_x = 0, pos_w = 0;
   bool per_channel = false;
   int variant = 0;   // caller's layout choice for qw (part of the cache key)
@@ -571,8 +573,18 @@ bool still_valid(const Prepared &p, const Tensor &w, const Tensor &s, const Tens
   auto same = [](const c10::weak_intrusive_ptr<c10::TensorImpl> &weak, const Tensor &t, uint32_t ver) {
     return !weak.expired() && weak._unsafe_get_target() == t.unsafeGetTensorImpl() && version_of(t) == ver;
   };
-  return same(p.w_impl, w, p.w_ver) && same(p.s_impl, s, p.s_ver) && same(p.m_impl, m, p.m_ver) &&
-         p.w_ptr == w.data_ptr();
+  if (!(same(p.w_impl, w, p.w_ver) && same(p.s_impl, s, p.s_ver) && same(p.m_impl, m, p.m_ver) &&
+        p.w_ptr == w.data_ptr() && p.s_ptr == s.data_ptr() && p.m_ptr == m.data_ptr()))
+    return false;
+  // Tensors without a version counter (inference tensors) and `.data =` swaps that keep the storage cannot be
+  // told apart by identity.  q-params that live on the host are compared by content (a few bytes); for device
+  // tensors the storage address above is what is checked -- reading them back would be the host synchronisation
+  // this cache exists to avoid (after writing into such a tensor in place, call torch_mlu::clear_weight_cache).
+  auto same_content = [](const Tensor &now, const Tensor &then) {
+    if (!now.device().is_cpu()) return true;
+    return now.numel() == then.numel() && now.scalar_type() == then.scalar_type() && at::equal(now.contiguous(), then);
+  };
+  return same_content(s, p.s_host) && same_content(m, p.m_host);
 }
 
 c10::weak_intrusive_ptr<c10::TensorImpl> weak_of(const Tensor &t) {
@@ -635,6 +647,10 @@ std::shared_ptr<Prepared> prepare(MakeDense make_dense, const Tensor &weight, co
   p->w_impl = weak_of(weight); p->s_impl = weak_of(q_scale); p->m_impl = weak_of(q_mode);
   p->w_ver = version_of(weight); p->s_ver = version_of(q_scale); p->m_ver = version_of(q_mode);
   p->w_ptr = weight.data_ptr();
+  p->s_ptr = q_scale.data_ptr();
+  p->m_ptr = q_mode.data_ptr();
+  p->s_host = q_scale.to(at::kCPU).contiguous().clone();
+  p->m_host = q_mode.to(at::kCPU).contiguous().clone();
   return p;
 }
 
@@ -648,8 +664,15 @@ std::shared_ptr<Prepared> prepared_for(const Tensor &weight, const Tensor &q_sca
     auto it = g_cache.find(key);
     if (it != g_cache.end()) {
       if (it->second->variant == variant && still_valid(*it->second, weight, q_scale, q_mode)) {
+        const auto cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
         if (!it->second->ready.query())  // still in flight on the stream that prepared it
-          it->second->ready.block(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+          it->second->ready.block(cur);
+        if (cur.id() != it->second->made_on) {
+          // read on another stream than the one the caching allocator knows these blocks by: tell it, so that
+          // an entry dropped while this stream's kernels still read it is not handed out again too early
+          it->second->qw.record_stream(cur);
+          if (it->second->new_scale.defined()) it->second->new_scale.record_stream(cur);
+        }
         return it->second;
       }
       g_cache.erase(it);
@@ -657,16 +680,23 @@ std::shared_ptr<Prepared> prepared_for(const Tensor &weight, const Tensor &q_sca
   }
   auto p = prepare(make_dense, weight, q_scale, q_mode);
   p->variant = variant;
-  p->ready.record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+  const auto made_on = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  p->made_on = made_on.id();
+  p->ready.record(made_on);
   if (use_cache) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
-    if (g_cache.size() > 4096) {  // drop entries whose weight is gone
-      for (auto it = g_cache.begin(); it != g_cache.end();)
-        it = it->second->w_impl.expired() ? g_cache.erase(it) : std::next(it);
-    }
+    // every miss sweeps out the entries whose weight tensor is gone (their quantized copies are device memory;
+    // misses are first uses of a weight, so the sweep is off the steady-state path)
+    for (auto it = g_cache.begin(); it != g_cache.end();)
+      it = it->second->w_impl.expired() ? g_cache.erase(it) : std::next(it);
     g_cache[key] = p;
   }
   return p;
+}
+
+int64_t cache_size_op() {
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  return (int64_t)g_cache.size();
 }
 
 void clear_cache_op() {
@@ -960,6 +990,7 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("maxpool_nhwc(Tensor x, int k, int stride, int pad) -> Tensor");
   m.def("global_avgpool_nhwc(Tensor x, int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> Tensor");
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
+  m.def("weight_cache_size() -> int", &cache_size_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
         "int[] dilation, int groups) -> str", &conv2d_route_op);
 }

@@ -200,6 +200,45 @@ def test_weight_cache_follows_inplace_updates():
     assert same_bits(ref["y"], y3.cpu().numpy())
 
 
+def test_weight_cache_sees_swapped_storage_and_host_qparams_by_content():
+    """what identity and version cannot tell: a `.data =` swap of q_scale (same tensor object, same version,
+    new storage), q-params that live on the host and change in place under inference mode (no version
+    counter), and entries of weights that no longer exist"""
+    note("weight cache: data swap, host q-params, purge")
+    torch.manual_seed(9)
+    ops = torch.ops.torch_mlu
+    x = torch.randn(1, 16, 8, 8).cuda()
+    w = (torch.randn(16, 16, 3, 3) * 0.1).cuda()
+    b = torch.zeros(16).cuda()
+    args = ([1, 1], [1, 1], [1, 1], 1)
+    q_mode = torch.tensor([1], dtype=torch.int32).cuda()
+
+    def want(q_scale):
+        return oops.conv2d(x.cpu().numpy(), w.cpu().numpy(), None, (1, 1), (1, 1), (1, 1), 1, q_scale.cpu().numpy(), [1])["y"]
+    q_scale = torch.tensor([127 / 4.0, 127 / 0.5]).cuda()
+    assert same_bits(want(q_scale), ops.conv2d(x, w, b, *args, q_scale, q_mode).cpu().numpy())
+    ver = q_scale._version
+    q_scale.data = torch.tensor([127 / 16.0, 127 / 0.5]).cuda()
+    assert q_scale._version == ver
+    assert same_bits(want(q_scale), ops.conv2d(x, w, b, *args, q_scale, q_mode).cpu().numpy())
+    with torch.inference_mode():
+        hs = torch.tensor([127 / 4.0, 127 / 0.5])       # host q-params, inference tensors: version 0 for ever
+        hm = torch.tensor([1], dtype=torch.int32)
+        wi, xi, bi = w.clone(), x.clone(), b.clone()
+        y1 = ops.conv2d(xi, wi, bi, *args, hs, hm)
+        hs[0] = 127 / 32.0
+        y2 = ops.conv2d(xi, wi, bi, *args, hs, hm)
+    assert same_bits(want(torch.tensor([127 / 4.0, 127 / 0.5])), y1.cpu().numpy())
+    assert same_bits(want(torch.tensor([127 / 32.0, 127 / 0.5])), y2.cpu().numpy())
+    # entries of dead weights go at the next miss, not when 4096 of them have piled up
+    ops.clear_weight_cache()
+    for i in range(5):
+        wt = (torch.randn(16, 16, 3, 3) * 0.1).cuda()
+        ops.conv2d(x, wt, b, *args, q_scale, q_mode)
+        del wt
+    assert ops.weight_cache_size() <= 2
+
+
 def test_cpu_tensors_are_refused():
     note("cpu refused")
     x, w, b = torch.randn(1, 4, 4, 4), torch.randn(4, 4, 1, 1), torch.zeros(4)
