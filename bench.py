@@ -24,11 +24,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0
-# HBM bytes moved by the igemm launches of one ResNet-50 bs64 step, from two rocprofv3 --pmc runs
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy in the same runs), keyed by
-# (workload, batch, parts the batch is split into): 2.133e9 read + 1.673e9 written with two parts,
-# 1.940e9 + 1.666e9 with the batch undivided.  Valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = {("resnet50", 64, 2): 3.806e9, ("resnet50", 64, 1): 3.606e9}
+# Where the HBM traffic of the convolution launches was measured (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --graph-only`); the bench line itself reports no traffic figure: it cannot read a counter.
+TRAFFIC_PROFILE = {"resnet50": "profiles/igemm_i8_resnet50_bs64_hbm_traffic.md"}
 
 
 def parse():
@@ -48,6 +46,13 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    ap.add_argument("--graph-only", action="store_true",
+                    help="time the graph replays and launch nothing else (no per-launch passes, no extras, no CPU "
+                         "baseline): the mode to run under rocprofv3, whose kernel table then holds the timed region only")
+    ap.add_argument("--probe", default="",
+                    help="launch one kernel --probe-iters times and exit (for rocprofv3 counter runs): "
+                         "gemm:MxNxK (config-2 epilogue), quantize, layer:NAME (that layer's launch of the workload), copy")
+    ap.add_argument("--probe-iters", type=int, default=20)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy (reference dispatch for scaling rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -68,7 +73,7 @@ def event_time(fn, iters, warm=3):
     return s.elapsed_time(e) * 1e-3 / iters
 
 
-def layer_profile(fused, x, iters=20):
+def layer_profile(fused, x, iters=20, only=None):
     """Time every kernel launch of one forward pass separately (HIP events, `iters` back-to-back
     launches each) and attach the algorithmic bytes / ops of each conv / fc launch."""
     import torch
@@ -78,7 +83,7 @@ def layer_profile(fused, x, iters=20):
     fused.forward(x, trace=trace)  # materialise every layer's quantized input once
     torch.cuda.synchronize()
     for l in fused.layers:
-        if l.kind not in ("conv", "fc") or l.name in fused._fused_away:
+        if l.kind not in ("conv", "fc") or l.name in fused._fused_away or (only and l.name != only):
             continue
         lq = fused.q[l.name]
         qx = trace[l.name].get("qx_dev", trace[l.name]["qx"])  # the tensor the kernel reads
@@ -127,23 +132,154 @@ def layer_profile(fused, x, iters=20):
     return rows
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus %d is not supported (every box has one GPU, "
-              "the path shards by batch with no communication)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-    import torch
-    torch.set_grad_enabled(False)
-    import catch_amd  # noqa: F401  (fails loudly if the HIP extension is missing)
-    from catch_amd import nets, pipeline
+def plan_launches(fused, n, h, w):
+    """Every launch of one untraced forward pass over n images of h x w, in launch order, with its algorithmic
+    bytes (the tensors the fused plan moves: integer inputs and weights, fp32 residual read, fp32 / fp16 and
+    integer outputs written) and integer operations, from the layer shapes alone (nothing is launched)."""
+    rows, shape = [], {}
+    cin = fused.cdev["input"]
+    for d in fused.q_demand["input"]:
+        if fused.stem:
+            sp = fused.stem["pad"]
+            oh, ow = h + 2 * sp, w + 2 * sp + fused.stem["extra"]
+        else:
+            oh, ow = h, w
+        shape[("input", "q")] = (oh, ow)
+        rows.append(dict(name="input", kind="quantize", ops=0, bytes=n * fused.chan["input"] * h * w * 4 + n * oh * ow * cin * d[0] // 8))
+    shape["input"] = (h, w)
+    for l in fused.layers:
+        if l.kind == "conv":
+            hi, wi = shape[l.src]
+            ho, wo = (hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1
+            shape[l.name] = (ho, wo)
+            if l.name in fused._fused_away:
+                continue
+            lq = fused.q[l.name]
+            n_out = n * ho * wo * fused.cdev[l.name]
+            ih, iw = shape[("input", "q")] if (fused.stem and l.name == fused.stem["name"]) else (hi, wi)
+            macs = n_out * (lq.qw.numel() // lq.qw.shape[0])
+            b = n * ih * iw * fused.cdev[l.src] * lq.bw_x // 8 + lq.qw.numel() * lq.qw.element_size()
+            ds = fused.shortcut_of.get(l.name)
+            if ds is not None:
+                dq = fused.q[ds.name]
+                macs += n_out * dq.qw.shape[-1]
+                b += n * ho * wo * fused.cdev[ds.src] * dq.bw_x // 8 + dq.qw.numel() * dq.qw.element_size()
+            elif l.add:
+                b += 4 * n_out
+            qd = fused.q_demand[l.name][0] if fused.q_demand[l.name] else None
+            want_y = fused.f_demand[l.name] or qd is None
+            y_half = fused.out_half and l.name in fused.outputs
+            b += ((2 if y_half else 4) * n_out if want_y else 0) + (n_out * qd[0] // 8 if qd else 0)
+            rows.append(dict(name=l.name, kind="conv", ops=2 * macs, bytes=b, m=n * ho * wo, n=fused.cdev[l.name],
+                             k=lq.qw.numel() // lq.qw.shape[0] + (fused.q[ds.name].qw.shape[-1] if ds is not None else 0)))
+            for d in fused.q_demand[l.name][1:]:
+                rows.append(dict(name=l.name, kind="quantize", ops=0, bytes=n_out * 4 + n_out * d[0] // 8))
+        elif l.kind == "fc":
+            lq = fused.q[l.name]
+            shape[l.name] = (1, 1)
+            k = lq.qw.shape[1]
+            rows.append(dict(name=l.name, kind="fc", ops=2 * n * k * lq.qw.shape[0], m=n, n=lq.qw.shape[0], k=k,
+                             bytes=n * k * lq.bw_x // 8 + lq.qw.numel() * lq.qw.element_size() + 4 * n * lq.qw.shape[0]))
+        elif l.kind == "maxpool":
+            hi, wi = shape[l.src]
+            ho, wo = (hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1
+            shape[l.name] = (ho, wo)
+            for form in fused._forms(l.name):
+                e = 4 if form == ("f",) else form[0] // 8
+                rows.append(dict(name=l.name, kind="maxpool", ops=0, bytes=n * fused.cdev[l.src] * e * (hi * wi + ho * wo)))
+        elif l.kind == "gap":
+            hi, wi = shape[l.src]
+            shape[l.name] = (1, 1)
+            c = fused.cdev[l.src]
+            if fused.f_demand[l.name] or not fused.q_demand[l.name]:
+                rows.append(dict(name=l.name, kind="avgpool", ops=0, bytes=n * c * 4 * (hi * wi + 1)))
+                for d in fused.q_demand[l.name]:
+                    rows.append(dict(name=l.name, kind="quantize", ops=0, bytes=n * c * (4 + d[0] // 8)))
+            else:
+                for d in fused.q_demand[l.name]:
+                    rows.append(dict(name=l.name, kind="avgpool+quantize", ops=0, bytes=n * c * (4 * hi * wi + d[0] // 8)))
+        elif l.kind == "upsample":
+            hi, wi = shape[l.src]
+            shape[l.name] = (hi * 2, wi * 2)
+            for form in fused._forms(l.name):  # torch's repeat_interleave, twice
+                e = 4 if form == ("f",) else form[0] // 8
+                rows.append(dict(name=l.name, kind="upsample", ops=0, bytes=n * fused.cdev[l.src] * e * hi * wi * 9))
+        elif l.kind == "concat":
+            shape[l.name] = shape[l.src[0]]
+            hi, wi = shape[l.name]
+            for form in fused._forms(l.name):
+                e = 4 if form == ("f",) else form[0] // 8
+                rows.append(dict(name=l.name, kind="concat", ops=0, bytes=2 * n * fused.cdev[l.name] * e * hi * wi))
+    return rows
 
-    if args.copy_probe:
-        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read + 1 GiB written
+
+def bound_of(ops, nbytes):
+    """which roof the launch's algorithmic work sits under: the time its bytes need at the HBM peak against the
+    time its operations need at the int8 matrix peak"""
+    return "hbm" if nbytes / (HBM_PEAK_GBS * 1e9) >= ops / (INT8_PEAK_TOPS * 1e12) else "mfma"
+
+
+def run_probe(args):
+    """one kernel, launched --probe-iters times on the current stream: what a rocprofv3 --pmc run should see"""
+    import torch
+    import catch_amd  # noqa: F401
+    ops = torch.ops.torch_mlu
+    what = args.probe
+    it = args.probe_iters
+    if what == "copy":  # the reference dispatch for scaling FETCH_SIZE / WRITE_SIZE: 1 GiB read, 1 GiB written
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        for _ in range(it):
+            dst.copy_(src)
+        desc = "1 GiB fp32 copy"
+    elif what.startswith("gemm:"):
+        m, n, k = (int(v) for v in what[5:].split("x"))
+        a, b, exp2, div, bias = gaussian_linear_operands(m, n, k)
+        for _ in range(it):
+            ops.qlinear(a, b, exp2, div, bias, 1, True, True, False, 0, 0, 1.0)
+        desc = "int8 GEMM %dx%dx%d, per-channel dequant + bias + ReLU, fp16 out" % (m, n, k)
+    elif what == "quantize":
+        n = 64 * 256 * 56 * 56
+        xs = [torch.randn(n, device="cuda") for _ in range(6)]
+        for i in range(it):
+            ops.quantize(xs[i % 6], 8, -5, 1.0)
+        desc = "quantize fp32 -> int8, %d elements, 6 rotating inputs" % n
+    elif what.startswith("layer:"):
+        from catch_amd import _native
+        fused, xg, _ = build_workload(args)
+        parts = list(xg.chunk(args.streams))
+        _native.kernel_lib().catchq_set_launch_sharing(args.streams)
+        rows = layer_profile(fused, parts[0], iters=it, only=what[6:])
+        _native.kernel_lib().catchq_set_launch_sharing(1)
+        desc = "%s of %s, %d images: %.2f us, %.1f GB/s, %.1f TOPS" % (
+            what[6:], args.workload, parts[0].shape[0], rows[0]["t"] * 1e6, rows[0]["bytes"] / rows[0]["t"] / 1e9,
+            rows[0]["ops"] / rows[0]["t"] / 1e12)
+    else:
+        sys.exit("unknown --probe " + what)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": what, "iters": it, "what": desc}))
+
+
+def gaussian_linear_operands(m, n, k):
+    """X[m,k], W[n,k] ~ N(0,1) (seeds 2, 3), bias N(0,1) (seed 4); X per-tensor int8, W per-channel int8:
+    the standalone linear configuration.  -> qx, qw, exp2, new_scale, bias"""
+    import torch
+    from catch_amd.pipeline import pos_from_scale
+    ops = torch.ops.torch_mlu
+    x = torch.randn(m, k, generator=torch.Generator().manual_seed(2)).cuda()
+    w = torch.randn(n, k, generator=torch.Generator().manual_seed(3)).cuda()
+    bias = torch.randn(n, generator=torch.Generator().manual_seed(4)).cuda()
+    pos_x = pos_from_scale(8, 127.0 / x.abs().max().item())
+    qx = ops.quantize(x, 8, pos_x, 1.0)
+    scales = (127.0 / w.abs().amax(1)).float()
+    qw, new_pos, new_scale = ops.quantize_per_channel(w, scales, 8)
+    return qx, qw, pos_x + int(new_pos.item()), new_scale, bias
+
+
+def build_workload(args):
+    """-> (fused plan, input batch on the device, dict(net, x, sd, layers, batch, side, what, detector, t_cal))"""
+    import torch
+    from catch_amd import nets, pipeline
     batch = args.batch or {"resnet50": 64, "resnet18": 64, "mobilenet_v2": 128, "darknet53_yolov3": 16}[args.workload]
     layers = nets.NETS[args.workload]()
     detector = args.workload == "darknet53_yolov3"
@@ -167,11 +303,37 @@ def main():
             sys.exit("--fractional-scale needs a checkpoint of scales; the detector's holds bit widths and positions")
         what += ", position + fractional scale"
     fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale)
-    xg = x.cuda()
     if args.streams < 1:
         sys.exit("--streams must be at least 1")
     while batch % args.streams:  # the largest number of equal parts not above what was asked for
         args.streams -= 1
+    return fused, x.cuda(), dict(net=net, x=x, sd=sd, layers=layers, batch=batch, side=side, what=what,
+                                 detector=detector, t_cal=t_cal)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (every box has one GPU, "
+              "the path shards by batch with no communication)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    torch.set_grad_enabled(False)
+    import catch_amd  # noqa: F401  (fails loudly if the HIP extension is missing)
+    from catch_amd import nets, pipeline
+
+    if args.probe:
+        run_probe(args)
+        return
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    fused, xg, w_ = build_workload(args)
+    net, x, sd, layers, batch, side, what, detector, t_cal = (w_[k] for k in ("net", "x", "sd", "layers", "batch", "side",
+                                                                               "what", "detector", "t_cal"))
     static_in, replay = fused.capture(xg, streams=args.streams)
     static_in.copy_(xg)
     for _ in range(args.warmup):
@@ -188,6 +350,30 @@ def main():
     outs = out if isinstance(out, tuple) else (out,)
     for o in outs:
         assert torch.isfinite(o.float()).all()
+
+    launches = plan_launches(fused, batch // args.streams, side, side)
+    config = {"workload": "%s %s, fused requant pipeline replayed from a HIP graph%s" % (
+        args.workload, what, "" if args.streams <= 1 else " (the batch in %d parts on parallel streams)" % args.streams),
+              "global_batch": batch, "calibration_images": args.calib_images, "graph_streams": args.streams,
+              "gop_per_step": round(2 * nets.conv_macs(layers, batch, side, side) / 1e9, 1)}
+    metric = ("int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
+              else "int8 %s images/sec" % args.workload)
+    if args.graph_only:
+        # nothing but the graph replays has been launched since the capture: a kernel trace of this run holds the
+        # timed region (plus the capture's own warm-up passes); the launch list names what one part's pass runs
+        conv_b = args.streams * sum(r["bytes"] for r in launches if r["kind"] == "conv")
+        all_b = args.streams * sum(r["bytes"] for r in launches)
+        print(json.dumps({"metric": metric, "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+                          "scaling": "weak", "vs_baseline": None, "dtype": "int16xint8" if detector else "int8",
+                          "data": "synthetic", "config": config,
+                          "roofline": {"bound": "hbm", "kernel": "whole timed step (graph replays only)",
+                                       "achieved": round(all_b / (ms_per_step * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                                       "unit": "GB/s", "frac": round(all_b / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                       "traffic": None, "algorithmic_bytes_per_step": all_b,
+                                       "algorithmic_bytes_of_the_convolutions": conv_b},
+                          "launches_per_part": [[r["name"], r["kind"], r["bytes"], r["ops"]] for r in launches]}))
+        return
 
     # ---- per-kernel roofline of the dominant family: the implicit-GEMM convolutions ------------
     # The launches measured are the ones the graph holds: with the batch in `streams` parts, every layer is
@@ -231,8 +417,11 @@ def main():
     for name, evs in timers.items():
         pairs = [(evs[i], evs[i + 1]) for i in range(0, len(evs), 2)]
         seq[name] = max(sum(a.elapsed_time(b) for a, b in pairs) / len(pairs) * 1e-3 - empty_s, 1e-7)
+    analytic = {r["name"]: r for r in launches if r["kind"] in ("conv", "fc")}
     for r in rows:
         r["t_seq"] = seq[r["name"]]
+        a = analytic[r["name"]]
+        assert (a["bytes"], a["ops"]) == (r["bytes"], r["ops"]), "launch accounting differs for %s: %r vs %r" % (r["name"], a, r)
     conv_rows = [r for r in rows if r["route"].startswith("mfma")]
     n_parts = len(parts)  # per step: every row's launch once per part
     t_conv = n_parts * sum(r["t_seq"] for r in conv_rows)
@@ -252,7 +441,7 @@ def main():
                     n_parts * len(conv_rows), len(conv_rows), n_parts),
                 "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, batch, n_parts)),
+                "traffic": None, "traffic_profile": TRAFFIC_PROFILE.get(args.workload),
                 "avg_launch_us": round(t_conv / max(n_parts * len(conv_rows), 1) * 1e6, 2),
                 "timing": "HIP events around each launch of eager forward passes over the parts, in sequence (%d passes), "
                           "minus the bracket's own share, 2*T(pair around one small kernel) - T(pair around two), "
@@ -269,16 +458,18 @@ def main():
                                       "frac": round(b_conv / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                                       "int8_tops": round(o_conv / (ms_per_step * 1e-3) / 1e12, 1)}}
 
-    result = {"metric": "int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
-              else "int8 %s images/sec" % args.workload,
+    result = {"metric": metric,
               "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
               "dtype": "int16xint8" if detector else "int8", "data": "synthetic",
-              "config": {"workload": "%s %s, fused requant pipeline replayed from a HIP graph%s" % (
-                  args.workload, what, "" if args.streams <= 1 else " (the batch in %d parts on parallel streams)" % args.streams),
-                         "global_batch": batch, "calibration_images": args.calib_images, "graph_streams": args.streams,
-                         "gop_per_step": round(2 * nets.conv_macs(layers, batch, side, side) / 1e9, 1)},
-              "roofline": roofline}
+              "config": config, "roofline": roofline,
+              # every conv / fc launch of one part, timed in sequence: [layer, M, N, K, us, GB/s, TOPS, which roof its
+              # algorithmic work sits under, fraction of that roof]
+              "layers": [[r["name"], analytic[r["name"]]["m"], analytic[r["name"]]["n"], analytic[r["name"]]["k"],
+                          round(r["t_seq"] * 1e6, 1), round(r["bytes"] / r["t_seq"] / 1e9), round(r["ops"] / r["t_seq"] / 1e12),
+                          bound_of(r["ops"], r["bytes"]),
+                          round(max(r["bytes"] / (HBM_PEAK_GBS * 1e9), r["ops"] / (INT8_PEAK_TOPS * 1e12)) / r["t_seq"], 3)]
+                         for r in rows]}
 
     if not args.no_extras:
         result["extras"] = extras()
@@ -295,57 +486,84 @@ def main():
         result["cpu_baseline"]["float_torch_cpu"] = {"value": round(n_cpu / (time.time() - t0), 2), "unit": "images/s",
                                                      "threads": _t.get_num_threads(),
                                                      "what": "the same network in fp32 through PyTorch's CPU kernels"}
+        # one thread of the same oracle on one image, for a per-core figure
+        import oracle as orc
+        n_thr = orc.num_threads()
+        orc.set_num_threads(1)
+        one = cpu_baseline(layers, sd, x[:1], outs[0][:1].float().cpu(), fused.outputs[0], args.fractional_scale)
+        orc.set_num_threads(n_thr)
+        result["cpu_baseline"]["one_thread"] = {"value": one["value"], "unit": "images/s", "cores": 1,
+                                                "sample": "1 image of the same batch through the whole network"}
     result["calibration_s"] = round(t_cal, 2)
     print(json.dumps(result))
 
 
 def extras():
     """standalone kernels: int8 linear (config shapes) and quantize streaming rate"""
-    import ctypes
     import torch
     ops = torch.ops.torch_mlu
     out = {}
-    from catch_amd.pipeline import pos_from_scale
-
-    def gaussian_operands(m, n, k):
-        """X[m,k], W[n,k] ~ N(0,1) (seeds 2, 3), X per-tensor int8, W per-channel int8: the standalone linear config"""
-        x = torch.randn(m, k, generator=torch.Generator().manual_seed(2)).cuda()
-        w = torch.randn(n, k, generator=torch.Generator().manual_seed(3)).cuda()
-        pos_x = pos_from_scale(8, 127.0 / x.abs().max().item())
-        qx = ops.quantize(x, 8, pos_x, 1.0)
-        scales = (127.0 / w.abs().amax(1)).float()
-        qw, new_pos, new_scale = ops.quantize_per_channel(w, scales, 8)
-        return qx, qw, pos_x + int(new_pos.item()), new_scale
 
     def time_gemm(a, b, exp2, div, bias, iters):
         return event_time(lambda: ops.qlinear(a, b, exp2, div, bias, 1, True, True, False, 0, 0, 1.0), iters, max(iters // 10, 3))
 
+    def vendor_int_mm(a, b, iters):
+        """the same integer product through torch._int_mm (the vendor GEMM library): int32 output, no epilogue --
+        context from the same box, not a like-for-like launch"""
+        try:
+            bt = b.t()
+            return event_time(lambda: torch._int_mm(a, bt), iters, max(iters // 10, 3))
+        except Exception as exc:  # the library may refuse a shape
+            return str(exc)[:80]
+
     for (m, n, k) in ((4096, 3072, 768), (4096, 768, 3072)):
-        bias = torch.randn(n, generator=torch.Generator().manual_seed(4)).cuda()
-        a, b, exp2, div = gaussian_operands(m, n, k)
+        a, b, exp2, div, bias = gaussian_linear_operands(m, n, k)
         t = time_gemm(a, b, exp2, div, bias, 200)
+        tv = vendor_int_mm(a, b, 200)
         out["linear_%dx%dx%d" % (m, n, k)] = {"us": round(t * 1e6, 2), "tops": round(2 * m * n * k / t / 1e12, 1),
                                              "mfma_frac": round(2 * m * n * k / t / 1e12 / INT8_PEAK_TOPS, 4),
                                              "operands": "N(0,1) quantized: X per tensor, W per channel",
-                                             "epilogue": "per-channel dequant + bias + ReLU, fp16 out"}
+                                             "epilogue": "per-channel dequant + bias + ReLU, fp16 out",
+                                             "torch_int_mm_us": round(tv * 1e6, 2) if isinstance(tv, float) else tv}
     # a GEMM large enough to be bound by the matrix cores, on two kinds of data: the rate depends on how many
     # operand bits toggle (the chip lowers its clock under high-toggle matrix work)
     m = n = k = 8192
-    bias = torch.randn(n, device="cuda")
-    a, b, exp2, div = gaussian_operands(m, n, k)
+    a, b, exp2, div, bias = gaussian_linear_operands(m, n, k)
     t_g = time_gemm(a, b, exp2, div, bias, 10)
+    tv_g = vendor_int_mm(a, b, 10)
     a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
     b = torch.randint(-128, 128, (n, k), dtype=torch.int8, device="cuda")
     t_u = time_gemm(a, b, -10, div, bias, 10)
+    tv_u = vendor_int_mm(a, b, 10)
+    a.zero_()
+    b.zero_()
+    t_z = time_gemm(a, b, -10, div, bias, 10)
     out["gemm_8192x8192x8192"] = {"us_gaussian_operands": round(t_g * 1e6, 1), "tops_gaussian_operands": round(2 * m * n * k / t_g / 1e12, 1),
                                   "us_uniform_operands": round(t_u * 1e6, 1), "tops_uniform_operands": round(2 * m * n * k / t_u / 1e12, 1),
-                                  "mfma_frac": round(2 * m * n * k / t_g / 1e12 / INT8_PEAK_TOPS, 4)}
+                                  "us_zero_operands": round(t_z * 1e6, 1), "tops_zero_operands": round(2 * m * n * k / t_z / 1e12, 1),
+                                  "mfma_frac": round(2 * m * n * k / t_g / 1e12 / INT8_PEAK_TOPS, 4),
+                                  "torch_int_mm_us_gaussian": round(tv_g * 1e6, 1) if isinstance(tv_g, float) else tv_g,
+                                  "torch_int_mm_us_uniform": round(tv_u * 1e6, 1) if isinstance(tv_u, float) else tv_u}
     del a, b
-    n = 64 * 256 * 56 * 56  # one ResNet-50 stage-1 activation, 822 MB of fp32: larger than the 256 MB cache
-    x = torch.randn(n, device="cuda")
-    t = event_time(lambda: ops.quantize(x, 8, -5, 1.0), 20, 3)
-    out["quantize_f32_to_i8"] = {"elements": n, "us": round(t * 1e6, 1), "gbs": round(5 * n / t / 1e9, 1),
-                                 "hbm_frac": round(5 * n / t / 1e9 / HBM_PEAK_GBS, 4)}
+    # quantize fp32 -> int8: 4 B read + 1 B written per element.  One ResNet-50 stage-1 activation (51.4 M elements)
+    # is 206 MB in + 51 MB out, about the size of the 256 MB last-level cache: repeated over one buffer pair that is
+    # a warm figure.  The cold one rotates over 6 pairs (1.54 GB), so no launch finds its operands cached.
+    n = 64 * 256 * 56 * 56
+    xs = [torch.randn(n, device="cuda") for _ in range(6)]
+    t_w = event_time(lambda: ops.quantize(xs[0], 8, -5, 1.0), 24, 3)
+    state = {"i": 0}
+
+    def cold():
+        state["i"] = (state["i"] + 1) % 6
+        return ops.quantize(xs[state["i"]], 8, -5, 1.0)
+    t_c = event_time(cold, 24, 6)
+    out["quantize_f32_to_i8"] = {"elements": n, "us": round(t_c * 1e6, 1), "gbs": round(5 * n / t_c / 1e9, 1),
+                                 "hbm_frac": round(5 * n / t_c / 1e9 / HBM_PEAK_GBS, 4),
+                                 "working_set": "6 input buffers in rotation, 1.23 GB of fp32 (cold: nothing cached)",
+                                 "warm": {"us": round(t_w * 1e6, 1), "gbs": round(5 * n / t_w / 1e9, 1),
+                                          "hbm_frac": round(5 * n / t_w / 1e9 / HBM_PEAK_GBS, 4),
+                                          "working_set": "one 206 MB input over and over (about the last-level cache's size)"}}
+    del xs
     return out
 
 
