@@ -79,12 +79,14 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
       const bool ok = m < p.M;
       const int64_t mm = ok ? m : 0;
       if constexpr (LOAD == LOAD_CONV) {
-        const int wo = (int)(mm % p.Wo);
-        const int64_t t = mm / p.Wo;
-        const int ho = (int)(t % p.Ho);
-        const int64_t img = t / p.Ho;
+        // fewer than 2^31 output pixels (checked by the launcher): 32-bit divisions
+        const unsigned mu = (unsigned)mm;
+        const unsigned t = mu / (unsigned)p.Wo;
+        const int wo = (int)(mu - t * (unsigned)p.Wo);
+        const unsigned img = t / (unsigned)p.Ho;
+        const int ho = (int)(t - img * (unsigned)p.Ho);
         const int hi0 = ho * p.sh - p.ph, wi0 = wo * p.sw - p.pw;
-        rowbase[j] = 2u * ((unsigned)(img * p.H * p.W * p.Ci) + (unsigned)((hi0 * p.W + wi0) * p.Ci));  // mod 2^32
+        rowbase[j] = 2u * ((unsigned)((int64_t)img * p.H * p.W * p.Ci) + (unsigned)((hi0 * p.W + wi0) * p.Ci));  // mod 2^32
         unsigned mask = 0;
         for (int r = 0; r < p.kh; ++r)
           for (int q = 0; q < p.kw; ++q)
@@ -439,6 +441,7 @@ int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, i
   p.H = H; p.W = W; p.Ci = Ci; p.Ho = Ho; p.Wo = Wo;
   p.kh = kh; p.kw = kw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
   p.K = kh * kw * Ci;
+  if (p.M >= (1ll << 31)) return -1;  // the loaders split a pixel index with 32-bit divisions
   if (Ci == 8 && ph == 0 && pw == 0 && dw == 1) {  // framed few-channel image: streaming kernel
     const int st = conv2d_stem_a16(x, w, N, H, W, Co, kh, kw, sh, sw, dh, Ho, Wo, e, s);
     if (st >= 0) return st;

@@ -12,7 +12,10 @@ int igemm_dma_launch(int load, const void *a, const void *b, IgemmParams p, cons
   // buffer offsets are 32-bit and 0x80000000 must stay out of range
   if (a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || a_bytes <= 0 || b_bytes <= 0) return -1;
   if (load == LOAD_GEMM) return igemm_dma_launch_gemm(a, b, p, e, a_bytes, b_bytes, s);
-  if (load == LOAD_CONV) return pick_dma_tile<LOAD_CONV>(a, b, p, e, a_bytes, b_bytes, s);
+  if (load == LOAD_CONV) {
+    if (p.M >= (1ll << 31)) return -1;  // the loader splits a pixel index with 32-bit divisions
+    return pick_dma_tile<LOAD_CONV>(a, b, p, e, a_bytes, b_bytes, s);
+  }
   return -1;
 }
 
