@@ -16,6 +16,9 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
 int gemm_nt_mfma_a16(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
 int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
                     int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
+int gemm_nt_mfma_a16w16(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
+int conv2d_mfma_a16w16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
+                       int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
 int conv2d_dual_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
                    int sh, int sw, int dh, int dw, int Ho, int Wo, const void *xs, const void *ws, int Hs, int Ws, int Cs,
                    int ss, const EpiDev &e, const ShortcutDev &sc, hipStream_t s);
@@ -23,7 +26,7 @@ bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
 
-enum Route { kDirect, kMfma, kMfmaA16, kDepthwise, kBad };
+enum Route { kDirect, kMfma, kMfmaA16, kMfmaA16W16, kDepthwise, kBad };
 
 static Route gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k, const void *a, const void *b) {
   if (a_bits == 8 && b_bits == 8 && k % 16 == 0 && k >= 16 && m > 0 && n > 0 && k < (1ll << 31) &&
@@ -33,6 +36,10 @@ static Route gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k,
   if (a_bits == 16 && b_bits == 8 && k % 8 == 0 && k >= 8 && m > 0 && n > 0 && m * k < (1ll << 30) &&
       n * k < (1ll << 31) && (!a || aligned16(a)) && (!b || aligned16(b)))
     return kMfmaA16;
+  // int16 x int16: four digit products per K step, exact 64-bit sums
+  if (a_bits == 16 && b_bits == 16 && k % 8 == 0 && k >= 8 && k < (1 << 16) && m > 0 && n > 0 && m * k < (1ll << 30) &&
+      n * k < (1ll << 30) && (!a || aligned16(a)) && (!b || aligned16(b)))
+    return kMfmaA16W16;
   return kDirect;
 }
 
@@ -50,6 +57,10 @@ static Route conv_route(int x_bits, int w_bits, const catchq_conv_desc_t *d, con
       (int64_t)d->n * d->h * d->w * d->ci < (1ll << 30) && (int64_t)d->co * d->kh * d->kw * d->ci < (1ll << 31) &&
       (!x || aligned16(x)) && (!w || aligned16(w)))
     return kMfmaA16;
+  if (x_bits == 16 && w_bits == 16 && d->groups == 1 && d->ci % 8 == 0 && d->kh * d->kw <= 32 &&
+      (int64_t)d->kh * d->kw * d->ci < (1 << 16) && (int64_t)d->n * d->h * d->w * d->ci < (1ll << 30) &&
+      (int64_t)d->co * d->kh * d->kw * d->ci < (1ll << 30) && (!x || aligned16(x)) && (!w || aligned16(w)))
+    return kMfmaA16W16;
   return kDirect;
 }
 
@@ -57,6 +68,7 @@ static const char *route_name(Route r) {
   switch (r) {
     case kMfma: return "mfma";
     case kMfmaA16: return "mfma_a16";
+    case kMfmaA16W16: return "mfma_a16w16";
     case kDepthwise: return "depthwise";
     case kDirect: return "direct";
     default: return "invalid";
@@ -106,6 +118,10 @@ CATCHQ_API int catchq_gemm_nt(const void *a, int a_bits, const void *b, int b_bi
     const int st = gemm_nt_mfma_a16(a, b, m, n, k, e, s);
     if (st >= 0) return st;
   }
+  if (route == kMfmaA16W16) {
+    const int st = gemm_nt_mfma_a16w16(a, b, m, n, k, e, s);
+    if (st >= 0) return st;
+  }
   return gemm_nt_direct(a, a_bits, b, b_bits, m, n, k, e, s);
 }
 
@@ -134,13 +150,19 @@ CATCHQ_API int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int 
       const int st2 = conv2d_mfma_a16(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h,
                                       d.stride_w, d.dil_h, d.dil_w, ho, wo, e, s);
       if (st2 >= 0) return st2;
-    }  // not eligible after all: fall through to the direct kernel
-    default: {
-      ConvDev cd = {d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h, d.stride_w,
-                    d.dil_h, d.dil_w, d.groups, ho, wo};
-      return conv2d_direct(x, x_bits, w, w_bits, cd, e, s);
+      break;  // not eligible after all: the direct kernel
     }
+    case kMfmaA16W16: {
+      const int st2 = conv2d_mfma_a16w16(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h,
+                                         d.stride_w, d.dil_h, d.dil_w, ho, wo, e, s);
+      if (st2 >= 0) return st2;
+      break;
+    }
+    default: break;
   }
+  ConvDev cd = {d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h, d.stride_w,
+                d.dil_h, d.dil_w, d.groups, ho, wo};
+  return conv2d_direct(x, x_bits, w, w_bits, cd, e, s);
 }
 
 // shapes the two-branch kernel serves (pointer alignment is checked at the call)

@@ -326,6 +326,213 @@ int gemm_nt_mfma_a16(const void *a, const void *b, int64_t M, int64_t N, int64_t
   return igemm_a16_launch(LOAD_GEMM, a, b, p, e, M * K * 2, N * K, s);
 }
 
+// ---- int16 x int16 ------------------------------------------------------------------------------------------
+// Both operands split into digits:  x = 256*xh + xl + 128,  w = 256*wh + wl + 128  (high byte signed, low byte
+// biased into int8), so
+//   sum x*w = 65536*S_hh + 256*(S_hl + S_lh) + S_ll + 32768*(sum xh + sum wh) + 128*(sum xl + sum wl) + 16384*Kp
+// with four int8 x int8 MFMA sums S_.. , the digit sums of the row (activations) and of the column (weights), which
+// the wave collects from the fragments it loads anyway, and Kp the number of K positions walked (whole steps: a
+// position beyond K, a row beyond M or N and an out-of-image tap all read as zeros, which decode to the value 0 on
+// either side, so the identity covers them).  Every partial sum fits an int32 (|S| <= Kp * 2^14); the combination
+// is done in 64-bit integers and is the exact sum, which is what the int16 x int16 contraction is defined on.
+// One tile shape (64 x 64, four waves of 32 x 32), element-wise epilogue from the accumulators.
+template <int LOAD>
+__global__ __launch_bounds__(256) void igemm_a16w16_kernel(const int16_t *__restrict__ A, const int16_t *__restrict__ B,
+                                                          IgemmParams p, EpiDev e, unsigned a_bytes, unsigned b_bytes) {
+  resolve_exp2(e);
+  constexpr int BM = 64, BN = 64, STAGES = 3;
+  constexpr int A_STAGE = BM * BK * 2, STAGE_BYTES = (BM + BN) * BK * 2;
+  constexpr int PIPE_BYTES = STAGES * STAGE_BYTES;
+  constexpr int NIA = BM / 8;                 // DMA instructions (1 KiB: 8 rows x 128 bytes) per stage and operand
+  constexpr int NI = (BM + BN) / 8 / 4;       // per wave
+  extern __shared__ __attribute__((aligned(16))) int8_t lds_dyn[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int logical = xcd_remap(blockIdx.x, p.nblocks);
+  const int tile_n = logical % p.tiles_n;
+  const int tile_m = logical / p.tiles_n;
+  const int64_t m0 = (int64_t)tile_m * BM;
+  const int n0 = tile_n * BN;
+
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A, 0, (int)a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)B, 0, (int)b_bytes, 0x00020000);
+  constexpr unsigned OOB = 0x80000000u;
+
+  unsigned rowbase[NI];
+  unsigned vmask[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int slot = wave * NI + j;
+    if (slot < NIA) {
+      const int64_t m = m0 + slot * 8 + (lane >> 3);
+      const bool ok = m < p.M;
+      const int64_t mm = ok ? m : 0;
+      if constexpr (LOAD == LOAD_CONV) {
+        const unsigned mu = (unsigned)mm;
+        const unsigned t = mu / (unsigned)p.Wo;
+        const int wo = (int)(mu - t * (unsigned)p.Wo);
+        const unsigned img = t / (unsigned)p.Ho;
+        const int ho = (int)(t - img * (unsigned)p.Ho);
+        const int hi0 = ho * p.sh - p.ph, wi0 = wo * p.sw - p.pw;
+        rowbase[j] = 2u * ((unsigned)((int64_t)img * p.H * p.W * p.Ci) + (unsigned)((hi0 * p.W + wi0) * p.Ci));  // mod 2^32
+        unsigned mask = 0;
+        for (int r = 0; r < p.kh; ++r)
+          for (int q = 0; q < p.kw; ++q)
+            if ((unsigned)(hi0 + r * p.dh) < (unsigned)p.H && (unsigned)(wi0 + q * p.dw) < (unsigned)p.W)
+              mask |= 1u << (r * p.kw + q);
+        vmask[j] = ok ? mask : 0u;
+      } else {
+        rowbase[j] = (unsigned)(mm * p.K * 2);
+        vmask[j] = ok ? 1u : 0u;
+      }
+    } else {
+      const int n = n0 + (slot - NIA) * 8 + (lane >> 3);
+      const bool ok = n < p.N;
+      rowbase[j] = (unsigned)((int64_t)(ok ? n : 0) * p.K * 2);
+      vmask[j] = ok ? 1u : 0u;
+    }
+  }
+  int k_lin = ((lane & 7) ^ (lane >> 3)) * 8;  // this lane's K position (elements) in either operand
+  int kr = 0, kq = 0, kci = k_lin, tap = 0;
+  unsigned tapbase = 0;
+  auto normalise_tap = [&]() {
+    while (kci >= p.Ci) {
+      kci -= p.Ci;
+      ++tap;
+      if (++kq == p.kw) { kq = 0; ++kr; }
+      tapbase = (unsigned)((kr * p.dh * p.W + kq * p.dw) * p.Ci);
+    }
+  };
+  if constexpr (LOAD == LOAD_CONV) normalise_tap();
+
+  auto issue_stage = [&](int stage_off) {
+    const bool k_ok = k_lin < p.K;
+    const unsigned a_koff = 2u * ((LOAD == LOAD_CONV) ? tapbase + (unsigned)kci : (unsigned)k_lin);
+    const unsigned a_bit = (LOAD == LOAD_CONV) ? (1u << tap) : 1u;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int slot = wave * NI + j;
+      const bool is_a = slot < NIA;  // wave-uniform
+      lds_ptr_t dst = (lds_ptr_t)(lds_dyn + stage_off + slot * 1024);
+      if (is_a) {
+        const unsigned voff = select_u32(k_ok && (vmask[j] & a_bit), rowbase[j] + a_koff, OOB);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, (int)voff, 0, 0, 0);
+      } else {
+        const unsigned voff = select_u32(k_ok && vmask[j], rowbase[j] + 2u * (unsigned)k_lin, OOB);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, (int)voff, 0, 0, 0);
+      }
+    }
+    k_lin += BK;
+    if constexpr (LOAD == LOAD_CONV) {
+      kci += BK;
+      normalise_tap();
+    }
+  };
+
+  v16i s_hh, s_hl, s_lh, s_ll;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { s_hh[r] = 0; s_hl[r] = 0; s_lh[r] = 0; s_ll[r] = 0; }
+  int xh_sum = 0, xl_sum = 0, wh_sum = 0, wl_sum = 0;
+
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)lds_dyn;
+  const unsigned c0 = (unsigned)(((fhalf * 2) ^ (frow & 7)) * 16);
+  const unsigned a_row = lds_base + (unsigned)((wave_m * 32 + frow) * (BK * 2));
+  const unsigned b_row = lds_base + (unsigned)(A_STAGE + (wave_n * 32 + frow) * (BK * 2));
+
+  auto half_step = [&](unsigned a_base, unsigned b_base, unsigned chunk) {
+    v4i fa0 = ds_read_b128<0>(a_base + chunk), fa1 = ds_read_b128<0>(a_base + (chunk ^ 16u));
+    v4i fb0 = ds_read_b128<0>(b_base + chunk), fb1 = ds_read_b128<0>(b_base + (chunk ^ 16u));
+    lgkm_wait<0>(fa0, fa1, fb0, fb1);
+    v4i xh, xl, wh, wl;
+    split_i16(fa0, fa1, xh, xl);
+    split_i16(fb0, fb1, wh, wl);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      xh_sum = __builtin_amdgcn_sdot4(xh[d], 0x01010101, xh_sum, false);
+      xl_sum = __builtin_amdgcn_sdot4(xl[d], 0x01010101, xl_sum, false);
+      wh_sum = __builtin_amdgcn_sdot4(wh[d], 0x01010101, wh_sum, false);
+      wl_sum = __builtin_amdgcn_sdot4(wl[d], 0x01010101, wl_sum, false);
+    }
+    s_hh = __builtin_amdgcn_mfma_i32_32x32x32_i8(xh, wh, s_hh, 0, 0, 0);
+    s_hl = __builtin_amdgcn_mfma_i32_32x32x32_i8(xh, wl, s_hl, 0, 0, 0);
+    s_lh = __builtin_amdgcn_mfma_i32_32x32x32_i8(xl, wh, s_lh, 0, 0, 0);
+    s_ll = __builtin_amdgcn_mfma_i32_32x32x32_i8(xl, wl, s_ll, 0, 0, 0);
+  };
+
+  const int nsteps = (p.K + BK - 1) / BK;
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue_stage(s * STAGE_BYTES);
+  int rd_off = 0, wr_off = (STAGES - 1) * STAGE_BYTES;
+  for (int step = 0; step < nsteps; ++step) {
+    CATCHQ_VMCNT(NI * (STAGES - 2));
+    __builtin_amdgcn_s_barrier();
+    issue_stage(wr_off);
+    half_step(a_row + (unsigned)rd_off, b_row + (unsigned)rd_off, c0);
+    half_step(a_row + (unsigned)rd_off, b_row + (unsigned)rd_off, c0 ^ 64u);
+    rd_off = (rd_off + STAGE_BYTES == PIPE_BYTES) ? 0 : rd_off + STAGE_BYTES;
+    wr_off = (wr_off + STAGE_BYTES == PIPE_BYTES) ? 0 : wr_off + STAGE_BYTES;
+  }
+  CATCHQ_VMCNT(0);
+
+  // a lane holds the digit sums of A row / B row (lane & 31) over its half of every K step: add the halves
+  xh_sum += __shfl_xor(xh_sum, 32, 64);
+  xl_sum += __shfl_xor(xl_sum, 32, 64);
+  wh_sum += __shfl_xor(wh_sum, 32, 64);
+  wl_sum += __shfl_xor(wl_sum, 32, 64);
+  // accumulator register r of a lane is row 8*(r>>2) + 4*(lane>>5) + (r&3), column lane & 31 of the 32 x 32 tile
+  const int64_t col_part = 32768ll * wh_sum + 128ll * wl_sum + 16384ll * ((int64_t)nsteps * BK);
+  const int n = n0 + wave_n * 32 + frow;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = 8 * (r >> 2) + 4 * fhalf + (r & 3);
+    const int rxh = __shfl(xh_sum, row, 64), rxl = __shfl(xl_sum, row, 64);
+    const int64_t m = m0 + wave_m * 32 + row;
+    if (n >= p.N || m >= p.M) continue;
+    const int64_t total = ((int64_t)s_hh[r] << 16) + (((int64_t)s_hl[r] + (int64_t)s_lh[r]) << 8) + (int64_t)s_ll[r] +
+                          32768ll * rxh + 128ll * rxl + col_part;
+    const int64_t idx = m * p.N + n;
+    epi_store(epi_value((float)total, idx, n, e), idx, e);
+  }
+}
+
+template <int LOAD>
+static int launch_a16w16(const void *a, const void *b, IgemmParams p, const EpiDev &e, int64_t a_bytes, int64_t b_bytes,
+                         hipStream_t s) {
+  if (a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || a_bytes <= 0 || b_bytes <= 0) return -1;
+  if (e.acc_out) return -1;  // the exact sum is a 64-bit integer: no int32 accumulator output
+  if (p.M >= (1ll << 31) - 64 || p.K >= (1 << 16)) return -1;  // 32-bit pixel index; partial sums within int32
+  p.tiles_n = (p.N + 63) / 64;
+  const int64_t nb = ((p.M + 63) / 64) * p.tiles_n;
+  if (nb > 0x7fffffff) return -1;
+  p.nblocks = (int)nb;
+  igemm_a16w16_kernel<LOAD><<<p.nblocks, 256, 3 * 128 * BK * 2, s>>>((const int16_t *)a, (const int16_t *)b, p, e,
+                                                                     (unsigned)a_bytes, (unsigned)b_bytes);
+  return launch_status();
+}
+
+// int16 x int16 contractions on the matrix cores; -1 when the shape is not eligible
+int gemm_nt_mfma_a16w16(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s) {
+  IgemmParams p = {};
+  p.M = M;
+  p.N = (int)N;
+  p.K = (int)K;
+  return launch_a16w16<LOAD_GEMM>(a, b, p, e, M * K * 2, N * K * 2, s);
+}
+
+int conv2d_mfma_a16w16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
+                       int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
+  IgemmParams p = {};
+  p.M = (int64_t)N * Ho * Wo;
+  p.N = Co;
+  p.H = H; p.W = W; p.Ci = Ci; p.Ho = Ho; p.Wo = Wo;
+  p.kh = kh; p.kw = kw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+  p.K = kh * kw * Ci;
+  return launch_a16w16<LOAD_CONV>(x, w, p, e, (int64_t)N * H * W * Ci * 2, (int64_t)Co * p.K * 2, s);
+}
+
 // ---- few-channel first layer, int16 activations -------------------------------------------------
 // Input [N, H, W, 8] int16 already framed by its zero padding, filter rows padded to 4 taps (weights
 // [Co][kh][4][8] int8, the extra tap zero).  A filter row is 64 contiguous bytes of an image row and

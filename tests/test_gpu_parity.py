@@ -267,6 +267,38 @@ def test_gemm_wide(bits, m, n, k):
     assert same_bits(orc.epilogue(acc, -20, None, bias), out["y"].cpu().numpy())
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (200, 130, 72), (1, 1, 8), (96, 75, 1024), (3 * 10 * 10, 64, 576), (500, 300, 8200)])
+def test_gemm_a16w16_extreme_digits(m, n, k):
+    """int16 x int16 on the matrix cores (four int8 digit products, digit sums of rows and columns, 64-bit
+    combination): every digit pattern that could break the split -- -32768, 32767, -1, 0, +-128, 255, 256, all
+    low bytes 0x80, all high bytes 0x80 -- on both operands, the exact int64 sums through a power-of-two
+    epilogue that loses nothing (|sum| < 2^24 is not required: the comparison is with the oracle's float of the
+    same integer), and K not a multiple of the 64-element step."""
+    assert cabi.lib().catchq_gemm_route(16, 16, m, n, k) == b"mfma_a16w16"
+    note("gemm_a16w16", m, n, k)
+    r = rng(m * 7 + n + k)
+    a, b = _ints(r, (m, k), 16), _ints(r, (n, k), 16)
+    ext = np.array([-32768, 32767, -1, 0, 128, -128, 255, 256, -129, 127, -32641, 32640], np.int16)
+    a[0, :min(k, 12)] = ext[:min(k, 12)]
+    b[0, :min(k, 12)] = ext[::-1][:min(k, 12)]
+    if m > 2 and n > 2:
+        a[1] = -32768; b[1] = -32768          # the largest product everywhere: 2^30 * K
+        a[2] = 32767; b[2] = -32768
+        a[m - 1] = 0x0080 - 0 if k else 0     # low byte 0x80, high byte 0
+        b[n - 1] = -128                        # 0xff80
+    acc, _ = orc.gemm_nt(a, b)
+    assert acc.dtype == np.int64 and (m < 3 or n < 3 or acc[1, 1] == k * 2 ** 30)
+    bias = r.standard_normal(n).astype(np.float32)
+    out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=-30, bias=cabi.dev(bias), want_acc=False)
+    assert same_bits(orc.epilogue(acc, -30, None, bias), out["y"].cpu().numpy())
+    # small values: the sums stay below 2^24, the fp32 output with exp2 = 0 and no bias is the integer itself
+    a2, b2 = (a // 4096).astype(np.int16), (b // 4096).astype(np.int16)
+    acc2, _ = orc.gemm_nt(a2, b2)
+    if np.abs(acc2).max() < 2 ** 24:
+        y2 = cabi.gemm_nt(cabi.dev(a2), cabi.dev(b2), want_acc=False)["y"].cpu().numpy()
+        assert np.array_equal(y2.astype(np.int64), acc2)
+
+
 @pytest.mark.parametrize("m,n,k", [(16384, 1024, 1024), (8192, 768, 320), (4096, 768, 256), (4096, 3072, 768)])
 def test_gemm_a16_tiles(m, n, k):
     """int16 x int8 on the matrix cores (the first shape takes the wide 128x256 tile), with the extreme digits

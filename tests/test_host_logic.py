@@ -116,7 +116,8 @@ def test_routes(lib):
     assert route(4, 64, 7, 1) == "mfma"
     assert route(32, 32, 3, 32) == "depthwise"
     assert route(4, 16, 3, 2) == "direct"
-    assert route(64, 64, 3, 1, (16, 16)) == "direct"
+    assert route(64, 64, 3, 1, (16, 16)) == "mfma_a16w16"
+    assert route(4, 32, 3, 1, (16, 16)) == "direct"
     assert route(64, 64, 3, 1, (16, 8)) == "mfma_a16"
     assert route(8, 32, 3, 1, (16, 8)) == "mfma_a16"
     assert route(4, 32, 3, 1, (16, 8)) == "direct"
@@ -124,7 +125,8 @@ def test_routes(lib):
     assert lib.catchq_gemm_route(8, 8, 4096, 3072, 768) == b"mfma"
     assert lib.catchq_gemm_route(8, 8, 10, 25, 10) == b"direct"
     assert lib.catchq_gemm_route(16, 8, 4096, 3072, 768) == b"mfma_a16"
-    assert lib.catchq_gemm_route(16, 16, 4096, 3072, 768) == b"direct"
+    assert lib.catchq_gemm_route(16, 16, 4096, 3072, 768) == b"mfma_a16w16"
+    assert lib.catchq_gemm_route(16, 16, 40, 30, 70000) == b"direct"  # K beyond what int32 digit sums hold
 
 
 # ------------------------------------------------------------------ the Python tool (A1/A2/A15)
