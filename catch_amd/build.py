@@ -81,8 +81,17 @@ def build_torch_ext(verbose=False):
     return out
 
 
+def build_probes(verbose=False):
+    """stand-alone measurement programs (catch_amd/lib/probe_mfma: what the matrix cores sustain on this device)"""
+    out = os.path.join(LIBDIR, "probe_mfma")
+    o = _run([HIPCC, "--offload-arch=gfx950", "-O3", "-o", out, os.path.join(CSRC, "probe_mfma.hip")])
+    if verbose and o.strip():
+        print(o)
+    return out
+
+
 def build_all(verbose=False):
-    return build_kernels(verbose), build_torch_ext(verbose)
+    return build_kernels(verbose), build_torch_ext(verbose), build_probes(verbose)
 
 
 if __name__ == "__main__":
@@ -91,3 +100,5 @@ if __name__ == "__main__":
         print(build_kernels(True))
     if which in ("torch", "all"):
         print(build_torch_ext(True))
+    if which in ("probes", "all"):
+        print(build_probes(True))
