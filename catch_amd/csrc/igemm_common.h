@@ -17,6 +17,12 @@ struct IgemmParams {
   unsigned img_stride, row_stride, pix_stride;
   int tiles_n;
   int nblocks;
+  // Order in which consecutive block ids walk the tile grid: 0 = row by row (all column tiles of one row tile,
+  // then the next row tile); g > 0 = in bands of g row tiles, column by column inside a band, so that the blocks
+  // running at the same time cover a g x (concurrent / g) patch of tiles and share both operands' panels in L2
+  // instead of streaming the whole B operand past every row tile.
+  int group_m;
+  int tiles_m;
 };
 
 constexpr int BK = 64;  // bytes of K per pipeline step (one LDS row)

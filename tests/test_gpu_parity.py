@@ -321,6 +321,25 @@ def test_gemm_a16_tiles(m, n, k):
     assert torch.equal(hi * 256 + lo + 128 * bsum[None, :], out["acc"])
 
 
+@pytest.mark.parametrize("m,n,k", [(4997, 2100, 512), (2500, 1100, 1024), (9001, 600, 256), (6000, 4100, 128)])
+def test_gemm_banded_tile_order(m, n, k):
+    """grids that are large in both directions walk their tiles in bands of eight row tiles; ragged last band,
+    ragged last row and column tiles: rows sampled from every band against the oracle, and every row of C
+    against the sum over K halves (two launches whose grids walk the same way)"""
+    note("gemm_banded", m, n, k)
+    r = rng(m + n + k)
+    a, b = _ints(r, (m, k), 8), _ints(r, (n, k), 8)
+    acc = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), y_dtype=None)["acc"]
+    rows = np.unique(np.concatenate([np.arange(0, m, 97), [m - 1, m - 2, 63, 64, 255, 256, 2047, 2048]]))
+    rows = rows[rows < m]
+    want, ovf = orc.gemm_nt(a[rows], b)
+    assert ovf == 0 and np.array_equal(want.astype(np.int32), acc.cpu().numpy()[rows])
+    h = k // 2
+    s = cabi.gemm_nt(cabi.dev(a[:, :h]), cabi.dev(b[:, :h]), y_dtype=None)["acc"] + \
+        cabi.gemm_nt(cabi.dev(a[:, h:]), cabi.dev(b[:, h:]), y_dtype=None)["acc"]
+    assert torch.equal(s, acc)
+
+
 def test_gemm_full_size_properties():
     """Config-2 sizes: too big for the oracle in seconds, so check what the integers must satisfy:
     rows of A that are copies give equal rows of C, and a sampled set of entries equals the
