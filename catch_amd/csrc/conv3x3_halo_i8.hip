@@ -1,0 +1,371 @@
+// 3x3 int8 convolution (stride 1, padding 1) with the input patch resident in LDS.
+//
+// The implicit-GEMM kernel fetches every input pixel nine times (once per filter tap) and synchronises
+// its block once per 64 bytes of K, which leaves a 3x3 layer bound by the load path when the image is
+// large and by the per-step latency chain when it is small.  Here a block owns a band of whole output
+// rows of one image (or a few whole small images): it loads the band's input rows plus a one-pixel
+// frame into LDS ONCE -- rows and columns outside the image arrive as zeros from the out-of-range
+// buffer loads, which is the convolution's padding -- and every filter tap then reads the A fragments
+// of its pixels from that patch at a shifted address.  Only the weights stream: stages of 256 bytes of
+// K for the block's output channels through a three-slot LDS ring, one barrier per stage, so a wave
+// issues 16 to 32 MFMAs per synchronisation instead of two.
+//
+//   patch        PR x PC pixels of CI bytes; the 16-byte chunks of a pixel are XOR-swizzled with low
+//                bits of the pixel index (on the source side of the LDS-DMA) so that the ds_read_b128
+//                of 32 consecutive pixels at one logical chunk spread over all banks
+//   output tile  P = TR * Wo consecutive output pixels (rows m0 .. m0 + P of the GEMM view), split
+//                into 32-row MFMA sub-tiles; wave w owns sub-tiles w and w + 4; BN = 32 * TN channels
+//   K order      (tap, channel), as the weight tensor [Co][3][3][Ci] stores it; a stage may end past
+//                K: weights beyond K read as zeros, the patch address of a tap >= 9 is clamped
+//
+// The integer sums are those of any other route (exact), the epilogue is the shared one.
+#include <type_traits>
+
+#include "igemm_i8_dma.inc"
+
+namespace catchq {
+
+struct HaloParams {
+  int N, H, W, Co;       // input [N, H, W, CI]; output [N, H, W, Co]
+  int TR;                // output rows per tile
+  int image_mode;        // 0: a band of TR rows of one image (the last band of an image may be shorter);
+                         // 1: TR = G * H, G whole images
+  int bands;             // bands per image (band mode)
+  int PR, PC;            // patch rows / columns (PC = W + 2)
+  int P;                 // output pixels per tile = TR * W
+  int nsub;              // 32-row sub-tiles per tile
+  int tiles_n, nblocks;
+  int64_t M;             // N * H * W
+  unsigned x_bytes, w_bytes;
+};
+
+// f(integral_constant<int, G>) for G = 0 .. N-1, expanded at compile time (a #pragma unroll over this many large
+// bodies is declined by the optimizer, and the fragment registers must never be indexed at run time)
+template <int G, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (G < N) {
+    f(std::integral_constant<int, G>{});
+    static_for<G + 1, N>(f);
+  }
+}
+
+// swizzle of a pixel's 16-byte chunk index; CH = chunks per pixel
+template <int CH>
+__device__ __forceinline__ unsigned halo_swz(unsigned pix) {
+  if constexpr (CH == 4) return (pix >> 2) & 3u;
+  else if constexpr (CH == 8) return (pix >> 1) & 7u;
+  else return pix & 15u;
+}
+
+template <int CI, int TN, int TMW, int EPI>
+__global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                          HaloParams hp, EpiDev e) {
+  resolve_exp2(e);
+  constexpr int CH = CI / 16;         // 16-byte chunks per pixel
+  constexpr int LOG_CI = CI == 64 ? 6 : CI == 128 ? 7 : CI == 256 ? 8 : 9;
+  constexpr int BN = 32 * TN;
+  constexpr int KS = 256;             // bytes of K per weight stage
+  constexpr int STAGES = 3;
+  constexpr int B_STAGE = BN * KS;
+  constexpr int NIB = BN / 4 / 4;     // weight DMA instructions (4 rows x 256 bytes) per wave and stage
+  constexpr int K = 9 * CI;
+  constexpr int NSTAGES = (K + KS - 1) / KS;
+  constexpr int SUBS_PER_TAP = CI / 32;  // MFMA K steps (32 bytes) per filter tap
+  constexpr int SUBS_PER_STAGE = KS / 32;
+  static_assert(BN / 4 % 4 == 0, "the weight rows must split evenly over the four waves");
+  static_assert(TMW == 1 || TMW == 2, "one or two sub-tiles per wave");
+  // 1 KiB alignment: fragment addresses are formed by XOR-ing chunk bits into a precomputed address
+  extern __shared__ __attribute__((aligned(1024))) int8_t lds_dyn[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int logical = xcd_remap(blockIdx.x, hp.nblocks);
+  const int tile_n = logical % hp.tiles_n;
+  const int tile_m = logical / hp.tiles_n;
+  const int n0 = tile_n * BN;
+  // first image, first output row and output pixel count of the tile
+  int img0, ho0, p_tile;
+  if (hp.image_mode) {
+    img0 = tile_m * (hp.TR / hp.H);
+    ho0 = 0;
+    p_tile = hp.P;
+  } else {
+    img0 = tile_m / hp.bands;
+    ho0 = (tile_m - img0 * hp.bands) * hp.TR;
+    const int rows = hp.H - ho0 < hp.TR ? hp.H - ho0 : hp.TR;
+    p_tile = rows * hp.W;
+  }
+  const int64_t m0 = ((int64_t)img0 * hp.H + ho0) * hp.W;
+  const int patch_bytes = (hp.PR * hp.PC * CI + 1023) / 1024 * 1024;
+  int8_t *ring = lds_dyn + patch_bytes;
+
+  const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc((void *)X, 0, (int)hp.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void *)Wt, 0, (int)hp.w_bytes, 0x00020000);
+  constexpr unsigned OOB = 0x80000000u;
+
+  // ---- the input patch: every 16-byte chunk once ------------------------------------------------------------
+  {
+    const int npix = hp.PR * hp.PC;
+    const int ninstr = patch_bytes / 1024;
+    constexpr int PPI = 64 / CH > 0 ? 64 / CH : 1;  // pixels per DMA instruction (CH <= 32)
+    // this lane's pixel in the wave's first instruction, then PPI * 4 pixels further per round
+    unsigned pix = (unsigned)(wave * 64 + lane) / CH;
+    const unsigned phys = (unsigned)lane % CH;
+    unsigned pr = pix / (unsigned)hp.PC, pc = pix - pr * (unsigned)hp.PC;
+    for (int i = wave; i < ninstr; i += 4) {
+      int img = img0, hi;
+      if (hp.image_mode) {
+        const unsigned g = pr / (unsigned)(hp.H + 2);
+        img += (int)g;
+        hi = (int)(pr - g * (unsigned)(hp.H + 2)) - 1;
+      } else {
+        hi = ho0 - 1 + (int)pr;
+      }
+      const int wi = (int)pc - 1;
+      const bool ok = (int)pix < npix && img < hp.N && (unsigned)hi < (unsigned)hp.H && (unsigned)wi < (unsigned)hp.W;
+      const unsigned src = (unsigned)((img * hp.H + hi) * hp.W + wi) * (unsigned)CI + ((phys ^ halo_swz<CH>(pix)) << 4);
+      const unsigned voff = select_u32(ok, src, OOB);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(lds_dyn + i * 1024), 16, (int)voff, 0, 0, 0);
+      pix += PPI * 4;
+      pc += PPI * 4;
+      while (pc >= (unsigned)hp.PC) { pc -= (unsigned)hp.PC; ++pr; }
+    }
+  }
+
+  // ---- the weight ring ---------------------------------------------------------------------------------------
+  // instruction b of a stage: rows 4b .. 4b+3 of the block's BN weight rows, 16 chunks each
+  unsigned wbase[NIB];
+  bool wrow_ok[NIB];
+#pragma unroll
+  for (int t = 0; t < NIB; ++t) {
+    const int rb = (wave * NIB + t) * 4 + (lane >> 4);
+    wrow_ok[t] = n0 + rb < hp.Co;
+    wbase[t] = (unsigned)(n0 + rb) * (unsigned)K + ((((unsigned)lane & 15u) ^ ((unsigned)rb & 15u)) << 4);
+  }
+  auto issue_weights = [&](int stage, int slot_off) {
+    const unsigned k0 = (unsigned)stage * KS;
+#pragma unroll
+    for (int t = 0; t < NIB; ++t) {
+      const unsigned kk = k0 + ((((unsigned)lane & 15u) ^ ((unsigned)((wave * NIB + t) * 4 + (lane >> 4)) & 15u)) << 4);
+      const unsigned voff = select_u32(wrow_ok[t] && kk < (unsigned)K, wbase[t] + k0, OOB);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_ptr_t)(ring + slot_off + (wave * NIB + t) * 1024), 16, (int)voff, 0,
+                                               0, 0);
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue_weights(s, s * B_STAGE);
+
+  // ---- this lane's fragment addresses: one per sub-tile and filter tap ------------------------------------------
+  // The A fragment of K step c (32 bytes: chunks 2c and 2c+1, this lane takes chunk 2c + fhalf) of a pixel sits at
+  //   pixel * CI + (((2c + fhalf) ^ swz(pixel)) << 4)  =  [pixel * CI + ((fhalf ^ swz(pixel)) << 4)]  ^  (c << 5):
+  // the bracket is fixed per (sub-tile, tap), the XOR mask is the same for every lane.
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)lds_dyn;
+  unsigned a0[TMW][9];
+#pragma unroll
+  for (int i = 0; i < TMW; ++i) {
+    int idx = (wave + 4 * i) * 32 + frow;
+    if (idx >= p_tile) idx = p_tile - 1;
+    const unsigned tr = (unsigned)idx / (unsigned)hp.W, wo = (unsigned)idx - tr * (unsigned)hp.W;
+    unsigned prow = tr;
+    if (hp.image_mode) {
+      const unsigned g = tr / (unsigned)hp.H;
+      prow = g * (unsigned)(hp.H + 2) + (tr - g * (unsigned)hp.H);
+    }
+    const unsigned pixbase = prow * (unsigned)hp.PC + wo;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) {
+      const unsigned pix = pixbase + (unsigned)(t / 3) * (unsigned)hp.PC + (unsigned)(t % 3);
+      a0[i][t] = lds_base + pix * (unsigned)CI + ((((unsigned)fhalf) ^ halo_swz<CH>(pix)) << 4);
+    }
+  }
+  // weights: row frow of a 32-row block, chunk (2c + fhalf) ^ (frow & 15) of the stage's 16
+  const unsigned ring_base = lds_base + (unsigned)patch_bytes;
+  const unsigned b0 = ring_base + (unsigned)frow * KS + ((((unsigned)fhalf) ^ ((unsigned)frow & 15u)) << 4);
+
+  v16i acc[TMW][TN];
+#pragma unroll
+  for (int i = 0; i < TMW; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  auto multiply = [&](v4i (&fa)[TMW], v4i (&fb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TMW; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  };
+
+  // the patch and the first weight stages: everything issued so far has landed, for every wave
+  CATCHQ_VMCNT(0);
+  __syncthreads();
+
+  // The whole K loop is unrolled: tap and chunk of every step are compile-time constants, a step costs one XOR
+  // per fragment address.  g counts 32-byte K steps; every SUBS_PER_STAGE of them a new weight stage begins.
+  constexpr int NSUB_K = 9 * SUBS_PER_TAP;
+  unsigned bslot = b0;  // this lane's weight fragment address in the stage being read
+  int wr_off = (STAGES - 1) * B_STAGE, rd_off = 0;
+  v4i fa[2][TMW], fb[2][TN];
+  auto fetch = [&](v4i (&xa)[TMW], v4i (&xb)[TN], int tap, int c, int cb) {
+#pragma unroll
+    for (int i = 0; i < TMW; ++i) xa[i] = ds_read_b128<0>(a0[i][tap] ^ (unsigned)(c << 5));
+    xb[0] = ds_read_b128<0>(bslot ^ (unsigned)(cb << 5));
+    if constexpr (TN > 1) xb[1] = ds_read_b128<32 * KS>(bslot ^ (unsigned)(cb << 5));
+  };
+  static_for<0, NSUB_K>([&](auto gc) {
+    constexpr int g = decltype(gc)::value;
+    constexpr int in_stage = g % SUBS_PER_STAGE;
+    if constexpr (in_stage == 0) {
+      constexpr int stage = g / SUBS_PER_STAGE;
+      if constexpr (stage > 0) {
+        CATCHQ_VMCNT(NIB * (STAGES - 2));  // this wave's part of the stage has landed
+        __builtin_amdgcn_s_barrier();      // ... and everyone's; the slot refilled below is no longer read
+      }
+      issue_weights(stage + STAGES - 1, wr_off);
+      bslot = b0 + (unsigned)rd_off;
+      rd_off = (rd_off + B_STAGE == STAGES * B_STAGE) ? 0 : rd_off + B_STAGE;
+      wr_off = (wr_off + B_STAGE == STAGES * B_STAGE) ? 0 : wr_off + B_STAGE;
+      fetch(fa[g & 1], fb[g & 1], g / SUBS_PER_TAP, g % SUBS_PER_TAP, in_stage);
+    }
+    // the next step's fragments are requested before this step's are waited for, inside a stage
+    constexpr bool more = (g + 1 < NSUB_K) && ((g + 1) % SUBS_PER_STAGE != 0);
+    if constexpr (more) {
+      fetch(fa[(g + 1) & 1], fb[(g + 1) & 1], (g + 1) / SUBS_PER_TAP, (g + 1) % SUBS_PER_TAP, (g + 1) % SUBS_PER_STAGE);
+      lgkm_wait_frags<TMW + TN, TMW, TN>(fa[g & 1], fb[g & 1]);
+    } else {
+      lgkm_wait_frags<0, TMW, TN>(fa[g & 1], fb[g & 1]);
+    }
+    multiply(fa[g & 1], fb[g & 1]);
+  });
+  CATCHQ_VMCNT(0);
+  __syncthreads();  // the ring is dead: it becomes the epilogue's staging area
+
+  IgemmParams p = {};
+  p.N = hp.Co;
+  p.M = (m0 + p_tile < hp.M) ? m0 + p_tile : hp.M;  // rows past the tile belong to the next one
+  constexpr int EPI_STRIDE = BN + 8;
+  int *stage_w = reinterpret_cast<int *>(ring) + wave * 32 * EPI_STRIDE;
+#pragma unroll
+  for (int i = 0; i < TMW; ++i) {
+    const int si = wave + 4 * i;
+    if (si * 32 >= p_tile) break;  // wave-uniform
+    igemm_epilogue<1, TN, EPI>(reinterpret_cast<v16i(&)[1][TN]>(acc[i]), stage_w, m0 + si * 32, n0, lane, p, e);
+  }
+}
+
+template <int CI, int TN, int TMW, int EPI>
+static int launch_halo_epi(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
+  auto kern = conv3x3_halo_kernel<CI, TN, TMW, EPI>;
+  if (lds_bytes > 64 * 1024) {
+    static std::atomic<bool> raised[64];
+    if (raise_lds_limit((const void *)kern, 160 * 1024, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
+  }
+  kern<<<hp.nblocks, 256, lds_bytes, s>>>((const int8_t *)x, (const int8_t *)w, hp, e);
+  return launch_status();
+}
+
+template <int CI, int TN, int TMW>
+static int launch_halo_tm(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
+  switch (pick_epilogue(hp.Co, e)) {
+    case EPI_SCALAR: return -1;
+    case EPI_Q8_RELU: return launch_halo_epi<CI, TN, TMW, EPI_Q8_RELU>(x, w, hp, e, lds_bytes, s);
+    default: return launch_halo_epi<CI, TN, TMW, EPI_VECTOR>(x, w, hp, e, lds_bytes, s);
+  }
+}
+
+template <int CI, int TN>
+static int launch_halo(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
+  // four or fewer sub-tiles: one per wave, no second set of accumulators
+  if (hp.nsub <= 4) return launch_halo_tm<CI, TN, 1>(x, w, hp, e, lds_bytes, s);
+  return launch_halo_tm<CI, TN, 2>(x, w, hp, e, lds_bytes, s);
+}
+
+// 3x3, stride 1, padding 1, no dilation, Ci in {64, 128, 256, 512}; -1: not this kernel's shape
+int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, const EpiDev &e, hipStream_t s) {
+  if (Ci != 64 && Ci != 128 && Ci != 256 && Ci != 512) return -1;
+  if (Co % 4 != 0 || W > 254 || (int64_t)N * H * W * Ci >= (1ll << 31) || (int64_t)Co * 9 * Ci >= (1ll << 31)) return -1;
+  if ((int64_t)N * H >= (1 << 24)) return -1;
+  HaloParams hp = {};
+  hp.N = N; hp.H = H; hp.W = W; hp.Co = Co;
+  hp.PC = W + 2;
+  hp.M = (int64_t)N * H * W;
+  hp.x_bytes = (unsigned)((int64_t)N * H * W * Ci);
+  hp.w_bytes = (unsigned)((int64_t)Co * 9 * Ci);
+  constexpr int kLdsLimit = 160 * 1024, kMaxP = 256, kRing1 = 3 * 32 * 256;
+  // Tile choice.  A tile of P pixels costs ceil(ceil(P / 32) / 4) rounds of MFMA work (four waves, one 32-row
+  // sub-tile each per round) plus about half a round of patch loading and synchronisation; the patch must fit
+  // beside the smaller weight ring.  Small images go whole, several per tile; larger ones are cut into bands of
+  // rows of equal height, the last band of an image possibly shorter.  Twice the cost is compared, in integers.
+  auto rounds2 = [](int pixels) { return 2 * (((pixels + 31) / 32 + 3) / 4) + 1; };
+  int best = 0, lds = 0, tn = 2;
+  int64_t tiles_m = 0;
+  if (H * W <= kMaxP / 2) {
+    int g_max = kMaxP / (H * W);
+    if (const char *t = tuning_env("CATCHQ_HALO_G")) g_max = atoi(t) < g_max ? atoi(t) : g_max;
+    int64_t best_cost = 0;  // cost of `best_g` images' worth of work, cross-multiplied
+    int best_g = 0;
+    for (int g = g_max; g >= 1; --g) {
+      const int patch = (g * (H + 2) * hp.PC * Ci + 1023) / 1024 * 1024;
+      if (patch + kRing1 > kLdsLimit) continue;
+      const int64_t cost = rounds2(g * H * W);  // per g images
+      if (!best_g || cost * best_g < best_cost * g) { best_g = g; best_cost = cost; lds = patch; }
+    }
+    if (!best_g) return -1;
+    best = best_g * H;
+    hp.image_mode = 1;
+    hp.PR = best_g * (H + 2);
+    hp.bands = 1;
+    tiles_m = ((int64_t)N + best_g - 1) / best_g;
+  } else {
+    // candidates: the balanced band heights ceil(H / bands), so that no tile is longer than it has to be
+    int tr_max = H;
+    if (const char *t = tuning_env("CATCHQ_HALO_TR")) tr_max = atoi(t) < tr_max ? atoi(t) : tr_max;
+    int64_t best_cost = 0;
+    for (int bands = 1; bands <= H; ++bands) {
+      const int tr = (H + bands - 1) / bands;
+      if (tr > tr_max || tr * W > kMaxP || (H + tr - 1) / tr != bands) continue;
+      const int patch = ((tr + 2) * hp.PC * Ci + 1023) / 1024 * 1024;
+      if (patch + kRing1 > kLdsLimit) continue;
+      const int64_t cost = (int64_t)bands * rounds2(tr * W);
+      if (!best || cost < best_cost) { best = tr; best_cost = cost; lds = patch; hp.bands = bands; }
+    }
+    if (!best) return -1;
+    hp.image_mode = 0;
+    hp.PR = best + 2;
+    tiles_m = (int64_t)N * hp.bands;
+  }
+  hp.TR = best;
+  hp.P = best * W;
+  hp.nsub = (hp.P + 31) / 32;
+  if (hp.nsub > 8) return -1;
+  // a tile that leaves half of the block's waves without a sub-tile is the implicit-GEMM kernel's case
+  if (hp.nsub < 3) return -1;
+  // 64 channels per block while that still gives every compute unit a block and the ring fits
+  int64_t min_blocks = 256;
+  if (const char *t = tuning_env("CATCHQ_HALO_MINBLK")) min_blocks = atoi(t);
+  if (lds + 3 * 64 * 256 > kLdsLimit || tiles_m * ((Co + 63) / 64) < min_blocks) tn = 1;
+  if (const char *t = tuning_env("CATCHQ_HALO_TN")) tn = atoi(t);
+  if (lds + 3 * 32 * tn * 256 > kLdsLimit) tn = 1;
+  hp.tiles_n = (Co + 32 * tn - 1) / (32 * tn);
+  const int64_t nb = tiles_m * hp.tiles_n;
+  if (nb > 0x7fffffff) return -1;
+  hp.nblocks = (int)nb;
+  int lds_bytes = lds + 3 * 32 * tn * 256;
+  const int epi_bytes = lds + 4 * 32 * (32 * tn + 8) * 4;  // the epilogue's staging area lies where the ring was
+  if (epi_bytes > lds_bytes) lds_bytes = epi_bytes;
+  if (lds_bytes > kLdsLimit) return -1;
+#define CATCHQ_HALO_CASE(C)                                                              \
+  case C:                                                                                \
+    return tn == 2 ? launch_halo<C, 2>(x, w, hp, e, lds_bytes, s) : launch_halo<C, 1>(x, w, hp, e, lds_bytes, s)
+  switch (Ci) {
+    CATCHQ_HALO_CASE(64);
+    CATCHQ_HALO_CASE(128);
+    CATCHQ_HALO_CASE(256);
+    default: CATCHQ_HALO_CASE(512);
+  }
+#undef CATCHQ_HALO_CASE
+}
+
+}  // namespace catchq

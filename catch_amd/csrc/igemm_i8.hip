@@ -295,6 +295,16 @@ static bool dma_enabled() {
   return on;
 }
 
+// CATCHQ_NO_HALO=1 (tuning builds) keeps 3x3 layers on the implicit-GEMM kernel
+static bool halo_enabled() {
+  static const bool on = [] {
+    const char *v = tuning_env("CATCHQ_NO_HALO");
+    return !(v && v[0] == '1');
+  }();
+  return on;
+}
+int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, const EpiDev &e, hipStream_t s);
+
 int gemm_nt_stream_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
 int conv2d_stem_i8(const void *x, const void *w, int N, int H, int W, int Co, int kh, int kw, int sh, int sw, int dh,
                    int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -350,6 +360,11 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
   if (dma_enabled() && kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
     // a pointwise convolution is a plain GEMM over the pixels
     const int st = gemm_nt_stream_i8(x, w, p.M, Co, Ci, e, s);
+    if (st >= 0) return st;
+  }
+  if (dma_enabled() && halo_enabled() && kh == 3 && kw == 3 && sh == 1 && sw == 1 && ph == 1 && pw == 1 && dh == 1 && dw == 1) {
+    // the input patch of a band of output rows stays in LDS for all nine taps
+    const int st = conv2d_halo_i8(x, w, N, H, W, Ci, Co, e, s);
     if (st >= 0) return st;
   }
   p.img_stride = (unsigned)(H * W * Ci); p.row_stride = (unsigned)(W * Ci); p.pix_stride = (unsigned)Ci;
