@@ -1,4 +1,4 @@
-// 3x3 int8 convolution (stride 1, padding 1) with the input patch resident in LDS.
+// 3x3 int8 convolution (stride 1 or 2, padding 1) with the input patch resident in LDS.
 //
 // The implicit-GEMM kernel fetches every input pixel nine times (once per filter tap) and synchronises
 // its block once per 64 bytes of K, which leaves a 3x3 layer bound by the load path when the image is
@@ -26,12 +26,14 @@
 namespace catchq {
 
 struct HaloParams {
-  int N, H, W, Co;       // input [N, H, W, CI]; output [N, H, W, Co]
+  int N, H, W, Co;       // output [N, H, W, Co]
+  int Hi, Wi;            // input [N, Hi, Wi, CI]
   int TR;                // output rows per tile
   int image_mode;        // 0: a band of TR rows of one image (the last band of an image may be shorter);
                          // 1: TR = G * H, G whole images
   int bands;             // bands per image (band mode)
-  int PR, PC;            // patch rows / columns (PC = W + 2)
+  int PR, PC;            // patch rows / columns (stride 1: PC = W + 2)
+  int img_rows;          // patch rows per image in image mode
   int P;                 // output pixels per tile = TR * W
   int nsub;              // 32-row sub-tiles per tile
   int tiles_n, nblocks;
@@ -49,15 +51,17 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-// swizzle of a pixel's 16-byte chunk index; CH = chunks per pixel
-template <int CH>
+// swizzle of a pixel's 16-byte chunk index; CH = chunks per pixel.  The lanes of a fragment read pixels S apart:
+// the bits of the pixel index that differ between neighbouring lanes select the chunk
+template <int CH, int S>
 __device__ __forceinline__ unsigned halo_swz(unsigned pix) {
-  if constexpr (CH == 4) return (pix >> 2) & 3u;
-  else if constexpr (CH == 8) return (pix >> 1) & 7u;
-  else return pix & 15u;
+  constexpr int SH = S == 2 ? 1 : 0;
+  if constexpr (CH == 4) return (pix >> (2 + SH)) & 3u;
+  else if constexpr (CH == 8) return (pix >> (1 + SH)) & 7u;
+  else return (pix >> SH) & 15u;
 }
 
-template <int CI, int TN, int TMW, int EPI>
+template <int CI, int TN, int TMW, int S, int EPI>
 __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
                                                           HaloParams hp, EpiDev e) {
   resolve_exp2(e);
@@ -116,15 +120,15 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
     for (int i = wave; i < ninstr; i += 4) {
       int img = img0, hi;
       if (hp.image_mode) {
-        const unsigned g = pr / (unsigned)(hp.H + 2);
+        const unsigned g = pr / (unsigned)hp.img_rows;
         img += (int)g;
-        hi = (int)(pr - g * (unsigned)(hp.H + 2)) - 1;
+        hi = (int)(pr - g * (unsigned)hp.img_rows) - 1;
       } else {
-        hi = ho0 - 1 + (int)pr;
+        hi = ho0 * S - 1 + (int)pr;
       }
       const int wi = (int)pc - 1;
-      const bool ok = (int)pix < npix && img < hp.N && (unsigned)hi < (unsigned)hp.H && (unsigned)wi < (unsigned)hp.W;
-      const unsigned src = (unsigned)((img * hp.H + hi) * hp.W + wi) * (unsigned)CI + ((phys ^ halo_swz<CH>(pix)) << 4);
+      const bool ok = (int)pix < npix && img < hp.N && (unsigned)hi < (unsigned)hp.Hi && (unsigned)wi < (unsigned)hp.Wi;
+      const unsigned src = (unsigned)((img * hp.Hi + hi) * hp.Wi + wi) * (unsigned)CI + ((phys ^ halo_swz<CH, S>(pix)) << 4);
       const unsigned voff = select_u32(ok, src, OOB);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(lds_dyn + i * 1024), 16, (int)voff, 0, 0, 0);
       pix += PPI * 4;
@@ -170,13 +174,15 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
     unsigned prow = tr;
     if (hp.image_mode) {
       const unsigned g = tr / (unsigned)hp.H;
-      prow = g * (unsigned)(hp.H + 2) + (tr - g * (unsigned)hp.H);
+      prow = g * (unsigned)hp.img_rows + (tr - g * (unsigned)hp.H) * S;
+    } else {
+      prow *= S;
     }
-    const unsigned pixbase = prow * (unsigned)hp.PC + wo;
+    const unsigned pixbase = prow * (unsigned)hp.PC + wo * S;
 #pragma unroll
     for (int t = 0; t < 9; ++t) {
       const unsigned pix = pixbase + (unsigned)(t / 3) * (unsigned)hp.PC + (unsigned)(t % 3);
-      a0[i][t] = lds_base + pix * (unsigned)CI + ((((unsigned)fhalf) ^ halo_swz<CH>(pix)) << 4);
+      a0[i][t] = lds_base + pix * (unsigned)CI + ((((unsigned)fhalf) ^ halo_swz<CH, S>(pix)) << 4);
     }
   }
   // weights: row frow of a 32-row block, chunk (2c + fhalf) ^ (frow & 15) of the stage's 16
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
   IgemmParams p = {};
   p.N = hp.Co;
   p.M = (m0 + p_tile < hp.M) ? m0 + p_tile : hp.M;  // rows past the tile belong to the next one
-  constexpr int EPI_STRIDE = BN + 8;
+  constexpr int EPI_STRIDE = 32 * TN + 8;
   int *stage_w = reinterpret_cast<int *>(ring) + wave * 32 * EPI_STRIDE;
 #pragma unroll
   for (int i = 0; i < TMW; ++i) {
@@ -255,9 +261,9 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
   }
 }
 
-template <int CI, int TN, int TMW, int EPI>
+template <int CI, int TN, int TMW, int S, int EPI>
 static int launch_halo_epi(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
-  auto kern = conv3x3_halo_kernel<CI, TN, TMW, EPI>;
+  auto kern = conv3x3_halo_kernel<CI, TN, TMW, S, EPI>;
   if (lds_bytes > 64 * 1024) {
     static std::atomic<bool> raised[64];
     if (raise_lds_limit((const void *)kern, 160 * 1024, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
@@ -266,32 +272,38 @@ static int launch_halo_epi(const void *x, const void *w, const HaloParams &hp, c
   return launch_status();
 }
 
-template <int CI, int TN, int TMW>
+template <int CI, int TN, int TMW, int S>
 static int launch_halo_tm(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
   switch (pick_epilogue(hp.Co, e)) {
     case EPI_SCALAR: return -1;
-    case EPI_Q8_RELU: return launch_halo_epi<CI, TN, TMW, EPI_Q8_RELU>(x, w, hp, e, lds_bytes, s);
-    default: return launch_halo_epi<CI, TN, TMW, EPI_VECTOR>(x, w, hp, e, lds_bytes, s);
+    case EPI_Q8_RELU: return launch_halo_epi<CI, TN, TMW, S, EPI_Q8_RELU>(x, w, hp, e, lds_bytes, s);
+    default: return launch_halo_epi<CI, TN, TMW, S, EPI_VECTOR>(x, w, hp, e, lds_bytes, s);
   }
 }
 
-template <int CI, int TN>
-static int launch_halo(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
+template <int CI, int S>
+static int launch_halo(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int tn, int lds_bytes, hipStream_t s) {
   // four or fewer sub-tiles: one per wave, no second set of accumulators
-  if (hp.nsub <= 4) return launch_halo_tm<CI, TN, 1>(x, w, hp, e, lds_bytes, s);
-  return launch_halo_tm<CI, TN, 2>(x, w, hp, e, lds_bytes, s);
+  if (hp.nsub <= 4)
+    return tn == 2 ? launch_halo_tm<CI, 2, 1, S>(x, w, hp, e, lds_bytes, s) : launch_halo_tm<CI, 1, 1, S>(x, w, hp, e, lds_bytes, s);
+  return tn == 2 ? launch_halo_tm<CI, 2, 2, S>(x, w, hp, e, lds_bytes, s) : launch_halo_tm<CI, 1, 2, S>(x, w, hp, e, lds_bytes, s);
 }
 
-// 3x3, stride 1, padding 1, no dilation, Ci in {64, 128, 256, 512}; -1: not this kernel's shape
-int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, const EpiDev &e, hipStream_t s) {
+// 3x3, stride 1 or 2 (both directions alike), padding 1, no dilation, Ci in {64, 128, 256, 512} (stride 2: not 64);
+// input [N, Hi, Wi, Ci]; -1: not this kernel's shape
+int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, int Co, int stride, const EpiDev &e,
+                   hipStream_t s) {
   if (Ci != 64 && Ci != 128 && Ci != 256 && Ci != 512) return -1;
-  if (Co % 4 != 0 || W > 254 || (int64_t)N * H * W * Ci >= (1ll << 31) || (int64_t)Co * 9 * Ci >= (1ll << 31)) return -1;
-  if ((int64_t)N * H >= (1 << 24)) return -1;
+  if (stride != 1 && !(stride == 2 && Ci != 64)) return -1;
+  const int H = (Hi - 1) / stride + 1, W = (Wi - 1) / stride + 1;
+  if (Co % 4 != 0 || Wi > 254 || (int64_t)N * Hi * Wi * Ci >= (1ll << 31) || (int64_t)Co * 9 * Ci >= (1ll << 31)) return -1;
+  if ((int64_t)N * Hi >= (1 << 24)) return -1;
   HaloParams hp = {};
-  hp.N = N; hp.H = H; hp.W = W; hp.Co = Co;
-  hp.PC = W + 2;
+  hp.N = N; hp.H = H; hp.W = W; hp.Co = Co; hp.Hi = Hi; hp.Wi = Wi;
+  hp.PC = (W - 1) * stride + 3;
+  hp.img_rows = (H - 1) * stride + 3;
   hp.M = (int64_t)N * H * W;
-  hp.x_bytes = (unsigned)((int64_t)N * H * W * Ci);
+  hp.x_bytes = (unsigned)((int64_t)N * Hi * Wi * Ci);
   hp.w_bytes = (unsigned)((int64_t)Co * 9 * Ci);
   constexpr int kLdsLimit = 160 * 1024, kMaxP = 256, kRing1 = 3 * 32 * 256;
   // Tile choice.  A tile of P pixels costs ceil(ceil(P / 32) / 4) rounds of MFMA work (four waves, one 32-row
@@ -307,7 +319,7 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     int64_t best_cost = 0;  // cost of `best_g` images' worth of work, cross-multiplied
     int best_g = 0;
     for (int g = g_max; g >= 1; --g) {
-      const int patch = (g * (H + 2) * hp.PC * Ci + 1023) / 1024 * 1024;
+      const int patch = (g * hp.img_rows * hp.PC * Ci + 1023) / 1024 * 1024;
       if (patch + kRing1 > kLdsLimit) continue;
       const int64_t cost = rounds2(g * H * W);  // per g images
       if (!best_g || cost * best_g < best_cost * g) { best_g = g; best_cost = cost; lds = patch; }
@@ -315,7 +327,7 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     if (!best_g) return -1;
     best = best_g * H;
     hp.image_mode = 1;
-    hp.PR = best_g * (H + 2);
+    hp.PR = best_g * hp.img_rows;
     hp.bands = 1;
     tiles_m = ((int64_t)N + best_g - 1) / best_g;
   } else {
@@ -326,21 +338,21 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     for (int bands = 1; bands <= H; ++bands) {
       const int tr = (H + bands - 1) / bands;
       if (tr > tr_max || tr * W > kMaxP || (H + tr - 1) / tr != bands) continue;
-      const int patch = ((tr + 2) * hp.PC * Ci + 1023) / 1024 * 1024;
+      const int patch = (((tr - 1) * stride + 3) * hp.PC * Ci + 1023) / 1024 * 1024;
       if (patch + kRing1 > kLdsLimit) continue;
       const int64_t cost = (int64_t)bands * rounds2(tr * W);
       if (!best || cost < best_cost) { best = tr; best_cost = cost; lds = patch; hp.bands = bands; }
     }
     if (!best) return -1;
     hp.image_mode = 0;
-    hp.PR = best + 2;
+    hp.PR = (best - 1) * stride + 3;
     tiles_m = (int64_t)N * hp.bands;
   }
   hp.TR = best;
   hp.P = best * W;
   hp.nsub = (hp.P + 31) / 32;
   if (hp.nsub > 8) return -1;
-  // a tile that leaves half of the block's waves without a sub-tile is the implicit-GEMM kernel's case
+  // tiles that leave waves of the block without a sub-tile are the implicit-GEMM kernel's case
   if (hp.nsub < 3) return -1;
   // 64 channels per block while that still gives every compute unit a block and the ring fits
   int64_t min_blocks = 256;
@@ -351,21 +363,27 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
   hp.tiles_n = (Co + 32 * tn - 1) / (32 * tn);
   const int64_t nb = tiles_m * hp.tiles_n;
   if (nb > 0x7fffffff) return -1;
+  // a stride-2 patch is four times its output and leaves room for one block per compute unit: past one round
+  // of blocks the implicit-GEMM kernel is faster (measured on the ResNet-50 downsampling layers at 32 and 64 images)
+  if (stride == 2 && nb > 256) return -1;
   hp.nblocks = (int)nb;
   int lds_bytes = lds + 3 * 32 * tn * 256;
   const int epi_bytes = lds + 4 * 32 * (32 * tn + 8) * 4;  // the epilogue's staging area lies where the ring was
   if (epi_bytes > lds_bytes) lds_bytes = epi_bytes;
   if (lds_bytes > kLdsLimit) return -1;
-#define CATCHQ_HALO_CASE(C)                                                              \
-  case C:                                                                                \
-    return tn == 2 ? launch_halo<C, 2>(x, w, hp, e, lds_bytes, s) : launch_halo<C, 1>(x, w, hp, e, lds_bytes, s)
-  switch (Ci) {
-    CATCHQ_HALO_CASE(64);
-    CATCHQ_HALO_CASE(128);
-    CATCHQ_HALO_CASE(256);
-    default: CATCHQ_HALO_CASE(512);
+  if (stride == 2) {
+    switch (Ci) {
+      case 128: return launch_halo<128, 2>(x, w, hp, e, tn, lds_bytes, s);
+      case 256: return launch_halo<256, 2>(x, w, hp, e, tn, lds_bytes, s);
+      default: return launch_halo<512, 2>(x, w, hp, e, tn, lds_bytes, s);
+    }
   }
-#undef CATCHQ_HALO_CASE
+  switch (Ci) {
+    case 64: return launch_halo<64, 1>(x, w, hp, e, tn, lds_bytes, s);
+    case 128: return launch_halo<128, 1>(x, w, hp, e, tn, lds_bytes, s);
+    case 256: return launch_halo<256, 1>(x, w, hp, e, tn, lds_bytes, s);
+    default: return launch_halo<512, 1>(x, w, hp, e, tn, lds_bytes, s);
+  }
 }
 
 }  // namespace catchq

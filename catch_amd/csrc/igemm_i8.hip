@@ -303,7 +303,8 @@ static bool halo_enabled() {
   }();
   return on;
 }
-int conv2d_halo_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, const EpiDev &e, hipStream_t s);
+int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, int Co, int stride, const EpiDev &e,
+                   hipStream_t s);
 
 int gemm_nt_stream_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
 int conv2d_stem_i8(const void *x, const void *w, int N, int H, int W, int Co, int kh, int kw, int sh, int sw, int dh,
@@ -362,9 +363,9 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
     const int st = gemm_nt_stream_i8(x, w, p.M, Co, Ci, e, s);
     if (st >= 0) return st;
   }
-  if (dma_enabled() && halo_enabled() && kh == 3 && kw == 3 && sh == 1 && sw == 1 && ph == 1 && pw == 1 && dh == 1 && dw == 1) {
+  if (dma_enabled() && halo_enabled() && kh == 3 && kw == 3 && sh == sw && ph == 1 && pw == 1 && dh == 1 && dw == 1) {
     // the input patch of a band of output rows stays in LDS for all nine taps
-    const int st = conv2d_halo_i8(x, w, N, H, W, Ci, Co, e, s);
+    const int st = conv2d_halo_i8(x, w, N, H, W, Ci, Co, sh, e, s);
     if (st >= 0) return st;
   }
   p.img_stride = (unsigned)(H * W * Ci); p.row_stride = (unsigned)(W * Ci); p.pix_stride = (unsigned)Ci;

@@ -469,41 +469,48 @@ def test_conv_wide(bits, case):
     assert same_bits(orc.epilogue(acc, -22, None, bias), out["y"].cpu().numpy())
 
 
-@pytest.mark.parametrize("n,h,w,ci,co", [
-    (2, 56, 56, 64, 64),      # bands of 4 rows of one image, 7 sub-tiles
-    (2, 28, 28, 128, 128),    # bands of 7 rows
-    (3, 14, 14, 256, 256),    # one whole image per tile
-    (5, 7, 7, 512, 512),      # two whole images per tile, odd batch: the last tile is half empty
-    (7, 7, 7, 64, 32),        # five images per tile, one 32-channel block
-    (1, 10, 12, 64, 100),     # ragged channel block (100 = 3 * 32 + 4); room for two images, one present
-    (2, 9, 31, 128, 68),      # odd width: a row is not a multiple of 32 pixels; bands of 3 rows
-    (1, 33, 17, 64, 64),      # bands of 11 rows, 187 pixels
-    (2, 4, 4, 256, 64),       # tiny images: 15 per tile
-    (1, 1, 1, 64, 64),        # a single pixel
-    (1, 60, 120, 64, 64),     # a band is two rows of 120 pixels
-    (1, 6, 254, 64, 32),      # the widest row this route takes: one row per tile
-    (1, 26, 26, 512, 64),     # the patch of a deep layer limits the band: 7, 7, 7 and 5 rows
-    (1, 52, 52, 256, 32),     # 13 bands of 4 rows
-    (2, 13, 40, 64, 32),      # bands of 5, 5 and 3 rows
+@pytest.mark.parametrize("n,h,w,ci,co,stride", [
+    (2, 56, 56, 64, 64, 1),      # bands of 4 rows of one image, 7 sub-tiles
+    (2, 28, 28, 128, 128, 1),    # bands of 7 rows
+    (3, 14, 14, 256, 256, 1),    # one whole image per tile
+    (5, 7, 7, 512, 512, 1),      # two whole images per tile, odd batch: the last tile is half empty
+    (7, 7, 7, 64, 32, 1),        # five images per tile, one 32-channel block
+    (1, 10, 12, 64, 100, 1),     # ragged channel block (100 = 3 * 32 + 4); room for two images, one present
+    (2, 9, 31, 128, 68, 1),      # odd width: a row is not a multiple of 32 pixels; bands of 3 rows
+    (1, 33, 17, 64, 64, 1),      # bands of 11 rows, 187 pixels
+    (2, 4, 4, 256, 64, 1),       # tiny images: 15 per tile
+    (1, 1, 1, 64, 64, 1),        # a single pixel
+    (1, 60, 120, 64, 64, 1),     # a band is two rows of 120 pixels
+    (1, 6, 254, 64, 32, 1),      # the widest row this route takes: one row per tile
+    (1, 26, 26, 512, 64, 1),     # the patch of a deep layer limits the band: 7, 7, 7 and 5 rows
+    (1, 52, 52, 256, 32, 1),     # 13 bands of 4 rows
+    (2, 13, 40, 64, 32, 1),      # bands of 5, 5 and 3 rows
+    (2, 56, 56, 128, 128, 2),    # stride 2: 28 x 28 outputs, bands of 7 rows over 15 input rows
+    (3, 28, 28, 256, 256, 2),    # 14 x 14 outputs in two bands
+    (3, 14, 14, 512, 512, 2),    # 7 x 7 outputs: one image per tile, two sub-tiles
+    (2, 15, 13, 128, 36, 2),     # odd input sides: 8 x 7 outputs, the last input row and column are used
+    (5, 6, 6, 256, 32, 2),       # 3 x 3 outputs, several images per tile
+    (1, 30, 50, 128, 64, 2),     # 15 x 25 outputs: bands of 8 and 7 rows
 ])
-def test_conv3x3_patch_resident(n, h, w, ci, co):
-    """3x3 / stride 1 / padding 1 layers whose input patch stays in LDS for all nine taps: int32 sums and the
+def test_conv3x3_patch_resident(n, h, w, ci, co, stride):
+    """3x3 / padding 1 layers (stride 1 or 2) whose input patch stays in LDS for all nine taps: int32 sums and the
     generic epilogue against the oracle, then the ReLU -> int8 instance the classifier layers use"""
-    note("conv3x3 patch-resident", n, h, w, ci, co)
-    r = rng(n * 1000 + h * 10 + ci + co)
+    note("conv3x3 patch-resident", n, h, w, ci, co, stride)
+    r = rng(n * 1000 + h * 10 + ci + co + stride)
     x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, 3, 3, ci), 8)
     x[0, 0, 0, :] = -128          # corners and edges carry the extremes: the padding must contribute nothing
     x[-1, -1, -1, :] = 127
     wt[0] = -128
-    acc, ovf = orc.conv2d_nhwc(x, wt, (1, 1), (1, 1), (1, 1), 1)
+    st = (stride, stride)
+    acc, ovf = orc.conv2d_nhwc(x, wt, (1, 1), st, (1, 1), 1)
     assert ovf == 0
     bias = r.standard_normal(co).astype(np.float32)
     div = r.uniform(0.5, 2.0, co).astype(np.float32)
-    out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), (1, 1), (1, 1), exp2=-14, chan_div=cabi.dev(div), bias=cabi.dev(bias))
+    out = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), (1, 1), st, exp2=-14, chan_div=cabi.dev(div), bias=cabi.dev(bias))
     assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
     assert same_bits(orc.epilogue(acc, -14, div, bias), out["y"].cpu().numpy())
     rcp = (np.float32(1.0) / div).astype(np.float32)
-    q = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), (1, 1), (1, 1), exp2=-14, chan_div=cabi.dev(div), chan_rcp=cabi.dev(rcp),
+    q = cabi.conv2d_nhwc(cabi.dev(x), cabi.dev(wt), (1, 1), st, exp2=-14, chan_div=cabi.dev(div), chan_rcp=cabi.dev(rcp),
                          bias=cabi.dev(bias), act=1, y_dtype=None, want_acc=False, q_bw=8, q_pos=-3)["q"]
     want = orc.quantize(orc.epilogue(acc, -14, div, bias, None, 1), 8, -3)
     assert same_bits(want, q.cpu().numpy())
