@@ -10,9 +10,9 @@
 // K for the block's output channels through a three-slot LDS ring, one barrier per stage, so a wave
 // issues 16 to 32 MFMAs per synchronisation instead of two.
 //
-//   patch        PR x PC pixels of CI bytes; the 16-byte chunks of a pixel are XOR-swizzled with low
-//                bits of the pixel index (on the source side of the LDS-DMA) so that the ds_read_b128
-//                of 32 consecutive pixels at one logical chunk spread over all banks
+//   patch        PR x PC pixels of CI bytes; the 16-byte chunks of a pixel are XOR-swizzled (on the source
+//                side of the LDS-DMA) with a key that counts output pixels, so that the ds_read_b128 of
+//                32 consecutive output pixels at one tap and one logical chunk spread over all banks
 //   output tile  P = TR * Wo consecutive output pixels (rows m0 .. m0 + P of the GEMM view), split
 //                into 32-row MFMA sub-tiles; wave w owns sub-tiles w and w + 4; BN = 32 * TN channels
 //   K order      (tap, channel), as the weight tensor [Co][3][3][Ci] stores it; a stage may end past
@@ -51,14 +51,21 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-// swizzle of a pixel's 16-byte chunk index; CH = chunks per pixel.  The lanes of a fragment read pixels S apart:
-// the bits of the pixel index that differ between neighbouring lanes select the chunk
-template <int CH, int S>
-__device__ __forceinline__ unsigned halo_swz(unsigned pix) {
+// Swizzle of a pixel's 16-byte chunk index; CH = chunks per pixel.  The 32 lanes of an A fragment read the patch
+// pixels of 32 consecutive OUTPUT pixels at one filter tap, and a ds_read_b128 is conflict-free when 16
+// consecutive lanes fall into 16 different 16-byte slots of a 256-byte LDS line.  The key is therefore taken from
+// h = (patch row / S) * Wo + (patch column / S): for a fixed tap h runs through consecutive integers with the
+// output pixel index, across the ends of output rows as well (the patch pixel index itself jumps there).
+template <int CH>
+__device__ __forceinline__ unsigned halo_swz(unsigned h) {
+  if constexpr (CH == 4) return (h >> 2) & 3u;
+  else if constexpr (CH == 8) return (h >> 1) & 7u;
+  else return h & 15u;
+}
+template <int S>
+__device__ __forceinline__ unsigned halo_key(unsigned prow, unsigned pcol, unsigned wo_count) {
   constexpr int SH = S == 2 ? 1 : 0;
-  if constexpr (CH == 4) return (pix >> (2 + SH)) & 3u;
-  else if constexpr (CH == 8) return (pix >> (1 + SH)) & 7u;
-  else return (pix >> SH) & 15u;
+  return (prow >> SH) * wo_count + (pcol >> SH);
 }
 
 template <int CI, int TN, int TMW, int S, int EPI>
@@ -128,7 +135,7 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
       }
       const int wi = (int)pc - 1;
       const bool ok = (int)pix < npix && img < hp.N && (unsigned)hi < (unsigned)hp.Hi && (unsigned)wi < (unsigned)hp.Wi;
-      const unsigned src = (unsigned)((img * hp.Hi + hi) * hp.Wi + wi) * (unsigned)CI + ((phys ^ halo_swz<CH, S>(pix)) << 4);
+      const unsigned src = (unsigned)((img * hp.Hi + hi) * hp.Wi + wi) * (unsigned)CI + ((phys ^ halo_swz<CH>(halo_key<S>(pr, pc, (unsigned)hp.W))) << 4);
       const unsigned voff = select_u32(ok, src, OOB);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(lds_dyn + i * 1024), 16, (int)voff, 0, 0, 0);
       pix += PPI * 4;
@@ -178,11 +185,12 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
     } else {
       prow *= S;
     }
-    const unsigned pixbase = prow * (unsigned)hp.PC + wo * S;
+    const unsigned pcol = wo * S;
 #pragma unroll
     for (int t = 0; t < 9; ++t) {
-      const unsigned pix = pixbase + (unsigned)(t / 3) * (unsigned)hp.PC + (unsigned)(t % 3);
-      a0[i][t] = lds_base + pix * (unsigned)CI + ((((unsigned)fhalf) ^ halo_swz<CH, S>(pix)) << 4);
+      const unsigned pr_t = prow + (unsigned)(t / 3), pc_t = pcol + (unsigned)(t % 3);
+      const unsigned pix = pr_t * (unsigned)hp.PC + pc_t;
+      a0[i][t] = lds_base + pix * (unsigned)CI + ((((unsigned)fhalf) ^ halo_swz<CH>(halo_key<S>(pr_t, pc_t, (unsigned)hp.W))) << 4);
     }
   }
   // weights: row frow of a 32-row block, chunk (2c + fhalf) ^ (frow & 15) of the stage's 16
