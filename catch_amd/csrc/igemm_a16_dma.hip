@@ -166,8 +166,8 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
   const unsigned b_k0 = (unsigned)((fhalf ^ swb) * 16), b_k1 = (unsigned)(((fhalf ^ swb) ^ 2) * 16);
   const unsigned b_row = lds_base + (unsigned)(A_STAGE + (wave_n * WN + frow) * BK);
 
-  auto half_step = [&](unsigned a_base, unsigned a_chunk, unsigned b_addr) {
-    v4i fa[TM][2], fb[TN];
+  // one half of a K step (32 int16 activations x 32 int8 weights per tile): fetch, then multiply
+  auto fetch_half = [&](v4i (&fa)[TM][2], v4i (&fb)[TN], unsigned a_base, unsigned a_chunk, unsigned b_addr) {
     const unsigned a_first = a_base + a_chunk, a_second = a_base + (a_chunk ^ 16u);
     // tile i of this wave sits 32 rows further: 4096 bytes for A, 2048 for B
     fa[0][0] = ds_read_b128<0>(a_first);
@@ -178,10 +178,8 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
     }
     fb[0] = ds_read_b128<0>(b_addr);
     if constexpr (TN > 1) fb[1] = ds_read_b128<2048>(b_addr);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) { lgkm_wait<0>(fa[i][0]); lgkm_wait<0>(fa[i][1]); }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) lgkm_wait<0>(fb[j]);
+  };
+  auto multiply_half = [&](v4i (&fa)[TM][2], v4i (&fb)[TN]) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -199,9 +197,22 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(co
   };
   static_assert(TM <= 2 && TN <= 2, "wave tile larger than 64x64");
 
+  // both halves are requested up front: the second half's fragments arrive while the first half is multiplied
   auto compute = [&](unsigned stage_off) {
-    half_step(a_row + stage_off, a_c0, b_row + stage_off + b_k0);
-    half_step(a_row + stage_off, a_c0 ^ 64u, b_row + stage_off + b_k1);
+    constexpr int NF = 2 * TM + TN;  // LDS reads per half
+    v4i fa0[TM][2], fb0[TN], fa1[TM][2], fb1[TN];
+    fetch_half(fa0, fb0, a_row + stage_off, a_c0, b_row + stage_off + b_k0);
+    fetch_half(fa1, fb1, a_row + stage_off, a_c0 ^ 64u, b_row + stage_off + b_k1);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) { lgkm_wait<NF>(fa0[i][0]); lgkm_wait<NF>(fa0[i][1]); }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) lgkm_wait<NF>(fb0[j]);
+    multiply_half(fa0, fb0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) { lgkm_wait<0>(fa1[i][0]); lgkm_wait<0>(fa1[i][1]); }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) lgkm_wait<0>(fb1[j]);
+    multiply_half(fa1, fb1);
   };
 
   // ---- pipeline (same schedule as the int8 kernel) ---------------------------------------------------
