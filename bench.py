@@ -43,6 +43,8 @@ def parse():
                     help="quantize with position and fractional scale (steps of absmax/qmax) instead of power-of-two steps")
     ap.add_argument("--streams", type=int, default=2,
                     help="parts the batch is split into inside the HIP graph, each on a stream of its own (1: one launch sequence)")
+    ap.add_argument("--chain-links", type=int, default=-1,
+                    help="longest residual chain recomputed inside a block's last launch (0: none, -1: the plan's own rule)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -91,8 +93,23 @@ def layer_profile(fused, x, iters=20, only=None):
         want_y = fused.f_demand[l.name] or qd is None
         y_half = fused.out_half and l.name in fused.outputs
         ds = fused.shortcut_of.get(l.name) if l.kind == "conv" else None
+        chain = fused.chain_of.get(l.name) if l.kind == "conv" else None
         extra_macs = extra_bytes = 0
-        if ds is not None:  # the block's projection shortcut runs inside this launch
+        if chain is not None:  # the residual chain back to the stage's shortcut is recomputed inside this launch
+            resid = None
+            n_pix = trace[l.name]["y"].numel() // trace[l.name]["y"].shape[-1]
+            cq = [fused.q[c.name] for c in chain]
+            xs = [trace[c.name]["qx"] for c in chain]
+            for c, k, sx in zip(chain[:-1], cq[:-1], xs[:-1]):
+                extra_macs += trace[l.name]["y"].numel() * k.qw.shape[-1]
+                extra_bytes += n_pix * sx.shape[-1] * sx.element_size() + k.qw.numel() * k.qw.element_size()
+
+            def run(chain=chain, cq=cq, xs=xs, qd=qd, want_y=want_y):
+                return ops.qconv2d_chain(xs, [k.qw for k in cq], [c.stride for c in chain], [k.exp2 for k in cq],
+                                         [k.chan_div for k in cq], [k.bias for k in cq], want_y, 8 if qd else 0,
+                                         qd[1] if qd else 0)
+            route = "mfma+chain%d" % len(chain)
+        elif ds is not None:  # the block's projection shortcut runs inside this launch
             dq = fused.q[ds.name]
             sx = trace[ds.name]["qx"]
             resid = None
@@ -160,9 +177,20 @@ def plan_launches(fused, n, h, w):
             macs = n_out * (lq.qw.numel() // lq.qw.shape[0])
             b = n * ih * iw * fused.cdev[l.src] * lq.bw_x // 8 + lq.qw.numel() * lq.qw.element_size()
             ds = fused.shortcut_of.get(l.name)
-            if ds is not None:
+            chain = fused.chain_of.get(l.name)
+            k_extra = 0
+            if chain is not None:
+                # every earlier link of the residual chain is recomputed inside this launch: its int8 input (the
+                # pixels the 1x1 taps touch) and its weights are read, its 2*K operations per output repeated
+                for c in chain[:-1]:
+                    cq = fused.q[c.name]
+                    macs += n_out * cq.qw.shape[-1]
+                    k_extra += cq.qw.shape[-1]
+                    b += n * ho * wo * fused.cdev[c.src] * cq.bw_x // 8 + cq.qw.numel() * cq.qw.element_size()
+            elif ds is not None:
                 dq = fused.q[ds.name]
                 macs += n_out * dq.qw.shape[-1]
+                k_extra = dq.qw.shape[-1]
                 b += n * ho * wo * fused.cdev[ds.src] * dq.bw_x // 8 + dq.qw.numel() * dq.qw.element_size()
             elif l.add:
                 b += 4 * n_out
@@ -171,7 +199,7 @@ def plan_launches(fused, n, h, w):
             y_half = fused.out_half and l.name in fused.outputs
             b += ((2 if y_half else 4) * n_out if want_y else 0) + (n_out * qd[0] // 8 if qd else 0)
             rows.append(dict(name=l.name, kind="conv", ops=2 * macs, bytes=b, m=n * ho * wo, n=fused.cdev[l.name],
-                             k=lq.qw.numel() // lq.qw.shape[0] + (fused.q[ds.name].qw.shape[-1] if ds is not None else 0)))
+                             k=lq.qw.numel() // lq.qw.shape[0] + k_extra))
             for d in fused.q_demand[l.name][1:]:
                 rows.append(dict(name=l.name, kind="quantize", ops=0, bytes=n_out * 4 + n_out * d[0] // 8))
         elif l.kind == "fc":
@@ -302,7 +330,8 @@ def build_workload(args):
         if detector:
             sys.exit("--fractional-scale needs a checkpoint of scales; the detector's holds bit widths and positions")
         what += ", position + fractional scale"
-    fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale)
+    fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale,
+                              chain_links=None if args.chain_links < 0 else args.chain_links)
     if args.streams < 1:
         sys.exit("--streams must be at least 1")
     while batch % args.streams:  # the largest number of equal parts not above what was asked for

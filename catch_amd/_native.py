@@ -39,6 +39,13 @@ class Shortcut(ctypes.Structure):
                 ("bias", ctypes.c_void_p)]
 
 
+class ChainLink(ctypes.Structure):
+    """struct catchq_chain_link"""
+    _fields_ = [("x", ctypes.c_void_p), ("w", ctypes.c_void_p), ("in_h", ctypes.c_int), ("in_w", ctypes.c_int),
+                ("ci", ctypes.c_int), ("stride", ctypes.c_int), ("exp2", ctypes.c_int), ("chan_div", ctypes.c_void_p),
+                ("chan_rcp", ctypes.c_void_p), ("bias", ctypes.c_void_p)]
+
+
 # name -> (restype, argtypes); every symbol include/catchq.h declares
 _I, _I64, _F, _P, _SZ = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 SIGNATURES = {
@@ -69,6 +76,7 @@ SIGNATURES = {
     "catchq_quantize_conv2d_nhwc": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, ctypes.POINTER(ConvDesc), _P, _P, _I, _P, _SZ, _P]),
     "catchq_conv2d_shortcut_workspace_size": (_I, [_I, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Shortcut),
                                                    ctypes.POINTER(_SZ)]),
+    "catchq_conv1x1_chain_nhwc": (_I, [ctypes.POINTER(ChainLink), _I, _I, _I, _I, _I, _P, _P, _I, _P]),
     "catchq_conv2d_shortcut_nhwc": (_I, [_P, _I, _P, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Epilogue),
                                          ctypes.POINTER(Shortcut), _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),

@@ -22,6 +22,16 @@ int conv2d_mfma_a16w16(const void *x, const void *w, int N, int H, int W, int Ci
 int conv2d_dual_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
                    int sh, int sw, int dh, int dw, int Ho, int Wo, const void *xs, const void *ws, int Hs, int Ws, int Cs,
                    int ss, const EpiDev &e, const ShortcutDev &sc, hipStream_t s);
+struct ChainLinkDev {  // igemm_i8_chain.hip
+  const int8_t *x, *w;
+  unsigned x_bytes, w_bytes;
+  int K;
+  unsigned img_stride, row_stride, pix_stride;
+  int exp2;
+  const float *chan_div, *chan_rcp, *bias;
+};
+int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int Wo, int Co, float *y, int8_t *q,
+                     int q_position, hipStream_t s);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -243,6 +253,39 @@ CATCHQ_API int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void
   catchq_epilogue_t em = *epilogue;
   em.resid = (const float *)workspace;
   return catchq_conv2d_nhwc(x, x_bits, w, w_bits, desc, &em, stream);
+}
+
+CATCHQ_API int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int nlinks, int n, int ho, int wo, int co,
+                                         float *y, void *q, int q_position, catchq_stream_t stream) {
+  if (!links || n < 0 || ho <= 0 || wo <= 0 || co <= 0 || (!y && !q)) return CATCHQ_ERR_ARG;
+  if (nlinks < 2 || nlinks > CATCHQ_CHAIN_MAX_LINKS) return CATCHQ_ERR_UNSUPPORTED;
+  if (q && (q_position < -126 || q_position > 126)) return CATCHQ_ERR_ARG;
+  ChainLinkDev dev[CATCHQ_CHAIN_MAX_LINKS];
+  for (int i = 0; i < nlinks; ++i) {
+    const catchq_chain_link_t &l = links[i];
+    if (l.in_h <= 0 || l.in_w <= 0 || l.ci <= 0 || l.stride <= 0) return CATCHQ_ERR_SHAPE;
+    if (catchq_conv_out_size(l.in_h, 1, 0, l.stride, 1) != ho || catchq_conv_out_size(l.in_w, 1, 0, l.stride, 1) != wo)
+      return CATCHQ_ERR_SHAPE;
+    if (n > 0 && (!l.x || !l.w)) return CATCHQ_ERR_ARG;
+    const int64_t xb = (int64_t)n * l.in_h * l.in_w * l.ci, wb = (int64_t)co * l.ci;
+    if (xb >= (1ll << 31) || wb >= (1ll << 31) || l.ci % 64 != 0) return CATCHQ_ERR_UNSUPPORTED;
+    if (!l.chan_div || !l.chan_rcp || !l.bias || l.exp2 < -64 || l.exp2 > 64) return CATCHQ_ERR_UNSUPPORTED;
+    dev[i].x = (const int8_t *)l.x;
+    dev[i].w = (const int8_t *)l.w;
+    dev[i].x_bytes = (unsigned)xb;
+    dev[i].w_bytes = (unsigned)wb;
+    dev[i].K = l.ci;
+    dev[i].img_stride = (unsigned)(l.in_h * l.in_w * l.ci);
+    dev[i].row_stride = (unsigned)(l.stride * l.in_w * l.ci);
+    dev[i].pix_stride = (unsigned)(l.stride * l.ci);
+    dev[i].exp2 = l.exp2;
+    dev[i].chan_div = l.chan_div;
+    dev[i].chan_rcp = l.chan_rcp;
+    dev[i].bias = l.bias;
+  }
+  if (n == 0) return CATCHQ_OK;
+  const int st = conv1x1_chain_i8(dev, nlinks, n, ho, wo, co, y, (int8_t *)q, q_position, as_stream(stream));
+  return st < 0 ? CATCHQ_ERR_UNSUPPORTED : st;
 }
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }

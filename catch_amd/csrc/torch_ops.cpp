@@ -467,6 +467,52 @@ std::tuple<Tensor, Tensor> qconv2d_shortcut_op(const Tensor &qx, const Tensor &q
   return std::make_tuple(o.y, o.q);
 }
 
+// Residual chain (catchq_conv1x1_chain_nhwc): xs[i] [N,Hi,Wi,Ci] int8 NHWC, ws[i] [Co,Ci] or [Co,1,1,Ci] int8;
+// link 0 is the projection shortcut, links 1.. the blocks' last 1x1 convolutions in order.
+std::tuple<Tensor, Tensor> qconv2d_chain_op(at::TensorList xs, at::TensorList ws, at::IntArrayRef strides,
+                                            at::IntArrayRef exp2s, at::TensorList chan_divs, at::TensorList biases,
+                                            bool want_y, int64_t q_bitwidth, int64_t q_position) {
+  const size_t nl = xs.size();
+  TORCH_CHECK(nl >= 2 && nl <= CATCHQ_CHAIN_MAX_LINKS, "qconv2d_chain: 2 .. ", CATCHQ_CHAIN_MAX_LINKS, " links expected");
+  TORCH_CHECK(ws.size() == nl && strides.size() == nl && exp2s.size() == nl && chan_divs.size() == nl && biases.size() == nl,
+              "qconv2d_chain: one entry per link expected in every list");
+  TORCH_CHECK(q_bitwidth == 0 || q_bitwidth == 8, "qconv2d_chain: int8 or no quantized output");
+  TORCH_CHECK(want_y || q_bitwidth == 8, "qconv2d_chain: no output requested");
+  c10::DeviceGuard guard(xs[0].device());
+  const int64_t n = xs[0].size(0), co = ws[0].size(0);
+  int ho = 0, wo = 0;
+  catchq_chain_link_t links[CATCHQ_CHAIN_MAX_LINKS];
+  std::vector<Tensor> keep;
+  for (size_t i = 0; i < nl; ++i) {
+    const Tensor &x = xs[i], &w = ws[i];
+    TORCH_CHECK(x.dim() == 4 && x.is_contiguous() && x.scalar_type() == at::kChar && x.size(0) == n,
+                "qconv2d_chain: int8 NHWC activations of one batch expected");
+    TORCH_CHECK(w.is_contiguous() && w.scalar_type() == at::kChar && w.size(0) == co && w.numel() == co * x.size(3),
+                "qconv2d_chain: int8 [Co,Ci] filters expected");
+    const int h = catchq_conv_out_size((int)x.size(1), 1, 0, (int)strides[i], 1);
+    const int w_ = catchq_conv_out_size((int)x.size(2), 1, 0, (int)strides[i], 1);
+    if (i == 0) { ho = h; wo = w_; }
+    TORCH_CHECK(h == ho && w_ == wo && ho > 0 && wo > 0, "qconv2d_chain: the links' output grids differ");
+    Tensor cd = as_f32_vec(chan_divs[i], co, "chan_div"), bs = as_f32_vec(biases[i], co, "bias");
+    Tensor rcp = reciprocals_for(cd);
+    TORCH_CHECK(rcp.defined(), "qconv2d_chain: a divisor without a usable reciprocal");
+    keep.push_back(cd); keep.push_back(bs); keep.push_back(rcp);
+    links[i].x = x.data_ptr(); links[i].w = w.data_ptr();
+    links[i].in_h = (int)x.size(1); links[i].in_w = (int)x.size(2); links[i].ci = (int)x.size(3);
+    links[i].stride = (int)strides[i];
+    links[i].exp2 = (int)exp2s[i];
+    links[i].chan_div = cd.data_ptr<float>(); links[i].chan_rcp = rcp.data_ptr<float>(); links[i].bias = bs.data_ptr<float>();
+  }
+  Tensor y, q;
+  if (want_y) y = at::empty({n, ho, wo, co}, xs[0].options().dtype(at::kFloat));
+  if (q_bitwidth == 8) q = at::empty({n, ho, wo, co}, xs[0].options().dtype(at::kChar));
+  if (n == 0) return std::make_tuple(y, q);
+  check_status(catchq_conv1x1_chain_nhwc(links, (int)nl, (int)n, ho, wo, (int)co, want_y ? y.data_ptr<float>() : nullptr,
+                                         q.defined() ? q.data_ptr() : nullptr, (int)q_position, current_stream()),
+               "torch_mlu::qconv2d_chain");
+  return std::make_tuple(y, q);
+}
+
 std::tuple<Tensor, Tensor, Tensor> qlinear_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
                                               const c10::optional<Tensor> &chan_div,
                                               const c10::optional<Tensor> &bias, int64_t act, bool want_y,
@@ -982,6 +1028,8 @@ TORCH_LIBRARY(torch_mlu, m) {
         "int s_stride, int s_exp2, Tensor? s_chan_div, Tensor? s_bias, int[] padding, int[] stride, int[] dilation, "
         "int act=0, bool want_y=True, bool y_half=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
         "float act_slope=0.0, bool resid_after_act=False) -> (Tensor, Tensor)");
+  m.def("qconv2d_chain(Tensor[] xs, Tensor[] ws, int[] strides, int[] exp2s, Tensor[] chan_divs, Tensor[] biases, "
+        "bool want_y=False, int q_bitwidth=8, int q_position=0) -> (Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
         "bool want_y=True, bool y_half=False, bool want_acc=False, int q_bitwidth=0, int q_position=0, "
         "float q_scale=1.0) -> (Tensor, Tensor, Tensor)");
@@ -1011,6 +1059,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("quantize_conv2d", &quantize_conv2d_op);
   m.impl("qconv2d", &qconv2d_op);
   m.impl("qconv2d_shortcut", &qconv2d_shortcut_op);
+  m.impl("qconv2d_chain", &qconv2d_chain_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);
   m.impl("global_avgpool_nhwc", &global_avgpool_nhwc_op);

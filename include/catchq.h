@@ -261,6 +261,37 @@ int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void *w, int w_
                                 const catchq_epilogue_t *epilogue, const catchq_shortcut_t *shortcut, void *workspace,
                                 size_t workspace_bytes, catchq_stream_t stream);
 
+/* Residual chain of a stage of bottleneck blocks, recomputed from its int8 inputs in one launch.
+ * In the reference every residual block ends in torch_mlu::conv2d (cnnl_conv2d,
+ * operators/cnnl/quantify_conv_forward.cpp:56-147) followed by a float add (cnnl_add, operators/cnnl/add.cpp)
+ * and ReLU (operators/cnnl/activation.cpp): block b stores y_b = relu(conv_b + y_{b-1}) in fp32 and block
+ * b+1 reads it back.  Here links[0] is the stage's 1x1 projection shortcut and links[1..] are the last 1x1
+ * convolutions of the stage's blocks, in order:
+ *   v_0 = float(acc_0) * 2^exp2_0 / chan_div_0[c] + bias_0[c]
+ *   v_i = relu(float(acc_i) * 2^exp2_i / chan_div_i[c] + bias_i[c] + v_{i-1}),   i = 1 .. nlinks-1
+ * with acc_i the 1x1 convolution of links[i].x [n, in_h, in_w, ci] (int8) with links[i].w [co, ci] (int8),
+ * taps every `stride` pixels, no padding, on the output grid [n, ho, wo].  The launch stores
+ * y = v_last (fp32, may be NULL) and q = sat(rne(v_last * 2^-q_position)) (int8, may be NULL) as NHWC
+ * [n, ho, wo, co].  Every operation is the one catchq_conv2d_nhwc / catchq_conv2d_shortcut_nhwc calls of the
+ * blocks, one after the other, would perform on the same integer sums in the same order, so y and q are
+ * theirs bit for bit; the blocks' fp32 outputs in between are never stored.
+ * Requirements (CATCHQ_ERR_UNSUPPORTED otherwise): 2 <= nlinks <= CATCHQ_CHAIN_MAX_LINKS, ci % 64 == 0,
+ * co % 4 == 0, chan_div / chan_rcp / bias given for every link (chan_rcp as in catchq_epilogue_t),
+ * -64 <= exp2 <= 64, every tensor below 2 GiB and 16-byte aligned. */
+#define CATCHQ_CHAIN_MAX_LINKS 8
+typedef struct catchq_chain_link {
+  const void *x;         /* device int8 [n, in_h, in_w, ci] */
+  const void *w;         /* device int8 [co, ci] */
+  int in_h, in_w, ci;
+  int stride;
+  int exp2;
+  const float *chan_div; /* device [co] */
+  const float *chan_rcp; /* device [co] */
+  const float *bias;     /* device [co] */
+} catchq_chain_link_t;
+int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int nlinks, int n, int ho, int wo, int co,
+                              float *y, void *q, int q_position, catchq_stream_t stream);
+
 /* ------------------------------------------------------------------ neighbours of the convolutions */
 
 /* Max pooling over an NHWC tensor whose elements are int8, int16 (quantized activations) or fp32

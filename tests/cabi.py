@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 from catch_amd import _native
-from catch_amd._native import ConvDesc, Epilogue, Shortcut, check
+from catch_amd._native import ChainLink, ConvDesc, Epilogue, Shortcut, check
 
 F32, F16 = 0, 1
 _INT = {8: torch.int8, 16: torch.int16, 31: torch.int32, 32: torch.int32}
@@ -150,6 +150,27 @@ def conv2d_shortcut_nhwc(x, w, sx, sw, sc_stride, sc_exp2, sc_chan_div=None, sc_
     check(lib().catchq_conv2d_shortcut_nhwc(ptr(x), x.element_size() * 8, ptr(w), w.element_size() * 8, ctypes.byref(d),
                                             ctypes.byref(e), ctypes.byref(sc), ptr(ws), need.value, stream()))
     return out, need.value
+
+
+def conv1x1_chain_nhwc(links, want_y=True, want_q=True, q_pos=0):
+    """links: dicts with x [N,H,W,Ci] int8, w [Co,Ci] int8, stride, exp2, chan_div, chan_rcp, bias (device tensors);
+    links[0] is the projection shortcut.  -> {"y": fp32 or None, "q": int8 or None}"""
+    n, co = links[0]["x"].shape[0], links[0]["w"].shape[0]
+    s0 = links[0]["stride"]
+    ho = lib().catchq_conv_out_size(links[0]["x"].shape[1], 1, 0, s0, 1)
+    wo = lib().catchq_conv_out_size(links[0]["x"].shape[2], 1, 0, s0, 1)
+    arr = (ChainLink * len(links))()
+    for a, l in zip(arr, links):
+        a.x, a.w = l["x"].data_ptr(), l["w"].data_ptr()
+        a.in_h, a.in_w, a.ci = l["x"].shape[1], l["x"].shape[2], l["x"].shape[3]
+        a.stride, a.exp2 = l["stride"], l["exp2"]
+        for k in ("chan_div", "chan_rcp", "bias"):
+            setattr(a, k, None if l.get(k) is None else l[k].data_ptr())
+    dev_ = links[0]["x"].device
+    y = torch.empty((n, ho, wo, co), dtype=torch.float32, device=dev_) if want_y else None
+    q = torch.empty((n, ho, wo, co), dtype=torch.int8, device=dev_) if want_q else None
+    check(lib().catchq_conv1x1_chain_nhwc(arr, len(links), n, ho, wo, co, ptr(y), ptr(q), q_pos, stream()))
+    return {"y": y, "q": q}
 
 
 def quantize_conv2d(x, pos_x, w, pos_w, x_bits=8, w_bits=8, padding=(0, 0), stride=(1, 1), dilation=(1, 1), groups=1,

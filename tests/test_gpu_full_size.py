@@ -57,12 +57,23 @@ def check_plan_rows(fused, x, images, rows_per_layer=3):
             kh = qw.shape[1]
             ho_n = (qx.shape[1] + 2 * pad - kh) // l.stride + 1
             ds = fused.shortcut_of.get(l.name)
+            chain = fused.chain_of.get(l.name)
             for n in images:
                 for ho in sorted(set([0, ho_n // 2, ho_n - 1][:rows_per_layer])):
                     band = _band(qx, n, ho * l.stride - pad, kh)
                     acc, ovf = orc.conv2d_nhwc(band, qw, (0, pad), (l.stride, l.stride), (1, 1), lq.groups)
                     assert ovf == 0 and acc.shape[1] == 1, l.name
-                    if ds is not None:
+                    if chain is not None:
+                        # the residual is the chain of the earlier blocks, shortcut first, evaluated on this row
+                        resid = None
+                        for i, c in enumerate(chain[:-1]):
+                            cq = fused.q[c.name]
+                            cx = keep[(c.src, cq.bw_x, cq.pos_x, cq.scale_x)]
+                            cacc, covf = orc.conv2d_nhwc(_band(cx, n, ho * c.stride, 1), cq.qw.cpu().numpy(), (0, 0),
+                                                         (c.stride, c.stride), (1, 1), 1)
+                            assert covf == 0
+                            resid = orc.epilogue(cacc, cq.exp2, _np(cq.chan_div), _np(cq.bias), resid, 0 if i == 0 else 1)
+                    elif ds is not None:
                         dq = fused.q[ds.name]
                         sx = keep[(ds.src, dq.bw_x, dq.pos_x, dq.scale_x)]
                         sacc, _ = orc.conv2d_nhwc(_band(sx, n, ho * ds.stride, 1), dq.qw.cpu().numpy(), (0, 0),
@@ -145,7 +156,8 @@ def test_resnet50_at_the_benchmark_shapes():
         logits, checked = check_plan_rows(fused, x.cuda(), (0, 17, 31))
     finally:
         lib.catchq_set_launch_sharing(max(before, 1))
-    assert checked > 300 and len(fused.shortcut_of) == 4
+    # the plan the benchmark runs: every stage's first block and the second block of the widest stage are residual chains
+    assert checked > 300 and sorted(len(c) for c in fused.chain_of.values()) == [2, 2, 2, 2, 3] and not fused.shortcut_of
     pick = [0, 31]
     t, _ = netref.run(layers, {k: v.detach().cpu().numpy() for k, v in sd.items()}, x[pick].numpy(), record=False)
     want = t[fused.outputs[0]].reshape(len(pick), -1)

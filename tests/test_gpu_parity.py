@@ -797,6 +797,67 @@ def test_conv_with_projection_shortcut(case):
     assert same_bits(y, out["y"].cpu().numpy())
 
 
+CHAIN_CASES = [
+    # N, Ho, Wo, Co, shortcut (Cs, stride), main channel counts (one per block)
+    (2, 14, 14, 256, (64, 1), (64,)),                  # first block of stage 1: shortcut + one block
+    (2, 14, 14, 256, (64, 1), (64, 64, 64)),           # all of stage 1
+    (2, 7, 7, 512, (256, 2), (128, 128, 128, 128)),    # stage 2: strided shortcut, two K steps per block
+    (3, 5, 7, 1024, (512, 2), (256, 256)),             # ragged pixel count, eight K steps in the shortcut
+    (1, 9, 9, 64, (128, 1), (64, 192)),                # Co < 128: 64x64 tiles; unequal K
+    (2, 6, 6, 132, (64, 1), (64, 64)),                 # Co % 128 != 0: a ragged column tile
+    (1, 3, 3, 2048, (1024, 2), (512, 512, 512)),       # stage 4: long K, few pixels
+    (2, 8, 8, 128, (64, 1), (64,) * 7),                # the most links the entry point takes
+]
+
+
+@pytest.mark.parametrize("case", CHAIN_CASES)
+def test_residual_chain(case):
+    """catchq_conv1x1_chain_nhwc against the oracle's block-by-block evaluation: shortcut (dequant + bias, fp32),
+    then every block's last convolution with the running fp32 tensor as its residual and ReLU; fp32 and int8
+    outputs of the last block, bit for bit, and of every prefix of the chain."""
+    n, ho, wo, co, (cs, ss), mains = case
+    note("residual_chain", case)
+    r = rng(n + ho + wo + co + cs + sum(mains))
+    links, run = [], None
+    for i, ci in enumerate((cs,) + tuple(mains)):
+        stride = ss if i == 0 else 1
+        h, w = (ho - 1) * stride + 1 + (stride - 1) * (i % 2), (wo - 1) * stride + 1
+        x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, 1, 1, ci), 8)
+        acc, ovf = orc.conv2d_nhwc(x, wt, (0, 0), (stride, stride), (1, 1), 1)
+        assert ovf == 0 and acc.shape == (n, ho, wo, co)
+        div, bias = r.uniform(0.6, 3.5, co).astype(np.float32), r.standard_normal(co).astype(np.float32)
+        exp2 = -10 - (i % 3) - (3 if ci > 256 else 0)
+        run = orc.epilogue(acc, exp2, div, bias, run, 0 if i == 0 else 1)
+        links.append(dict(x=cabi.dev(x), w=cabi.dev(wt.reshape(co, ci)), stride=stride, exp2=exp2, chan_div=cabi.dev(div),
+                          chan_rcp=cabi.dev(np.float32(1) / div), bias=cabi.dev(bias)))
+        if i == 0:
+            continue
+        out = cabi.conv1x1_chain_nhwc(links, q_pos=-3)
+        assert same_bits(run, out["y"].cpu().numpy()), i
+        assert same_bits(orc.quantize(run, 8, -3), out["q"].cpu().numpy()), i
+    q_only = cabi.conv1x1_chain_nhwc(links, want_y=False, q_pos=-2)
+    assert q_only["y"] is None and same_bits(orc.quantize(run, 8, -2), q_only["q"].cpu().numpy())
+    y_only = cabi.conv1x1_chain_nhwc(links, want_q=False)
+    assert y_only["q"] is None and same_bits(run, y_only["y"].cpu().numpy())
+
+
+def test_residual_chain_argument_checks():
+    note("residual_chain errors")
+    x = torch.zeros((1, 8, 8, 64), dtype=torch.int8, device="cuda")
+    w = torch.zeros((64, 64), dtype=torch.int8, device="cuda")
+    v = torch.ones(64, device="cuda")
+    ok = dict(x=x, w=w, stride=1, exp2=0, chan_div=v, chan_rcp=v, bias=v)
+    with pytest.raises(Exception):  # a single link is an ordinary convolution
+        cabi.conv1x1_chain_nhwc([ok])
+    with pytest.raises(Exception):  # grids differ: 4x4 against 8x8
+        cabi.conv1x1_chain_nhwc([ok, dict(ok, stride=2)])
+    with pytest.raises(Exception):  # no reciprocals
+        cabi.conv1x1_chain_nhwc([ok, dict(ok, chan_rcp=None)])
+    x48 = torch.zeros((1, 8, 8, 48), dtype=torch.int8, device="cuda")
+    with pytest.raises(Exception):  # channels not a multiple of 64
+        cabi.conv1x1_chain_nhwc([ok, dict(ok, x=x48, w=torch.zeros((64, 48), dtype=torch.int8, device="cuda"))])
+
+
 def test_conv_shortcut_argument_checks():
     note("conv_shortcut errors")
     x = torch.zeros((1, 8, 8, 16), dtype=torch.int8, device="cuda")

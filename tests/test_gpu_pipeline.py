@@ -174,14 +174,50 @@ def test_projection_shortcuts_fused_into_block_end(depth, expect):
     sd = pipeline.calibrate(net, x, "int8", True)
     fused = pipeline.FusedNet(layers, sd)
     plain = pipeline.FusedNet(layers, sd, fuse_shortcuts=False)
-    assert sorted(fused.shortcut_of) == expect and not plain.shortcut_of
-    assert sorted(l.name for l in fused.shortcut_of.values()) == [e.rsplit(".", 1)[0] + ".ds" for e in expect]
+    # (a bottleneck block's shortcut is the first link of a residual chain, a basic block's one half of a two-branch launch)
+    inside = dict(fused.shortcut_of, **{n: c[0] for n, c in fused.chain_of.items() if len(c) == 2})
+    assert sorted(inside) == expect and not plain.shortcut_of and not plain.chain_of
+    assert sorted(l.name for l in inside.values()) == [e.rsplit(".", 1)[0] + ".ds" for e in expect]
     timers = {}
     a = fused.forward(x.cuda(), timers=timers)
     b = plain.forward(x.cuda())
     torch.cuda.synchronize()
     assert torch.equal(a, b)
     assert not any(n.endswith(".ds") for n in timers)  # no launch of their own
+    check_against_oracle(layers, sd, x, fused)
+
+
+@pytest.mark.parametrize("limit", [None, 0, 2, 3, 8])
+def test_resnet50_residual_chains(limit):
+    """Blocks whose residual branch is recomputed from int8 tensors inside their last convolution's launch
+    (chain_links): every tensor the plan still produces equals the block-by-block plan's, the logits equal the
+    oracle's; with 8 links every block of every stage is a chain and no fp32 tensor is left between blocks."""
+    note("residual chains, resnet50, limit", limit)
+    layers = nets.resnet(50)
+    net = nets.FloatNet(layers, seed=8).eval()
+    x = torch.randn(3, 3, 96, 96, generator=torch.Generator().manual_seed(9))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd, chain_links=limit)
+    plain = pipeline.FusedNet(layers, sd, chain_links=0)
+    lens = {n: len(c) for n, c in fused.chain_of.items()}
+    if limit == 0:
+        assert not lens and sorted(fused.shortcut_of) == ["l1.0.c3", "l2.0.c3", "l3.0.c3", "l4.0.c3"]
+    elif limit == 2:
+        assert lens == {"l1.0.c3": 2, "l2.0.c3": 2, "l3.0.c3": 2, "l4.0.c3": 2} and not fused.shortcut_of
+    elif limit == 8:
+        assert len(lens) == 16 and lens["l3.5.c3"] == 7 and lens["l4.2.c3"] == 4 and not fused.shortcut_of
+        assert not any(fused.f_demand[n] for n in lens if n != "l4.2.c3")
+    else:
+        assert lens["l1.0.c3"] == 2 and lens["l1.1.c3"] == 3 and "l1.2.c3" not in lens
+    for name, c in fused.chain_of.items():
+        assert c[-1].name == name and c[0].name.endswith(".ds") and [l.name[:2] for l in c] == [name[:2]] * len(c)
+    ka, kb = {}, {}
+    a = fused.forward(x.cuda(), keep=ka)
+    b = plain.forward(x.cuda(), keep=kb)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    for key, t in ka.items():
+        assert torch.equal(t, kb[key]), key
     check_against_oracle(layers, sd, x, fused)
 
 
