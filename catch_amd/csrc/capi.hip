@@ -27,6 +27,7 @@ struct ChainLinkDev {  // igemm_i8_chain.hip
   unsigned x_bytes, w_bytes;
   int K;
   unsigned img_stride, row_stride, pix_stride;
+  int dense, k_shift;
   int exp2;
   const float *chan_div, *chan_rcp, *bias;
 };
@@ -278,6 +279,8 @@ CATCHQ_API int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int n
     dev[i].img_stride = (unsigned)(l.in_h * l.in_w * l.ci);
     dev[i].row_stride = (unsigned)(l.stride * l.in_w * l.ci);
     dev[i].pix_stride = (unsigned)(l.stride * l.ci);
+    dev[i].dense = (l.stride == 1 && l.in_h == ho && l.in_w == wo) ? 1 : 0;
+    dev[i].k_shift = -1;
     dev[i].exp2 = l.exp2;
     dev[i].chan_div = l.chan_div;
     dev[i].chan_rcp = l.chan_rcp;

@@ -27,6 +27,8 @@ struct ChainLinkDev {
   unsigned x_bytes, w_bytes;
   int K;                                        // bytes per input pixel = channels (multiple of 64)
   unsigned img_stride, row_stride, pix_stride;  // bytes per image / per OUTPUT row / per OUTPUT column of x
+  int dense;    // stride 1 on an input of the output's extent: pixel m sits at m * K, no (image, row, column) split
+  int k_shift;  // log2(K) when K is a power of two, else -1
   int exp2;
   const float *chan_div, *chan_rcp, *bias;
 };
@@ -41,6 +43,7 @@ struct ChainParams {
   int8_t *q;
   int q_neg_pos;
   int y_stream;
+  int any_strided;  // some link is not dense
   ChainLinkDev link[kChainMaxLinks];
 };
 
@@ -75,23 +78,26 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
   const int lrow = lane >> 2;
   const unsigned lchunk16 = (unsigned)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
   bool row_ok[NI];
-  unsigned r_img[NI], r_ho[NI], r_wo[NI];  // A rows: the pixel; B rows: r_img = channel
+  unsigned r_idx[NI];                      // A rows: the pixel index; B rows: the channel
+  unsigned r_img[NI], r_ho[NI], r_wo[NI];  // A rows, only when some link is strided: the pixel split up
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const int trow = (wave * NI + j) * 16 + lrow;
-    if (trow < BM) {
+    r_img[j] = r_ho[j] = r_wo[j] = 0;
+    if ((wave * NI + j) * 16 < BM) {  // wave-uniform
       const int64_t m = m0 + trow;
       row_ok[j] = m < cp.M;
-      const unsigned mu = row_ok[j] ? (unsigned)m : 0u;
-      const unsigned t = mu / (unsigned)cp.Wo;
-      r_wo[j] = mu - t * (unsigned)cp.Wo;
-      r_img[j] = t / (unsigned)cp.Ho;
-      r_ho[j] = t - r_img[j] * (unsigned)cp.Ho;
+      r_idx[j] = row_ok[j] ? (unsigned)m : 0u;
+      if (cp.any_strided) {
+        const unsigned t = r_idx[j] / (unsigned)cp.Wo;
+        r_wo[j] = r_idx[j] - t * (unsigned)cp.Wo;
+        r_img[j] = t / (unsigned)cp.Ho;
+        r_ho[j] = t - r_img[j] * (unsigned)cp.Ho;
+      }
     } else {
       const int n = n0 + trow - BM;
       row_ok[j] = n < cp.N;
-      r_img[j] = row_ok[j] ? (unsigned)n : 0u;
-      r_ho[j] = r_wo[j] = 0;
+      r_idx[j] = row_ok[j] ? (unsigned)n : 0u;
     }
   }
   // the issuing side of the ring: link and K offset of the next step to request
@@ -105,8 +111,10 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       const bool is_a = (wave * NI + j) * 16 < BM;  // wave-uniform
-      const unsigned b = is_a ? r_img[j] * ln.img_stride + r_ho[j] * ln.row_stride + r_wo[j] * ln.pix_stride
-                              : r_img[j] * (unsigned)ln.K;
+      unsigned b;
+      if (is_a && !ln.dense) b = r_img[j] * ln.img_stride + r_ho[j] * ln.row_stride + r_wo[j] * ln.pix_stride;
+      else b = ln.k_shift >= 0 ? r_idx[j] << ln.k_shift : r_idx[j] * (unsigned)ln.K;
+      // an offset at or above 2^31 is out of range for every buffer here and stays so when a K offset is added
       base[j] = (row_ok[j] && i < L) ? b + lchunk16 : OOB;
     }
   };
@@ -118,7 +126,7 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
     for (int j = 0; j < NI; ++j) {
       const int slot = wave * NI + j;
       const bool is_a = slot * 16 < BM;
-      const unsigned voff = base[j] == OOB ? OOB : base[j] + (unsigned)ik;
+      const unsigned voff = base[j] + (unsigned)ik;
       lds_ptr_t dst = (lds_ptr_t)(lds_dyn + stage_off + slot * 1024);
       if (is_a) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, (int)voff, 0, 0, 0);
       else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, (int)voff, 0, 0, 0);
@@ -160,10 +168,6 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
 
   v16i acc[TN];
   float prev[TN][16];
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) prev[j][r] = 0.0f;
 
   auto fetch = [&](v4i &fa, v4i (&fb)[TN], unsigned a_addr, unsigned b_addr) {
     fa = ds_read_b128<0>(a_addr);
@@ -174,37 +178,40 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
   };
 
   int rd_off = 0, wr_off = (STAGES - 1) * STAGE_BYTES;
-  for (int i = 0; i < L; ++i) {
+  // one K step of 64 bytes; FIRST: the link's sums start from zero (the matrix instruction takes the constant)
+  auto step = [&](auto first_c) {
+    constexpr bool FIRST = decltype(first_c)::value;
+    CATCHQ_VMCNT(NI * (STAGES - 2));  // this wave's part of the stage has landed
+    __builtin_amdgcn_s_barrier();     // ... and everyone's; the slot refilled below is no longer read
+    const unsigned a0 = a_row + (unsigned)rd_off, b0 = b_row + (unsigned)rd_off;
+    v4i fa[2], fb[2][TN];
+    fetch(fa[0], fb[0], a0 + off_k, b0 + off_k);
+    fetch(fa[1], fb[1], a0 + (off_k ^ 32u), b0 + (off_k ^ 32u));
+    issue_step(wr_off);
+    {
+      v4i(&one)[1] = reinterpret_cast<v4i(&)[1]>(fa[0]);
+      lgkm_wait_frags<1 + TN, 1, TN>(one, fb[0]);
+    }
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[j][r] = 0;
-    const int nsteps = cp.link[i].K >> 6;
-    for (int s = 0; s < nsteps; ++s) {
-      CATCHQ_VMCNT(NI * (STAGES - 2));  // this wave's part of the stage has landed
-      __builtin_amdgcn_s_barrier();     // ... and everyone's; the slot refilled below is no longer read
-      const unsigned a0 = a_row + (unsigned)rd_off, b0 = b_row + (unsigned)rd_off;
-      v4i fa[2], fb[2][TN];
-      fetch(fa[0], fb[0], a0 + off_k, b0 + off_k);
-      fetch(fa[1], fb[1], a0 + (off_k ^ 32u), b0 + (off_k ^ 32u));
-      issue_step(wr_off);
-      {
-        v4i(&one)[1] = reinterpret_cast<v4i(&)[1]>(fa[0]);
-        lgkm_wait_frags<1 + TN, 1, TN>(one, fb[0]);
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0], fb[0][j], acc[j], 0, 0, 0);
-      {
-        v4i(&one)[1] = reinterpret_cast<v4i(&)[1]>(fa[1]);
-        lgkm_wait_frags<0, 1, TN>(one, fb[1]);
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[1], fb[1][j], acc[j], 0, 0, 0);
-      rd_off = (rd_off + STAGE_BYTES == PIPE_BYTES) ? 0 : rd_off + STAGE_BYTES;
-      wr_off = (wr_off + STAGE_BYTES == PIPE_BYTES) ? 0 : wr_off + STAGE_BYTES;
+      acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0], fb[0][j], FIRST ? zero : acc[j], 0, 0, 0);
+    {
+      v4i(&one)[1] = reinterpret_cast<v4i(&)[1]>(fa[1]);
+      lgkm_wait_frags<0, 1, TN>(one, fb[1]);
     }
-    // fold this link into the running values: v = acc / d + bias (reciprocal form), then relu(v + previous)
-    // for every link after the shortcut
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[1], fb[1][j], acc[j], 0, 0, 0);
+    rd_off = (rd_off + STAGE_BYTES == PIPE_BYTES) ? 0 : rd_off + STAGE_BYTES;
+    wr_off = (wr_off + STAGE_BYTES == PIPE_BYTES) ? 0 : wr_off + STAGE_BYTES;
+  };
+  // one link: its K steps, then its sums are folded into the running values: v = acc / d + bias (reciprocal
+  // form), and relu(v + previous) for every link after the shortcut
+  auto link = [&](int i, auto shortcut_c) {
+    constexpr bool SHORTCUT = decltype(shortcut_c)::value;
+    const int nsteps = cp.link[i].K >> 6;
+    step(std::true_type{});
+    for (int s = 1; s < nsteps; ++s) step(std::false_type{});
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int c = wave_n * WN + j * 32 + frow;
@@ -212,14 +219,16 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         float v = div_by_rcp((float)acc[j][r], d, rc) + b;
-        if (i > 0) {
+        if constexpr (!SHORTCUT) {
           v = v + prev[j][r];
           v = (v > 0.0f) ? v : 0.0f;
         }
         prev[j][r] = v;
       }
     }
-  }
+  };
+  link(0, std::true_type{});
+  for (int i = 1; i < L; ++i) link(i, std::false_type{});
   CATCHQ_VMCNT(0);
   __syncthreads();  // the ring is dead: it becomes the staging area
 
@@ -235,33 +244,41 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
   constexpr int NIT = 32 / RPI;
   const int cg = lane % CPR, rsub = lane / CPR;
   const int64_t m_w = m0 + wave_m * WM;
-  const int n = n0 + wave_n * WN + cg * 4;
-  const bool n_ok = n < cp.N;
+  const int n_w = n0 + wave_n * WN;
   const float hi = __builtin_ldexpf(127.0f, -cp.q_neg_pos);
   const float sc = __builtin_ldexpf(1.0f, cp.q_neg_pos);
   v4f vv[NIT];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) vv[it] = *reinterpret_cast<const v4f *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
+  // an element's index: a wave-uniform 64-bit part plus a 32-bit per-lane part
+  const int64_t uni = m_w * (int64_t)cp.N + n_w;
+  const unsigned lane_off = (unsigned)rsub * (unsigned)cp.N + (unsigned)(cg * 4);
+  const unsigned it_step = (unsigned)RPI * (unsigned)cp.N;
+  auto emit = [&](auto full_c) {
+    constexpr bool FULL = decltype(full_c)::value;
+    const bool n_ok = FULL || n_w + cg * 4 < cp.N;
 #pragma unroll
-  for (int it = 0; it < NIT; ++it) {
-    const int64_t m = m_w + it * RPI + rsub;
-    if (!n_ok || m >= cp.M) continue;
-    const int64_t idx = m * cp.N + n;
-    if (cp.y) store_stream(reinterpret_cast<v4f *>(cp.y + idx), vv[it], cp.y_stream != 0);
-    if (cp.q) {
-      // values are >= 0 and never NaN (the ReLU above): sat(rne(x * 2^-pos)) = low byte of the float
-      // fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23), as in the shared epilogue
-      unsigned b[4];
+    for (int it = 0; it < NIT; ++it) {
+      if (!FULL && !(n_ok && m_w + it * RPI + rsub < cp.M)) continue;
+      const unsigned off = lane_off + it * it_step;
+      if (cp.y) store_stream(reinterpret_cast<v4f *>((cp.y + uni) + off), vv[it], cp.y_stream != 0);
+      if (cp.q) {
+        // values are >= 0 and never NaN (the ReLU above): sat(rne(x * 2^-pos)) = low byte of the float
+        // fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23), as in the shared epilogue
+        unsigned b[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const float x = __builtin_amdgcn_fmed3f(vv[it][t], 0.0f, hi);
-        b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
+        for (int t = 0; t < 4; ++t) {
+          const float x = __builtin_amdgcn_fmed3f(vv[it][t], 0.0f, hi);
+          b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
+        }
+        const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+        const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+        *reinterpret_cast<unsigned *>((cp.q + uni) + off) = lo | hi2;
       }
-      const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-      const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
-      *reinterpret_cast<unsigned *>(cp.q + idx) = lo | hi2;
     }
-  }
+  };
+  if (m_w + 32 <= cp.M && n_w + WN <= cp.N) emit(std::true_type{});  // wave-uniform: the tile lies inside the matrix
+  else emit(std::false_type{});
 }
 
 template <int BM, int BN, int STAGES, int MINW>
@@ -302,6 +319,10 @@ int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int W
     if (!ln.chan_div || !ln.chan_rcp || !ln.bias || ln.exp2 < -64 || ln.exp2 > 64) return -1;
     if (!aligned16(ln.x) || !aligned16(ln.w)) return -1;
     cp.link[i] = ln;
+    cp.link[i].k_shift = -1;
+    for (int sft = 6; sft < 31; ++sft)
+      if (ln.K == (1 << sft)) cp.link[i].k_shift = sft;
+    if (!ln.dense) cp.any_strided = 1;
   }
   int variant = 0;
   if (const char *v = tuning_env("CATCHQ_CHAIN_VARIANT")) variant = atoi(v);
@@ -309,8 +330,8 @@ int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int W
   switch (variant) {
     case 1: return launch_chain<64, 128, 2, 1>(cp, s);
     case 2: return launch_chain<64, 128, 2, 4>(cp, s);
-    case 3: return launch_chain<64, 128, 3, 4>(cp, s);
-    default: return launch_chain<64, 128, 3, 1>(cp, s);
+    case 3: return launch_chain<64, 128, 3, 1>(cp, s);
+    default: return launch_chain<64, 128, 3, 4>(cp, s);
   }
 }
 
