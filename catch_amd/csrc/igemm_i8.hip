@@ -360,8 +360,15 @@ int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, in
   p.K = kh * kw * Ci;
   if (dma_enabled() && kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
     // a pointwise convolution is a plain GEMM over the pixels
-    const int st = gemm_nt_stream_i8(x, w, p.M, Co, Ci, e, s);
+    int st = gemm_nt_stream_i8(x, w, p.M, Co, Ci, e, s);
     if (st >= 0) return st;
+    // ... and takes the GEMM loader of the pipelined kernel: a row's address is its index times K, with no
+    // (image, row, column) split and no tap masks in front of the first load
+    const char *as_gemm = tuning_env("CATCHQ_PW_AS_GEMM");
+    if (Ci % 16 == 0 && !(as_gemm && atoi(as_gemm) == 0)) {
+      st = igemm_dma_launch(LOAD_GEMM, x, w, p, e, p.M * Ci, (int64_t)Co * Ci, s);
+      if (st >= 0) return st;
+    }
   }
   if (dma_enabled() && halo_enabled() && kh == 3 && kw == 3 && sh == sw && ph == 1 && pw == 1 && dh == 1 && dw == 1) {
     // the input patch of a band of output rows stays in LDS for all nine taps
