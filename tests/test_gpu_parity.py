@@ -153,6 +153,8 @@ def _ints(r, shape, bits):
 
 
 GEMM_SHAPES = [(1, 1, 16), (5, 7, 16), (128, 128, 64), (130, 70, 80), (257, 129, 1040), (64, 1000, 2048),
+               # a handful of blocks, long K: 128-byte steps through a four-stage ring (K ending inside a step, ragged tiles)
+               (100, 200, 1072), (33, 500, 4096), (7, 65, 1936),
                (300, 64, 48), (1, 10, 10), (20, 125, 100), (33, 17, 7),
                # many rows, short K, narrow N: the streaming kernel, one shape per (K steps, N fragments) class
                (5000, 96, 16), (4100, 16, 32), (8200, 144, 32), (4099, 24, 96), (6000, 64, 64), (4097, 160, 32),
@@ -375,6 +377,7 @@ CONV_CASES = [
     (2, 32, 13, 13, 64, 3, 3, (1, 1), (2, 2), (1, 1), 1),      # 3x3 stride 2
     (1, 48, 10, 12, 40, 3, 3, (2, 2), (1, 1), (2, 2), 1),      # dilation
     (1, 128, 7, 7, 256, 3, 3, (1, 1), (1, 1), (1, 1), 1),
+    (2, 128, 9, 9, 96, 3, 3, (1, 1), (2, 2), (1, 1), 1),       # few blocks, K = 1152: the wide ring with the im2col loader
     (1, 16, 5, 5, 32, 5, 5, (2, 2), (1, 1), (1, 1), 1),
     (1, 80, 8, 8, 16, 7, 1, (3, 0), (1, 1), (1, 1), 1),        # asymmetric kernel
     (2, 4, 30, 30, 64, 7, 7, (3, 3), (2, 2), (1, 1), 1),       # 4-channel input, 7x7 s2 (network stem)
