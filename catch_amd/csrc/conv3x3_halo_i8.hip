@@ -68,8 +68,8 @@ __device__ __forceinline__ unsigned halo_key(unsigned prow, unsigned pcol, unsig
   return (prow >> SH) * wo_count + (pcol >> SH);
 }
 
-template <int CI, int TN, int TMW, int S, int EPI>
-__global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+template <int CI, int TN, int TMW, int S, int EPI, int NW = 4>
+__global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
                                                           HaloParams hp, EpiDev e) {
   resolve_exp2(e);
   constexpr int CH = CI / 16;         // 16-byte chunks per pixel
@@ -78,12 +78,13 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
   constexpr int KS = 256;             // bytes of K per weight stage
   constexpr int STAGES = 3;
   constexpr int B_STAGE = BN * KS;
-  constexpr int NIB = BN / 4 / 4;     // weight DMA instructions (4 rows x 256 bytes) per wave and stage
+  constexpr int NIB = BN / 4 / NW;    // weight DMA instructions (4 rows x 256 bytes) per wave and stage
   constexpr int K = 9 * CI;
   constexpr int NSTAGES = (K + KS - 1) / KS;
   constexpr int SUBS_PER_TAP = CI / 32;  // MFMA K steps (32 bytes) per filter tap
   constexpr int SUBS_PER_STAGE = KS / 32;
-  static_assert(BN / 4 % 4 == 0, "the weight rows must split evenly over the four waves");
+  static_assert(NW == 4 || NW == 8, "four or eight waves");
+  static_assert(BN / 4 % NW == 0, "the weight rows must split evenly over the waves");
   static_assert(TMW == 1 || TMW == 2, "one or two sub-tiles per wave");
   // 1 KiB alignment: fragment addresses are formed by XOR-ing chunk bits into a precomputed address
   extern __shared__ __attribute__((aligned(1024))) int8_t lds_dyn[];
@@ -121,10 +122,10 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
     const int ninstr = patch_bytes / 1024;
     constexpr int PPI = 64 / CH > 0 ? 64 / CH : 1;  // pixels per DMA instruction (CH <= 32)
     // this lane's pixel in the wave's first instruction, then PPI * 4 pixels further per round
-    unsigned pix = (unsigned)(wave * 64 + lane) / CH;
+    unsigned pix = (unsigned)(wave * 64 + lane) / CH;  // (NW waves: instruction i of the patch belongs to wave i % NW)
     const unsigned phys = (unsigned)lane % CH;
     unsigned pr = pix / (unsigned)hp.PC, pc = pix - pr * (unsigned)hp.PC;
-    for (int i = wave; i < ninstr; i += 4) {
+    for (int i = wave; i < ninstr; i += NW) {
       int img = img0, hi;
       if (hp.image_mode) {
         const unsigned g = pr / (unsigned)hp.img_rows;
@@ -138,8 +139,8 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
       const unsigned src = (unsigned)((img * hp.Hi + hi) * hp.Wi + wi) * (unsigned)CI + ((phys ^ halo_swz<CH>(halo_key<S>(pr, pc, (unsigned)hp.W))) << 4);
       const unsigned voff = select_u32(ok, src, OOB);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr_t)(lds_dyn + i * 1024), 16, (int)voff, 0, 0, 0);
-      pix += PPI * 4;
-      pc += PPI * 4;
+      pix += PPI * NW;
+      pc += PPI * NW;
       while (pc >= (unsigned)hp.PC) { pc -= (unsigned)hp.PC; ++pr; }
     }
   }
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
   unsigned a0[TMW][9];
 #pragma unroll
   for (int i = 0; i < TMW; ++i) {
-    int idx = (wave + 4 * i) * 32 + frow;
+    int idx = (wave + NW * i) * 32 + frow;
     if (idx >= p_tile) idx = p_tile - 1;
     const unsigned tr = (unsigned)idx / (unsigned)hp.W, wo = (unsigned)idx - tr * (unsigned)hp.W;
     unsigned prow = tr;
@@ -263,34 +264,39 @@ __global__ __launch_bounds__(256) void conv3x3_halo_kernel(const int8_t *__restr
   int *stage_w = reinterpret_cast<int *>(ring) + wave * 32 * EPI_STRIDE;
 #pragma unroll
   for (int i = 0; i < TMW; ++i) {
-    const int si = wave + 4 * i;
+    const int si = wave + NW * i;
     if (si * 32 >= p_tile) break;  // wave-uniform
     igemm_epilogue<1, TN, EPI>(reinterpret_cast<v16i(&)[1][TN]>(acc[i]), stage_w, m0 + si * 32, n0, lane, p, e);
   }
 }
 
-template <int CI, int TN, int TMW, int S, int EPI>
+template <int CI, int TN, int TMW, int S, int EPI, int NW>
 static int launch_halo_epi(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
-  auto kern = conv3x3_halo_kernel<CI, TN, TMW, S, EPI>;
+  auto kern = conv3x3_halo_kernel<CI, TN, TMW, S, EPI, NW>;
   if (lds_bytes > 64 * 1024) {
     static std::atomic<bool> raised[64];
     if (raise_lds_limit((const void *)kern, 160 * 1024, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
   }
-  kern<<<hp.nblocks, 256, lds_bytes, s>>>((const int8_t *)x, (const int8_t *)w, hp, e);
+  kern<<<hp.nblocks, 64 * NW, lds_bytes, s>>>((const int8_t *)x, (const int8_t *)w, hp, e);
   return launch_status();
 }
 
-template <int CI, int TN, int TMW, int S>
+template <int CI, int TN, int TMW, int S, int NW = 4>
 static int launch_halo_tm(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
   switch (pick_epilogue(hp.Co, e)) {
     case EPI_SCALAR: return -1;
-    case EPI_Q8_RELU: return launch_halo_epi<CI, TN, TMW, S, EPI_Q8_RELU>(x, w, hp, e, lds_bytes, s);
-    default: return launch_halo_epi<CI, TN, TMW, S, EPI_VECTOR>(x, w, hp, e, lds_bytes, s);
+    case EPI_Q8_RELU: return launch_halo_epi<CI, TN, TMW, S, EPI_Q8_RELU, NW>(x, w, hp, e, lds_bytes, s);
+    default: return launch_halo_epi<CI, TN, TMW, S, EPI_VECTOR, NW>(x, w, hp, e, lds_bytes, s);
   }
 }
 
 template <int CI, int S>
-static int launch_halo(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int tn, int lds_bytes, hipStream_t s) {
+static int launch_halo(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int tn, int lds_bytes, int waves,
+                       hipStream_t s) {
+  // five to eight sub-tiles on eight waves: one each, two waves per SIMD that overlap each other's fragment
+  // fetches and multiplications
+  if (waves == 8)
+    return tn == 2 ? launch_halo_tm<CI, 2, 1, S, 8>(x, w, hp, e, lds_bytes, s) : launch_halo_tm<CI, 1, 1, S, 8>(x, w, hp, e, lds_bytes, s);
   // four or fewer sub-tiles: one per wave, no second set of accumulators
   if (hp.nsub <= 4)
     return tn == 2 ? launch_halo_tm<CI, 2, 1, S>(x, w, hp, e, lds_bytes, s) : launch_halo_tm<CI, 1, 1, S>(x, w, hp, e, lds_bytes, s);
@@ -376,21 +382,24 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, 
   if (stride == 2 && nb > 256) return -1;
   hp.nblocks = (int)nb;
   int lds_bytes = lds + 3 * 32 * tn * 256;
-  const int epi_bytes = lds + 4 * 32 * (32 * tn + 8) * 4;  // the epilogue's staging area lies where the ring was
+  int waves = 4;
+  if (hp.nsub > 4 && lds + 8 * 32 * (32 * tn + 8) * 4 <= kLdsLimit) waves = 8;
+  if (const char *t = tuning_env("CATCHQ_HALO_WAVES")) waves = (atoi(t) == 8 && hp.nsub > 4) ? 8 : 4;
+  const int epi_bytes = lds + waves * 32 * (32 * tn + 8) * 4;  // the epilogue's staging area lies where the ring was
   if (epi_bytes > lds_bytes) lds_bytes = epi_bytes;
   if (lds_bytes > kLdsLimit) return -1;
   if (stride == 2) {
     switch (Ci) {
-      case 128: return launch_halo<128, 2>(x, w, hp, e, tn, lds_bytes, s);
-      case 256: return launch_halo<256, 2>(x, w, hp, e, tn, lds_bytes, s);
-      default: return launch_halo<512, 2>(x, w, hp, e, tn, lds_bytes, s);
+      case 128: return launch_halo<128, 2>(x, w, hp, e, tn, lds_bytes, waves, s);
+      case 256: return launch_halo<256, 2>(x, w, hp, e, tn, lds_bytes, waves, s);
+      default: return launch_halo<512, 2>(x, w, hp, e, tn, lds_bytes, waves, s);
     }
   }
   switch (Ci) {
-    case 64: return launch_halo<64, 1>(x, w, hp, e, tn, lds_bytes, s);
-    case 128: return launch_halo<128, 1>(x, w, hp, e, tn, lds_bytes, s);
-    case 256: return launch_halo<256, 1>(x, w, hp, e, tn, lds_bytes, s);
-    default: return launch_halo<512, 1>(x, w, hp, e, tn, lds_bytes, s);
+    case 64: return launch_halo<64, 1>(x, w, hp, e, tn, lds_bytes, waves, s);
+    case 128: return launch_halo<128, 1>(x, w, hp, e, tn, lds_bytes, waves, s);
+    case 256: return launch_halo<256, 1>(x, w, hp, e, tn, lds_bytes, waves, s);
+    default: return launch_halo<512, 1>(x, w, hp, e, tn, lds_bytes, waves, s);
   }
 }
 
