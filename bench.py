@@ -466,7 +466,7 @@ def main():
         print("sum of conv/fc launches (%d parts of %d images): %.1f us repeated back to back, %.1f us in sequence; graph step: %.1f us" % (
             n_parts, parts[0].shape[0], t_all * 1e6, n_parts * sum(r["t_seq"] for r in rows) * 1e6, ms_per_step * 1e3), file=sys.stderr)
     roofline = {"bound": "hbm", "kernel": "%s (all %d launches of one step: %d layers x %d parts of the batch)" % (
-                    "igemm_a16_dma_kernel" if detector else "igemm_i8_dma_kernel + conv3x3_halo_kernel + igemm_i8_dual_kernel",
+                    "igemm_a16_dma_kernel" if detector else "igemm_i8_dma_kernel + conv3x3_halo_kernel + igemm_i8_chain_kernel",
                     n_parts * len(conv_rows), len(conv_rows), n_parts),
                 "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
