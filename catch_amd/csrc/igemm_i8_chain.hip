@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
   constexpr int NI = (BM + BN) / 16 / NW;  // DMA instructions (16 rows x 64 bytes) per wave and stage
   static_assert((BM + BN) / 16 % NW == 0, "tile rows must split evenly over the waves");
   constexpr int EPI_STRIDE = WN + 8;
-  constexpr int EPI_BYTES = NW * 32 * EPI_STRIDE * 4;
+  constexpr int EPI_BYTES = NW * 16 * EPI_STRIDE * 4;  // the staging area holds 16 rows of a wave's 32 at a time
   constexpr int FRONT_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;  // ring, later the staging area
   extern __shared__ __attribute__((aligned(16))) int8_t lds_dyn[];
   float *consts = reinterpret_cast<float *>(lds_dyn + FRONT_BYTES);  // [link][div' | rcp' | bias][BN]
@@ -232,53 +232,59 @@ __global__ __launch_bounds__(256, MINW) void igemm_i8_chain_kernel(ChainParams c
   CATCHQ_VMCNT(0);
   __syncthreads();  // the ring is dead: it becomes the staging area
 
-  // ---- the last link's values leave through the wave's staging area: a lane then owns 4 consecutive channels
-  // of one pixel (16-byte fp32 / 4-byte int8 stores, rows contiguous) ------------------------------------------
-  float *stage = reinterpret_cast<float *>(lds_dyn) + wave * 32 * EPI_STRIDE;
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = prev[j][r];
+  // ---- the last link's values leave through the wave's staging area, 16 of its 32 rows at a time: a lane then
+  // owns 4 consecutive channels of one pixel (16-byte fp32 / 4-byte int8 stores, rows contiguous).  The small area
+  // keeps the block's LDS low enough for four blocks per compute unit with a two-stage ring. -------------------
+  float *stage = reinterpret_cast<float *>(lds_dyn) + wave * 16 * EPI_STRIDE;
   constexpr int CPR = WN / 4;    // 4-channel groups per staged row
   constexpr int RPI = 64 / CPR;  // rows the wave moves per iteration
-  constexpr int NIT = 32 / RPI;
+  constexpr int NIT = 16 / RPI;  // iterations per pass of 16 rows
   const int cg = lane % CPR, rsub = lane / CPR;
-  const int64_t m_w = m0 + wave_m * WM;
   const int n_w = n0 + wave_n * WN;
   const float hi = __builtin_ldexpf(127.0f, -cp.q_neg_pos);
   const float sc = __builtin_ldexpf(1.0f, cp.q_neg_pos);
-  v4f vv[NIT];
-#pragma unroll
-  for (int it = 0; it < NIT; ++it) vv[it] = *reinterpret_cast<const v4f *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
-  // an element's index: a wave-uniform 64-bit part plus a 32-bit per-lane part
-  const int64_t uni = m_w * (int64_t)cp.N + n_w;
   const unsigned lane_off = (unsigned)rsub * (unsigned)cp.N + (unsigned)(cg * 4);
   const unsigned it_step = (unsigned)RPI * (unsigned)cp.N;
-  auto emit = [&](auto full_c) {
-    constexpr bool FULL = decltype(full_c)::value;
-    const bool n_ok = FULL || n_w + cg * 4 < cp.N;
 #pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      if (!FULL && !(n_ok && m_w + it * RPI + rsub < cp.M)) continue;
-      const unsigned off = lane_off + it * it_step;
-      if (cp.y) store_stream(reinterpret_cast<v4f *>((cp.y + uni) + off), vv[it], cp.y_stream != 0);
-      if (cp.q) {
-        // values are >= 0 and never NaN (the ReLU above): sat(rne(x * 2^-pos)) = low byte of the float
-        // fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23), as in the shared epilogue
-        unsigned b[4];
+  for (int h = 0; h < 2; ++h) {
+    // rows 16h .. 16h+15 of the accumulator block are its registers 8h .. 8h+7 (row = 8 (r / 4) + 4 fhalf + r % 4);
+    // the wave's LDS operations complete in order, so these writes cannot overtake the previous pass's reads
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const float x = __builtin_amdgcn_fmed3f(vv[it][t], 0.0f, hi);
-          b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = prev[j][8 * h + r];
+    v4f vv[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) vv[it] = *reinterpret_cast<const v4f *>(stage + (it * RPI + rsub) * EPI_STRIDE + cg * 4);
+    // an element's index: a wave-uniform 64-bit part plus a 32-bit per-lane part
+    const int64_t m_w = m0 + wave_m * WM + 16 * h;
+    const int64_t uni = m_w * (int64_t)cp.N + n_w;
+    auto emit = [&](auto full_c) {
+      constexpr bool FULL = decltype(full_c)::value;
+      const bool n_ok = FULL || n_w + cg * 4 < cp.N;
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        if (!FULL && !(n_ok && m_w + it * RPI + rsub < cp.M)) continue;
+        const unsigned off = lane_off + it * it_step;
+        if (cp.y) store_stream(reinterpret_cast<v4f *>((cp.y + uni) + off), vv[it], cp.y_stream != 0);
+        if (cp.q) {
+          // values are >= 0 and never NaN (the ReLU above): sat(rne(x * 2^-pos)) = low byte of the float
+          // fma(min(x, 127 * 2^pos), 2^-pos, 1.5 * 2^23), as in the shared epilogue
+          unsigned b[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const float x = __builtin_amdgcn_fmed3f(vv[it][t], 0.0f, hi);
+            b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, sc, 12582912.0f));
+          }
+          const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+          const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+          *reinterpret_cast<unsigned *>((cp.q + uni) + off) = lo | hi2;
         }
-        const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-        const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
-        *reinterpret_cast<unsigned *>((cp.q + uni) + off) = lo | hi2;
       }
-    }
-  };
-  if (m_w + 32 <= cp.M && n_w + WN <= cp.N) emit(std::true_type{});  // wave-uniform: the tile lies inside the matrix
-  else emit(std::false_type{});
+    };
+    if (m_w + 16 <= cp.M && n_w + WN <= cp.N) emit(std::true_type{});  // wave-uniform: the rows lie inside the matrix
+    else emit(std::false_type{});
+  }
 }
 
 template <int BM, int BN, int STAGES, int MINW>
@@ -288,7 +294,7 @@ static int launch_chain(ChainParams &cp, hipStream_t s) {
   const int64_t nb = tiles_m * cp.tiles_n;
   if (nb > 0x7fffffff) return CATCHQ_ERR_SHAPE;
   cp.nblocks = (int)nb;
-  constexpr int PIPE = STAGES * (BM + BN) * 64, EPI = 4 * 32 * (BN / 2 + 8) * 4;
+  constexpr int PIPE = STAGES * (BM + BN) * 64, EPI = 4 * 16 * (BN / 2 + 8) * 4;
   const int lds_bytes = (PIPE > EPI ? PIPE : EPI) + cp.nlinks * 3 * BN * 4;
   igemm_i8_chain_kernel<BM, BN, STAGES, MINW><<<cp.nblocks, 256, lds_bytes, s>>>(cp);
   return launch_status();
@@ -331,8 +337,16 @@ int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int W
     case 1: return launch_chain<64, 128, 2, 1>(cp, s);
     case 2: return launch_chain<64, 128, 2, 4>(cp, s);
     case 3: return launch_chain<64, 128, 3, 1>(cp, s);
-    default: return launch_chain<64, 128, 3, 4>(cp, s);
+    default: break;
   }
+  // every link a single K step: the fold between two steps covers the load of the next, a two-stage ring is
+  // enough and leaves LDS for four blocks per compute unit
+  int max_k = 0;
+  for (int i = 0; i < nlinks; ++i) max_k = links[i].K > max_k ? links[i].K : max_k;
+  int k2 = 64;
+  if (const char *v = tuning_env("CATCHQ_CHAIN_K2")) k2 = atoi(v);
+  if (max_k <= k2) return launch_chain<64, 128, 2, 4>(cp, s);
+  return launch_chain<64, 128, 3, 4>(cp, s);
 }
 
 }  // namespace catchq
