@@ -14,8 +14,9 @@
 // block) is traded for matrix-core work (2K operations per element and link) and ~7 vector operations.
 //
 // All links' K steps form one sequence that streams through one LDS ring (LDS-DMA, 64-byte steps, three
-// stages): while the last step of a link is multiplied, the first steps of the next link are already
-// on their way, so a link costs no pipeline drain of its own.
+// stages, or two when every link is a single step and the fold between two steps covers the next load):
+// while the last step of a link is multiplied, the first steps of the next link are already on their way,
+// so a link costs no pipeline drain of its own.
 #include "igemm_i8_dma.inc"
 
 namespace catchq {

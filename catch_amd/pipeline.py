@@ -230,8 +230,11 @@ class FusedNet(object):
         self.chain_of = {}
         if fuse_shortcuts and chain_links != 0:
             self._plan_chains(chain_links)
+        # a shortcut has no launch of its own when its one reader, the first block's last convolution, evaluates it
+        # itself (as a two-branch launch or as the head of a chain); later blocks' chains recompute it either way
         self._fused_away = set(ds.name for ds in self.shortcut_of.values())
-        self._fused_away.update(links[0].name for links in self.chain_of.values())
+        self._fused_away.update(links[0].name for links in self.chain_of.values()
+                                if links[1].name in self.chain_of or links[1].name in self.shortcut_of)
 
     @staticmethod
     def _default_chain_links(co):
