@@ -664,6 +664,13 @@ int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, i
     const int st = conv2d_stem_a16(x, w, N, H, W, Co, kh, kw, sh, sw, dh, Ho, Wo, e, s);
     if (st >= 0) return st;
   }
+  // a pointwise convolution is a plain GEMM over the pixels: row address = index x K, no pixel split and no
+  // tap masks in front of the first load
+  const char *as_gemm = tuning_env("CATCHQ_PW_AS_GEMM");
+  if (kh == 1 && kw == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && !(as_gemm && atoi(as_gemm) == 0)) {
+    const int st = igemm_a16_launch(LOAD_GEMM, x, w, p, e, p.M * Ci * 2, (int64_t)Co * Ci, s);
+    if (st >= 0) return st;
+  }
   return igemm_a16_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci * 2, (int64_t)Co * p.K, s);
 }
 
