@@ -384,7 +384,9 @@ def main():
     config = {"workload": "%s %s, fused requant pipeline replayed from a HIP graph%s" % (
         args.workload, what, "" if args.streams <= 1 else " (the batch in %d parts on parallel streams)" % args.streams),
               "global_batch": batch, "calibration_images": args.calib_images, "graph_streams": args.streams,
-              "gop_per_step": round(2 * nets.conv_macs(layers, batch, side, side) / 1e9, 1)}
+              "gop_per_step": round(2 * nets.conv_macs(layers, batch, side, side) / 1e9, 1),
+              # blocks whose residual branch is recomputed from int8 tensors inside their last launch: links per launch
+              "residual_chains": {n: len(c) for n, c in fused.chain_of.items()}}
     metric = ("int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
               else "int8 %s images/sec" % args.workload)
     if args.graph_only:
