@@ -27,6 +27,11 @@ INT8_PEAK_TOPS = 5000.0
 # Where the HBM traffic of the convolution launches was measured (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --graph-only`); the bench line itself reports no traffic figure: it cannot read a counter.
 TRAFFIC_PROFILE = {"resnet50": "profiles/igemm_i8_resnet50_bs64_hbm_traffic.md"}
+# rocprofv3 --kernel-trace --stats summaries of `bench.py --graph-only`, by (workload, parts of the batch)
+KERNEL_PROFILE = {("resnet50", 2): "profiles/resnet50_bs64_graph_two_streams_kernel_stats.md",
+                  ("resnet50", 1): "profiles/resnet50_bs64_graph_one_stream_kernel_stats.md",
+                  ("mobilenet_v2", 2): "profiles/mobilenet_v2_bs128_kernel_stats.md",
+                  ("darknet53_yolov3", 2): "profiles/darknet53_yolov3_bs16_kernel_stats.md"}
 
 
 def parse():
@@ -53,7 +58,8 @@ def parse():
                          "baseline): the mode to run under rocprofv3, whose kernel table then holds the timed region only")
     ap.add_argument("--probe", default="",
                     help="launch one kernel --probe-iters times and exit (for rocprofv3 counter runs): "
-                         "gemm:MxNxK (config-2 epilogue), quantize, layer:NAME (that layer's launch of the workload), copy")
+                         "gemm:MxNxK (config-2 epilogue), quantize, dequantize, absmax, frame, layer:NAME (that layer's "
+                         "launch of the workload), copy, mfma (what the int8 matrix cores sustain: prints its own rates)")
     ap.add_argument("--probe-iters", type=int, default=20)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy (reference dispatch for scaling rocprofv3 "
@@ -84,8 +90,10 @@ def layer_profile(fused, x, iters=20, only=None):
     trace = {}
     fused.forward(x, trace=trace)  # materialise every layer's quantized input once
     torch.cuda.synchronize()
+    fused_heads = set(h.name for h in fused.head_of.values()
+                      if fused.head_fuses(h, *trace[h.name]["qx"].shape[:3]))
     for l in fused.layers:
-        if l.kind not in ("conv", "fc") or l.name in fused._fused_away or (only and l.name != only):
+        if l.kind not in ("conv", "fc") or l.name in fused._fused_away or l.name in fused_heads or (only and l.name != only):
             continue
         lq = fused.q[l.name]
         qx = trace[l.name].get("qx_dev", trace[l.name]["qx"])  # the tensor the kernel reads
@@ -95,7 +103,22 @@ def layer_profile(fused, x, iters=20, only=None):
         ds = fused.shortcut_of.get(l.name) if l.kind == "conv" else None
         chain = fused.chain_of.get(l.name) if l.kind == "conv" else None
         extra_macs = extra_bytes = 0
-        if chain is not None:  # the residual chain back to the stage's shortcut is recomputed inside this launch
+        head = fused.head_of.get(l.name) if l.kind == "conv" else None
+        if head is not None and head.name in fused_heads:
+            # the 1x1 layer in front runs inside this launch: its input and filters are read, its output never stored
+            hq = fused.q[head.name]
+            hx = trace[head.name]["qx"]
+            resid = None
+            extra_macs = trace[head.name]["y"].numel() * hq.qw.shape[-1]
+            extra_bytes = hx.numel() + hq.qw.numel() - qx.numel()  # instead of this layer's own input tensor
+
+            def run(l=l, lq=lq, hq=hq, hx=hx, qd=qd, want_y=want_y):
+                return ops.qconv2d_head(hx, hq.qw, hq.exp2, hq.chan_div, hq.bias, lq.pos_x, lq.qw, lq.exp2, lq.chan_div,
+                                        lq.bias, fused.padding(l), [1, 1], [1, 1],
+                                        {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}[l.act], want_y, y_half,
+                                        qd[0] if qd else 0, qd[1] if qd else 0, 1.0, 0.1)
+            route = "mfma+head"
+        elif chain is not None:  # the residual chain back to the stage's shortcut is recomputed inside this launch
             resid = None
             n_pix = trace[l.name]["y"].numel() // trace[l.name]["y"].shape[-1]
             cq = [fused.q[c.name] for c in chain]
@@ -169,7 +192,7 @@ def plan_launches(fused, n, h, w):
             hi, wi = shape[l.src]
             ho, wo = (hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1
             shape[l.name] = (ho, wo)
-            if l.name in fused._fused_away:
+            if l.name in fused._fused_away or fused.head_fuses(l, n, hi, wi):
                 continue
             lq = fused.q[l.name]
             n_out = n * ho * wo * fused.cdev[l.name]
@@ -179,6 +202,11 @@ def plan_launches(fused, n, h, w):
             ds = fused.shortcut_of.get(l.name)
             chain = fused.chain_of.get(l.name)
             k_extra = 0
+            head = fused.head_of.get(l.name)
+            if head is not None and fused.head_fuses(head, n, hi, wi):
+                hq = fused.q[head.name]
+                macs += n * hi * wi * fused.cdev[head.name] * hq.qw.shape[-1]
+                b += n * hi * wi * (fused.cdev[head.src] - fused.cdev[l.src]) + hq.qw.numel()
             if chain is not None:
                 # every earlier link of the residual chain is recomputed inside this launch: its int8 input (the
                 # pixels the 1x1 taps touch) and its weights are read, its 2*K operations per output repeated
@@ -241,6 +269,24 @@ def plan_launches(fused, n, h, w):
     return rows
 
 
+def head_hw(fused, head, side):
+    """extent of the tensor the 1x1 layer `head` reads, for a network input of side x side"""
+    shape = {"input": (side, side)}
+    for l in fused.layers:
+        if l is head:
+            return shape[l.src]
+        if l.kind in ("conv", "maxpool"):
+            hi, wi = shape[l.src]
+            shape[l.name] = ((hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1)
+        elif l.kind == "upsample":
+            shape[l.name] = tuple(2 * v for v in shape[l.src])
+        elif l.kind == "concat":
+            shape[l.name] = shape[l.src[0]]
+        else:
+            shape[l.name] = (1, 1)
+    raise KeyError(head.name)
+
+
 def bound_of(ops, nbytes):
     """which roof the launch's algorithmic work sits under: the time its bytes need at the HBM peak against the
     time its operations need at the int8 matrix peak"""
@@ -266,6 +312,14 @@ def run_probe(args):
         for _ in range(it):
             ops.qlinear(a, b, exp2, div, bias, 1, True, True, False, 0, 0, 1.0)
         desc = "int8 GEMM %dx%dx%d, per-channel dequant + bias + ReLU, fp16 out" % (m, n, k)
+    elif what == "mfma":
+        print(json.dumps({"probe": what, "mfma_ceiling": mfma_ceiling(seconds=2.0)}))
+        return
+    elif what in ("dequantize", "absmax", "frame"):
+        fn, nbytes, desc = streaming_cases()[{"dequantize": "dequantize_i8_to_f32", "absmax": "quantize_param_f32",
+                                              "frame": "quantize_frame"}[what]]
+        for _ in range(it):
+            fn()
     elif what == "quantize":
         n = 64 * 256 * 56 * 56
         xs = [torch.randn(n, device="cuda") for _ in range(6)]
@@ -273,12 +327,11 @@ def run_probe(args):
             ops.quantize(xs[i % 6], 8, -5, 1.0)
         desc = "quantize fp32 -> int8, %d elements, 6 rotating inputs" % n
     elif what.startswith("layer:"):
-        from catch_amd import _native
         fused, xg, _ = build_workload(args)
         parts = list(xg.chunk(args.streams))
-        _native.kernel_lib().catchq_set_launch_sharing(args.streams)
+        ops.set_launch_sharing(args.streams)
         rows = layer_profile(fused, parts[0], iters=it, only=what[6:])
-        _native.kernel_lib().catchq_set_launch_sharing(1)
+        ops.set_launch_sharing(1)
         desc = "%s of %s, %d images: %.2f us, %.1f GB/s, %.1f TOPS" % (
             what[6:], args.workload, parts[0].shape[0], rows[0]["t"] * 1e6, rows[0]["bytes"] / rows[0]["t"] / 1e9,
             rows[0]["ops"] / rows[0]["t"] / 1e12)
@@ -286,6 +339,71 @@ def run_probe(args):
         sys.exit("unknown --probe " + what)
     torch.cuda.synchronize()
     print(json.dumps({"probe": what, "iters": it, "what": desc}))
+
+
+def mfma_ceiling(seconds=1.0):
+    """The rate a register-resident loop of v_mfma_i32_32x32x32_i8 (no memory access, two waves per SIMD) sustains on
+    operands of three kinds; the device lowers its clock under high-toggle matrix work, so the rate depends on them."""
+    import ctypes
+    import torch
+    from catch_amd import _native
+    lib = _native.kernel_lib()
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    blocks, iters = 512, 20000
+    g = torch.Generator().manual_seed(1234)
+    kinds = {"zero_operands": torch.zeros(1 << 20, dtype=torch.int8),
+             "uniform_random_bytes": torch.randint(-128, 128, (1 << 20,), generator=g, dtype=torch.int8),
+             "normal_bytes_sigma_32": (torch.randn(1 << 20, generator=g) * 32).round().clamp(-128, 127).to(torch.int8)}
+    out = {}
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for name, host in kinds.items():
+        dev = host.cuda()
+
+        def run(n_it):
+            _native.check(lib.catchq_diag_mfma_i8_loop(ctypes.c_void_p(dev.data_ptr()), n_it, blocks,
+                                                       ctypes.c_void_p(sink.data_ptr()), stream), "mfma loop")
+        run(1000)
+        torch.cuda.synchronize()
+        total_s = total_ops = 0.0
+        while total_s < seconds:
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            run(iters)
+            e.record()
+            e.synchronize()
+            total_s += s.elapsed_time(e) * 1e-3
+            total_ops += blocks * 4.0 * iters * 4 * 65536
+        out[name] = {"tops": round(total_ops / total_s / 1e12, 1), "frac_of_peak": round(total_ops / total_s / 1e12 / INT8_PEAK_TOPS, 4)}
+    return out
+
+
+def streaming_cases():
+    """the streaming kernels beside quantize fp32 -> int8, each over inputs in rotation (6 buffers, so that no launch
+    finds its operands in the 256 MB last-level cache): name -> (launch, algorithmic bytes per launch, description)"""
+    import torch
+    ops = torch.ops.torch_mlu
+    n = 64 * 256 * 56 * 56  # one ResNet-50 stage-1 activation: 51.4 M elements
+    state = {"i": 0}
+
+    def rot(bufs):
+        state["i"] = (state["i"] + 1) % len(bufs)
+        return bufs[state["i"]]
+    cases = {}
+    q8 = [torch.randint(-128, 128, (n,), dtype=torch.int8, device="cuda") for _ in range(6)]
+    cases["dequantize_i8_to_f32"] = (lambda: ops.dequantize(rot(q8), -5, 1.7), 5 * n,
+                                     "int8 -> fp32, y = q * 2^-5 / 1.7, %d elements" % n)
+    x32 = [torch.randn(n, device="cuda") for _ in range(6)]
+    cases["quantize_param_f32"] = (lambda: ops.quantize_param(rot(x32), 8, 1), 4 * n,
+                                   "max-abs reduction + position and scale, fp32, %d elements (two launches)" % n)
+    cases["quantize_f32_to_i16"] = (lambda: ops.quantize(rot(x32), 16, -12, 1.0), 6 * n, "fp32 -> int16, %d elements" % n)
+    x16 = [t.half() for t in x32]
+    cases["quantize_f16_to_i8"] = (lambda: ops.quantize(rot(x16), 8, -5, 1.0), 3 * n, "fp16 -> int8, %d elements" % n)
+    imgs = [torch.randn(64, 3, 224, 224, device="cuda") for _ in range(12)]
+    cases["quantize_frame"] = (lambda: ops.quantize_nhwc_frame(rot(imgs), 8, -5, 4, 230, 231, 3, 3, 1.0),
+                               64 * 3 * 224 * 224 * 4 + 64 * 230 * 231 * 4,
+                               "network input 64x3x224x224 fp32 NCHW -> int8 NHWC (4 channels) inside the first layer's zero "
+                               "frame [64,230,231,4]")
+    return cases
 
 
 def gaussian_linear_operands(m, n, k):
@@ -386,7 +504,9 @@ def main():
               "global_batch": batch, "calibration_images": args.calib_images, "graph_streams": args.streams,
               "gop_per_step": round(2 * nets.conv_macs(layers, batch, side, side) / 1e9, 1),
               # blocks whose residual branch is recomputed from int8 tensors inside their last launch: links per launch
-              "residual_chains": {n: len(c) for n, c in fused.chain_of.items()}}
+              "residual_chains": {n: len(c) for n, c in fused.chain_of.items()},
+              # 3x3 layers whose launch also computes the 1x1 layer in front of them
+              "fused_heads": sorted(n for n, h in fused.head_of.items() if fused.head_fuses(h, batch // args.streams, *head_hw(fused, h, side)))}
     metric = ("int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
               else "int8 %s images/sec" % args.workload)
     if args.graph_only:
@@ -410,8 +530,7 @@ def main():
     # The launches measured are the ones the graph holds: with the batch in `streams` parts, every layer is
     # launched once per part, on that part's images.
     parts = list(xg.chunk(args.streams))
-    from catch_amd import _native
-    _native.kernel_lib().catchq_set_launch_sharing(args.streams)  # the tile shapes the graph's launches were given
+    torch.ops.torch_mlu.set_launch_sharing(args.streams)  # the tile shapes the graph's launches were given
     rows = layer_profile(fused, parts[0])
     # Launch durations in their real sequence: HIP events around every conv/fc launch of eager forward
     # passes on the stream the kernels run on (no graph: a captured launch cannot be bracketed; one part
@@ -423,7 +542,7 @@ def main():
         for part in parts:
             fused.forward(part, timers=t_)
     torch.cuda.synchronize()
-    _native.kernel_lib().catchq_set_launch_sharing(1)
+    torch.ops.torch_mlu.set_launch_sharing(1)
     # The part of a bracketed duration that is the bracket's, not the kernel's: a pair of events around one small
     # kernel reads T1, around two of them T2; T2 - T1 is one kernel (and the gap before it), so 2*T1 - T2 is what
     # does not grow with the kernels in between.  (An empty pair reads more, 5.1 us: the markers' own processing
@@ -473,6 +592,9 @@ def main():
                 "achieved": round(b_conv / t_conv / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(b_conv / t_conv / 1e9 / HBM_PEAK_GBS, 4),
                 "traffic": None, "traffic_profile": TRAFFIC_PROFILE.get(args.workload),
+                # the committed kernel trace of the same graph whose per-launch durations give the same fraction
+                "frac_profile": KERNEL_PROFILE.get((args.workload, args.streams)),
+                "frac_over_timed_step": round(b_conv / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(t_conv / max(n_parts * len(conv_rows), 1) * 1e6, 2),
                 "timing": "HIP events around each launch of eager forward passes over the parts, in sequence (%d passes), "
                           "minus the bracket's own share, 2*T(pair around one small kernel) - T(pair around two), "
@@ -516,6 +638,8 @@ def main():
 
     if not args.no_extras:
         result["extras"] = extras()
+        if args.workload == "resnet50":
+            result["extras"].update(other_networks())
         if args.workload == "resnet50" and not args.fractional_scale:  # the modules quantize in power-of-two steps
             result["extras"]["dropin_modules"] = dropin_flow(net, x, args.calib_images, out)
     if not args.no_cpu_baseline:
@@ -616,6 +740,50 @@ def extras():
                                           "hbm_frac": round(5 * n / t_w / 1e9 / HBM_PEAK_GBS, 4),
                                           "working_set": "one 206 MB input over and over (about the last-level cache's size)"}}
     del xs
+    # the other streaming kernels, cold
+    for name, (fn, nbytes, desc) in streaming_cases().items():
+        t = event_time(fn, 24, 6)
+        out[name] = {"us": round(t * 1e6, 1), "gbs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
+                     "what": desc, "working_set": "inputs in rotation (cold: nothing cached)"}
+    torch.cuda.empty_cache()
+    return out
+
+
+def other_networks(steps=20):
+    """the other two network configurations, each as its own fused plan replayed from a HIP graph (two parts of the
+    batch on parallel streams): throughput, algorithmic bytes and integer operations of one step, fractions of the roofs"""
+    import argparse as _ap
+    import torch
+    from catch_amd import nets
+    out = {}
+    for workload, key in (("mobilenet_v2", "mobilenet_v2_bs128"), ("darknet53_yolov3", "darknet53_yolov3_bs16")):
+        a = _ap.Namespace(workload=workload, batch=0, calib_images=8, fractional_scale=False, streams=2, chain_links=-1)
+        fused, xg, w_ = build_workload(a)
+        static_in, replay = fused.capture(xg, streams=a.streams)
+        static_in.copy_(xg)
+        for _ in range(5):
+            replay()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            o = replay()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / steps
+        for t in (o if isinstance(o, tuple) else (o,)):
+            assert torch.isfinite(t.float()).all()
+        launches = plan_launches(fused, w_["batch"] // a.streams, w_["side"], w_["side"])
+        nbytes = a.streams * sum(r["bytes"] for r in launches)
+        nops = 2 * nets.conv_macs(w_["layers"], w_["batch"], w_["side"], w_["side"])
+        mfma_ops = nops * (2 if w_["detector"] else 1)  # an int16 x int8 product is two int8 matrix-core passes
+        out[key] = {"images_per_s": round(w_["batch"] / (ms * 1e-3), 1), "ms_per_step": round(ms, 4), "steps": steps,
+                    "what": w_["what"], "algorithmic_bytes_per_step": nbytes, "gop_per_step": round(nops / 1e9, 1),
+                    "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                    "tops": round(nops / (ms * 1e-3) / 1e12, 1),
+                    "mfma_frac": round(mfma_ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4)}
+        del fused, static_in, replay, xg, w_
+        torch.cuda.empty_cache()
     return out
 
 

@@ -22,7 +22,13 @@ class Epilogue(ctypes.Structure):
                 ("y_dtype", ctypes.c_int), ("acc_out", ctypes.c_void_p), ("q", ctypes.c_void_p),
                 ("q_bitwidth", ctypes.c_int), ("q_position", ctypes.c_int), ("q_scale", ctypes.c_float),
                 ("act_slope", ctypes.c_float), ("resid_after_act", ctypes.c_int),
-                ("exp2_dev", ctypes.c_void_p * 2)]
+                ("exp2_dev", ctypes.c_void_p * 2), ("half_steps", ctypes.c_int), ("sharing", ctypes.c_int)]
+
+
+class PointwiseHead(ctypes.Structure):
+    """struct catchq_pointwise_head"""
+    _fields_ = [("w", ctypes.c_void_p), ("ci", ctypes.c_int), ("exp2", ctypes.c_int), ("chan_div", ctypes.c_void_p),
+                ("chan_rcp", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("q_position", ctypes.c_int)]
 
 
 class ConvDesc(ctypes.Structure):
@@ -50,7 +56,6 @@ class ChainLink(ctypes.Structure):
 _I, _I64, _F, _P, _SZ = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 SIGNATURES = {
     "catchq_version": (_I, []),
-    "catchq_set_launch_sharing": (_I, [_I]),
     "catchq_status_string": (ctypes.c_char_p, [_I]),
     "catchq_pos_from_scale": (_I, [_I, _F, ctypes.POINTER(_I)]),
     "catchq_quant_params": (_I, [_I, _F, ctypes.POINTER(_I), ctypes.POINTER(_F), ctypes.POINTER(_F)]),
@@ -76,11 +81,16 @@ SIGNATURES = {
     "catchq_quantize_conv2d_nhwc": (_I, [_P, _I, _P, _I, _P, _I, _P, _I, ctypes.POINTER(ConvDesc), _P, _P, _I, _P, _SZ, _P]),
     "catchq_conv2d_shortcut_workspace_size": (_I, [_I, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Shortcut),
                                                    ctypes.POINTER(_SZ)]),
-    "catchq_conv1x1_chain_nhwc": (_I, [ctypes.POINTER(ChainLink), _I, _I, _I, _I, _I, _P, _P, _I, _P]),
+    "catchq_conv1x1_chain_nhwc": (_I, [ctypes.POINTER(ChainLink), _I, _I, _I, _I, _I, _P, _P, _I, _I, _P]),
     "catchq_conv2d_shortcut_nhwc": (_I, [_P, _I, _P, _I, ctypes.POINTER(ConvDesc), ctypes.POINTER(Epilogue),
                                          ctypes.POINTER(Shortcut), _P, _SZ, _P]),
+    "catchq_conv1x1_conv3x3_workspace_size": (_I, [ctypes.POINTER(PointwiseHead), ctypes.POINTER(ConvDesc),
+                                                   ctypes.POINTER(Epilogue), ctypes.POINTER(_SZ)]),
+    "catchq_conv1x1_conv3x3_nhwc": (_I, [_P, ctypes.POINTER(PointwiseHead), _P, ctypes.POINTER(ConvDesc),
+                                         ctypes.POINTER(Epilogue), _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
+    "catchq_diag_mfma_i8_loop": (_I, [_P, _I, _I, _P, _P]),
 }
 
 _BUILD_HINT = "build it with `python catch_amd/build.py` (hipcc cross-compiles gfx950 without a GPU)"

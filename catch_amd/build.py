@@ -19,7 +19,7 @@ INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
-KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "igemm_i8_dma_gemm.hip", "igemm_i8_dma_conv.hip", "igemm_i8_dual.hip", "igemm_i8_chain.hip", "conv3x3_halo_i8.hip", "igemm_a16_dma.hip", "pw_i8.hip", "dwconv_i8.hip", "pool.hip", "capi.hip",
+KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "igemm_i8_dma_gemm.hip", "igemm_i8_dma_conv.hip", "igemm_i8_dual.hip", "igemm_i8_chain.hip", "conv3x3_halo_i8.hip", "igemm_a16_dma.hip", "pw_i8.hip", "dwconv_i8.hip", "pool.hip", "diag.hip", "capi.hip",
                   "host_math.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from the fp32 epilogue math.
@@ -81,17 +81,8 @@ def build_torch_ext(verbose=False):
     return out
 
 
-def build_probes(verbose=False):
-    """stand-alone measurement programs (catch_amd/lib/probe_mfma: what the matrix cores sustain on this device)"""
-    out = os.path.join(LIBDIR, "probe_mfma")
-    o = _run([HIPCC, "--offload-arch=gfx950", "-O3", "-o", out, os.path.join(CSRC, "probe_mfma.hip")])
-    if verbose and o.strip():
-        print(o)
-    return out
-
-
 def build_all(verbose=False):
-    return build_kernels(verbose), build_torch_ext(verbose), build_probes(verbose)
+    return build_kernels(verbose), build_torch_ext(verbose)
 
 
 if __name__ == "__main__":
@@ -100,5 +91,3 @@ if __name__ == "__main__":
         print(build_kernels(True))
     if which in ("torch", "all"):
         print(build_torch_ext(True))
-    if which in ("probes", "all"):
-        print(build_probes(True))

@@ -54,9 +54,6 @@ class MLUConvNd(torch.nn.Module, MLUModel):
                 self.bias.copy_(ref.bias)
 
     # -- calibration ----------------------------------------------------------------------------
-    def _observer_forward_hook(self, module, inputs, output):
-        return self.observer(*inputs)
-
     def _float_forward(self, x):
         if self.padding_mode == "circular":
             pads = []
@@ -75,49 +72,16 @@ class MLUConvNd(torch.nn.Module, MLUModel):
         return op(input, self.weight, self.bias, list(self.padding), list(self.stride), list(self.dilation),
                   self.groups, self.scale, self.quantized_mode)
 
-    # -- checkpoint format: weight, bias, scale, quantized_mode [, quantized_by_channel,
-    #    scale_weight_per_channel, input_mean, input_std] (conv.py:77-131) ---------------------------
+    # -- checkpoint format (conv.py:77-131): the keys are written and read by MLUModel ------------------------
     def _save_to_state_dict(self, destination, prefix, keep_vars):
         super()._save_to_state_dict(destination, prefix, keep_vars)
-        if self.weight is not None:
-            destination[prefix + "weight"] = self.weight
-        if self.bias is not None:
-            destination[prefix + "bias"] = self.bias
-        if not self.quant:
-            return
-        weight_observer = self.qconfig.weight()
-        weight_observer(self.weight)
-        weight_observer.calculate_qparams()
-        self.observer.calculate_qparams()
-        self.set_quantized_mode(torch.Tensor([2 if self.observer.dtype == "int16" else 1]))
-        if weight_observer._get_name() == "MLUPerChannelMinMaxObserver":
-            destination[prefix + "quantized_by_channel"] = torch.tensor([1])
-            destination[prefix + "scale_weight_per_channel"] = torch.tensor(weight_observer.scales)
-            self.set_scale(torch.tensor([self.observer.scale, 0.0]))
-        else:
-            self.set_scale(torch.tensor([self.observer.scale, weight_observer.scale]))
-        destination[prefix + "scale"] = self.scale.data
-        destination[prefix + "quantized_mode"] = self.quantized_mode.data
-        if self.input_std is not None:
-            destination[prefix + "input_mean"] = self.input_mean.data.mul(255)
-            destination[prefix + "input_std"] = self.input_std.data.mul(255)
+        self.save_qparams(destination, prefix)
 
     def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
                               error_msgs):
         super()._load_from_state_dict(state_dict, prefix, local_metadata, False, missing_keys, unexpected_keys,
                                       error_msgs)
-        if prefix + "scale" in state_dict:
-            self.set_scale(state_dict[prefix + "scale"], state_dict.get(prefix + "scale_weight_per_channel"))
-        if prefix + "quantized_mode" in state_dict:
-            self.set_quantized_mode(state_dict[prefix + "quantized_mode"],
-                                    state_dict.get(prefix + "quantized_by_channel"))
-        if prefix + "input_mean" in state_dict and prefix + "input_std" in state_dict:
-            self.set_mean_std(state_dict[prefix + "input_mean"], state_dict[prefix + "input_std"])
-        if state_dict.get(prefix + "bias") is None:
-            self.set_bias_with_zeros(self.out_channels)
-        for lst in (missing_keys, unexpected_keys):  # the quantization keys are optional both ways
-            for k in [k for k in lst if k.startswith(prefix)]:
-                lst.remove(k)
+        self.load_qparams(state_dict, prefix, self.out_channels, missing_keys, unexpected_keys)
 
     def extra_repr(self):
         return ("{in_channels}, {out_channels}, kernel_size={kernel_size}, stride={stride}, padding={padding}, "
@@ -125,18 +89,9 @@ class MLUConvNd(torch.nn.Module, MLUModel):
                ", scale={}, quantized_mode={}".format(self.scale, self.quantized_mode)
 
     def _apply(self, fn, recurse=True):
-        # The reference has no override: .half() turns the q-params into half tensors, and its per-channel
-        # derivation then runs in half as well.  That is followed for int8, where half holds every number of
-        # that derivation.  int16 q-params stay fp32: 32767 / absmax exceeds the largest half for absmax < 0.5,
-        # and half holds neither 32767 nor the integers above 2048.
         kept = None if self.scale is None else self.scale.detach().clone()
         super()._apply(fn)
-        if kept is not None and self.scale is not None and self.scale.dtype != torch.float32:
-            int8 = self.quantized_mode is not None and self.quantized_mode.numel() == 1 \
-                and int(self.quantized_mode.flatten()[0]) in (1, 3)
-            if not int8 or not bool(torch.isfinite(self.scale.float()).all()):
-                self.scale = Parameter(kept.detach().to(device=self.scale.device, dtype=torch.float32),
-                                       requires_grad=False)
+        self.keep_wide_scale(kept)
         return self
 
     def _get_name(self):
@@ -151,7 +106,6 @@ class MLUConvNd(torch.nn.Module, MLUModel):
                 mod.groups, mod.bias is not None, mod.padding_mode)
         q.set_weight_bias(mod.weight, mod.bias)
         if gen_quant:
-            q.quant = True
             if cls is MLUConv3d:
                 assert mod.qconfig.activation().qscheme["per_channel"] is False, \
                     "MLUConv3d does not support per_channel quantization, set per_channel False in qconfig!"
@@ -169,9 +123,7 @@ class MLUConvNd(torch.nn.Module, MLUModel):
                         logging.warning("firstconv with default mean [0,0,0] and std [1,1,1]: check that this is intended")
                     q.set_mean_std(torch.Tensor(conf["mean"]), torch.Tensor(conf["std"]))
                 MLUConv2d.is_first_layer = False
-            q.qconfig = mod.qconfig
-            q.observer = q.qconfig.activation()
-            q.register_forward_hook(q._observer_forward_hook)
+            q.start_calibration(mod.qconfig)
         return q
 
 

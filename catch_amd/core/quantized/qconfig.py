@@ -1,19 +1,9 @@
 """(activation observer factory, weight observer factory) pairs.
 Counterpart of torch_mlu/core/quantized/qconfig.py."""
-from collections import namedtuple
-
-import torch.nn as nn
+from torch.quantization import QConfig  # the pair type with its "pass a class, not an instance" check
 
 from .observer import (NoopObserver, default_mlu_observer, mlu_activation_observer, mlu_norm_observer,
                        mlu_weight_observer, mlu_weight_per_channel_observer)
-
-
-class QConfig(namedtuple("QConfig", ["activation", "weight"])):
-    def __new__(cls, activation, weight):
-        if isinstance(activation, nn.Module) or isinstance(weight, nn.Module):
-            raise ValueError("QConfig received observer instance, please pass observer class instead. "
-                             "Use MyObserver.with_args(x=1) to override arguments to constructor if needed")
-        return super().__new__(cls, activation, weight)
 
 
 default_mlu_qconfig = QConfig(activation=default_mlu_observer, weight=default_mlu_observer)

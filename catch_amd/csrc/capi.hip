@@ -32,7 +32,11 @@ struct ChainLinkDev {  // igemm_i8_chain.hip
   const float *chan_div, *chan_rcp, *bias;
 };
 int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int Wo, int Co, float *y, int8_t *q,
-                     int q_position, hipStream_t s);
+                     int q_position, int sharing, hipStream_t s);
+bool conv2d_head_halo_i8_ok(int N, int H, int W, int K1, int Cm, int Co);
+int conv2d_head_halo_i8(const void *x, int K1, const void *w1, const float *div1, const float *rcp1, const float *bias1,
+                        int exp2_1, int q_position1, const void *w, int N, int H, int W, int Cm, int Co, const EpiDev &e,
+                        hipStream_t s);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -257,8 +261,8 @@ CATCHQ_API int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void
 }
 
 CATCHQ_API int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int nlinks, int n, int ho, int wo, int co,
-                                         float *y, void *q, int q_position, catchq_stream_t stream) {
-  if (!links || n < 0 || ho <= 0 || wo <= 0 || co <= 0 || (!y && !q)) return CATCHQ_ERR_ARG;
+                                         float *y, void *q, int q_position, int sharing, catchq_stream_t stream) {
+  if (!links || n < 0 || ho <= 0 || wo <= 0 || co <= 0 || (!y && !q) || sharing < 0) return CATCHQ_ERR_ARG;
   if (nlinks < 2 || nlinks > CATCHQ_CHAIN_MAX_LINKS) return CATCHQ_ERR_UNSUPPORTED;
   if (q && (q_position < -126 || q_position > 126)) return CATCHQ_ERR_ARG;
   ChainLinkDev dev[CATCHQ_CHAIN_MAX_LINKS];
@@ -270,6 +274,9 @@ CATCHQ_API int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int n
     if (n > 0 && (!l.x || !l.w)) return CATCHQ_ERR_ARG;
     const int64_t xb = (int64_t)n * l.in_h * l.in_w * l.ci, wb = (int64_t)co * l.ci;
     if (xb >= (1ll << 31) || wb >= (1ll << 31) || l.ci % 64 != 0) return CATCHQ_ERR_UNSUPPORTED;
+    // element strides of the taps, in 64 bits first: a huge stride on a one-pixel output grid passes the size checks
+    const int64_t row_stride = (int64_t)l.stride * l.in_w * l.ci, pix_stride = (int64_t)l.stride * l.ci;
+    if (row_stride >= (1ll << 31) || pix_stride >= (1ll << 31)) return CATCHQ_ERR_UNSUPPORTED;
     if (!l.chan_div || !l.chan_rcp || !l.bias || l.exp2 < -64 || l.exp2 > 64) return CATCHQ_ERR_UNSUPPORTED;
     dev[i].x = (const int8_t *)l.x;
     dev[i].w = (const int8_t *)l.w;
@@ -277,8 +284,8 @@ CATCHQ_API int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int n
     dev[i].w_bytes = (unsigned)wb;
     dev[i].K = l.ci;
     dev[i].img_stride = (unsigned)(l.in_h * l.in_w * l.ci);
-    dev[i].row_stride = (unsigned)(l.stride * l.in_w * l.ci);
-    dev[i].pix_stride = (unsigned)(l.stride * l.ci);
+    dev[i].row_stride = (unsigned)row_stride;
+    dev[i].pix_stride = (unsigned)pix_stride;
     dev[i].dense = (l.stride == 1 && l.in_h == ho && l.in_w == wo) ? 1 : 0;
     dev[i].k_shift = -1;
     dev[i].exp2 = l.exp2;
@@ -287,8 +294,77 @@ CATCHQ_API int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int n
     dev[i].bias = l.bias;
   }
   if (n == 0) return CATCHQ_OK;
-  const int st = conv1x1_chain_i8(dev, nlinks, n, ho, wo, co, y, (int8_t *)q, q_position, as_stream(stream));
+  const int st = conv1x1_chain_i8(dev, nlinks, n, ho, wo, co, y, (int8_t *)q, q_position, sharing, as_stream(stream));
   return st < 0 ? CATCHQ_ERR_UNSUPPORTED : st;
+}
+
+// shapes the head kernel serves (pointer alignment and the epilogue variant are checked at the call)
+static bool head_fusable(const catchq_pointwise_head_t *hd, const catchq_conv_desc_t *d, const catchq_epilogue_t *e) {
+  return d->groups == 1 && d->kh == 3 && d->kw == 3 && d->pad_h == 1 && d->pad_w == 1 && d->stride_h == 1 && d->stride_w == 1 &&
+         d->dil_h == 1 && d->dil_w == 1 && hd->chan_div && hd->chan_rcp && hd->bias && hd->exp2 >= -64 && hd->exp2 <= 64 &&
+         !e->exp2_dev[0] && !e->exp2_dev[1] && conv2d_head_halo_i8_ok(d->n, d->h, d->w, hd->ci, d->ci, d->co);
+}
+
+static int check_head(const catchq_pointwise_head_t *hd, const catchq_conv_desc_t *d) {
+  if (!hd) return CATCHQ_ERR_ARG;
+  if (hd->ci <= 0) return CATCHQ_ERR_SHAPE;
+  if (hd->exp2 < -126 || hd->exp2 > 126 || hd->q_position < -126 || hd->q_position > 126) return CATCHQ_ERR_ARG;
+  if (d->groups != 1) return CATCHQ_ERR_UNSUPPORTED;
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_conv1x1_conv3x3_workspace_size(const catchq_pointwise_head_t *head, const catchq_conv_desc_t *desc,
+                                                     const catchq_epilogue_t *epilogue, size_t *bytes) {
+  int ho, wo;
+  int st = check_conv(desc, &ho, &wo);
+  if (st != CATCHQ_OK) return st;
+  if (!bytes) return CATCHQ_ERR_ARG;
+  st = check_epi(epilogue);
+  if (st != CATCHQ_OK) return st;
+  st = check_head(head, desc);
+  if (st != CATCHQ_OK) return st;
+  *bytes = head_fusable(head, desc, epilogue) ? 0 : (size_t)desc->n * desc->h * desc->w * desc->ci;
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_conv1x1_conv3x3_nhwc(const void *x, const catchq_pointwise_head_t *head, const void *w,
+                                           const catchq_conv_desc_t *desc, const catchq_epilogue_t *epilogue,
+                                           void *workspace, size_t workspace_bytes, catchq_stream_t stream) {
+  int ho, wo;
+  int st = check_conv(desc, &ho, &wo);
+  if (st != CATCHQ_OK) return st;
+  st = check_epi(epilogue);
+  if (st != CATCHQ_OK) return st;
+  st = check_head(head, desc);
+  if (st != CATCHQ_OK) return st;
+  if (desc->n == 0) return CATCHQ_OK;
+  if (!x || !w || !head->w) return CATCHQ_ERR_ARG;
+  const catchq_conv_desc_t &d = *desc;
+  if (head_fusable(head, desc, epilogue)) {
+    const EpiDev e = make_epi(epilogue, (int64_t)d.n * ho * wo * d.co);
+    const int st2 = conv2d_head_halo_i8(x, head->ci, head->w, head->chan_div, head->chan_rcp, head->bias, head->exp2,
+                                        head->q_position, w, d.n, d.h, d.w, d.ci, d.co, e, as_stream(stream));
+    if (st2 >= 0) return st2;
+  }
+  // two launches: the head's int8 output goes through the workspace
+  const size_t need = (size_t)d.n * d.h * d.w * d.ci;
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return CATCHQ_ERR_ARG;
+  catchq_conv_desc_t dh = {d.n, d.h, d.w, head->ci, d.ci, 1, 1, 0, 0, 1, 1, 1, 1, 1};
+  catchq_epilogue_t eh;
+  memset(&eh, 0, sizeof(eh));
+  eh.exp2 = head->exp2;
+  eh.chan_div = head->chan_div;
+  eh.chan_rcp = head->chan_rcp;
+  eh.bias = head->bias;
+  eh.act = CATCHQ_ACT_RELU;
+  eh.q = workspace;
+  eh.q_bitwidth = 8;
+  eh.q_position = head->q_position;
+  eh.q_scale = 1.0f;
+  eh.sharing = epilogue->sharing;
+  st = catchq_conv2d_nhwc(x, 8, head->w, 8, &dh, &eh, stream);
+  if (st != CATCHQ_OK) return st;
+  return catchq_conv2d_nhwc(workspace, 8, w, 8, desc, epilogue, stream);
 }
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }

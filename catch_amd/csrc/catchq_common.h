@@ -23,8 +23,11 @@ inline hipStream_t as_stream(catchq_stream_t s) { return reinterpret_cast<hipStr
 inline int launch_status() { return hipGetLastError() == hipSuccess ? CATCHQ_OK : CATCHQ_ERR_LAUNCH; }
 
 // compute units one launch should plan its tile shapes for: the device's 256, divided by the number of
-// launches the caller says share the device (catchq_set_launch_sharing)
-int planned_cus();
+// launches the caller says share the device (catchq_epilogue_t::sharing)
+inline int planned_cus(int sharing) {
+  const int cus = 256 / (sharing < 1 ? 1 : sharing);
+  return cus < 1 ? 1 : cus;
+}
 
 // Allow `kern` more than the default 64 KiB of dynamic LDS: needed once per kernel and device.  `raised` is the
 // call site's own flag array (one per kernel instance); setting the attribute twice is harmless, so relaxed
@@ -43,7 +46,8 @@ inline int raise_lds_limit(const void *kern, int bytes, std::atomic<bool> (&rais
 }
 
 // Tuning switches read from the environment exist only in builds made with -DCATCHQ_TUNING (A/B timing of tile
-// shapes and load paths); the shipped library reads no environment variable.
+// shapes and load paths); the shipped kernel library reads no environment variable.  (The PyTorch extension on top
+// of it has one run-time switch, CATCHQ_WEIGHT_CACHE=0, which turns its prepared-weight cache off.)
 inline const char *tuning_env(const char *name) {
 #ifdef CATCHQ_TUNING
   return std::getenv(name);
@@ -131,6 +135,8 @@ struct EpiDev {
   // the floating output / the residual is too large to stay cached until it is next used: written / read with
   // the non-temporal hint so that it does not push the operands and the int8 output out of the caches
   int y_stream, resid_stream;
+  int cus;  // compute units the launch plans its tiles for (planned_cus of the caller's hint)
+  int half_steps;  // fp16 output: round to binary16 after the scaling, the division and the bias (generic epilogues only)
 };
 
 // The second operand pair of a two-branch launch: the projection shortcut of a residual block.  Its
@@ -145,13 +151,16 @@ struct ShortcutDev {
 inline EpiDev make_epi(const catchq_epilogue_t *e, int64_t out_elems = 0) {
   EpiDev d;
   // a quarter of the 256 MB last-level cache, of this launch's share of it
-  const int64_t kStreamBytes = (64ll << 20) * planned_cus() / 256;
+  d.cus = planned_cus(e->sharing);
+  const int64_t kStreamBytes = (64ll << 20) * d.cus / 256;
   d.y_stream = (e->y && out_elems * (e->y_dtype == CATCHQ_F16 ? 2 : 4) >= kStreamBytes) ? 1 : 0;
   d.resid_stream = (e->resid && out_elems * 4 >= kStreamBytes) ? 1 : 0;
   d.exp2 = e->exp2;
   d.chan_div = e->chan_div;
   const bool dev_exp = e->exp2_dev[0] || e->exp2_dev[1];
-  d.chan_rcp = (e->chan_div && e->chan_rcp && !dev_exp && e->exp2 >= -64 && e->exp2 <= 64) ? e->chan_rcp : nullptr;
+  d.half_steps = (e->half_steps && e->y && e->y_dtype == CATCHQ_F16) ? 1 : 0;
+  // (the reciprocal form folds the power of two into the division: not with a rounding between the two)
+  d.chan_rcp = (e->chan_div && e->chan_rcp && !dev_exp && !d.half_steps && e->exp2 >= -64 && e->exp2 <= 64) ? e->chan_rcp : nullptr;
   d.bias = e->bias;
   d.resid = e->resid;
   d.act = e->act;
@@ -177,6 +186,7 @@ inline int check_epi(const catchq_epilogue_t *e) {
   if (e->act < CATCHQ_ACT_NONE || e->act > CATCHQ_ACT_LEAKY) return CATCHQ_ERR_ARG;
   if (e->exp2 < -126 || e->exp2 > 126) return CATCHQ_ERR_ARG;
   if (e->q && (e->q_position < -126 || e->q_position > 126)) return CATCHQ_ERR_ARG;
+  if (e->sharing < 0) return CATCHQ_ERR_ARG;
   return CATCHQ_OK;
 }
 
@@ -192,10 +202,19 @@ __device__ __forceinline__ void resolve_exp2(EpiDev &e) {
 }
 
 // value after dequant / bias / residual / activation; facc = float(acc) (one RNE conversion)
+__device__ __forceinline__ float round_f16(float v) { return __half2float(__float2half_rn(v)); }
+
 __device__ __forceinline__ float epi_value(float facc, int64_t idx, int c, const EpiDev &e) {
   float v = __builtin_ldexpf(facc, e.exp2);
-  if (e.chan_div) v = v / e.chan_div[c];
-  if (e.bias) v = v + e.bias[c];
+  if (e.half_steps) v = round_f16(v);
+  if (e.chan_div) {
+    v = v / e.chan_div[c];
+    if (e.half_steps) v = round_f16(v);
+  }
+  if (e.bias) {
+    v = v + e.bias[c];
+    if (e.half_steps) v = round_f16(v);
+  }
   if (e.resid && !e.resid_after) v = v + e.resid[idx];
   if (e.act == CATCHQ_ACT_LEAKY) v = (v > 0.0f) ? v : v * e.act_slope;
   else if (e.act >= CATCHQ_ACT_RELU) v = (v > 0.0f) ? v : 0.0f;

@@ -19,6 +19,16 @@
 //                K: weights beyond K read as zeros, the patch address of a tap >= 9 is clamped
 //
 // The integer sums are those of any other route (exact), the epilogue is the shared one.
+//
+// With a head (HEAD = true) the patch is not loaded but computed: the block input goes through the 1x1
+// convolution + ReLU + int8 requantization that precedes the 3x3 layer in a bottleneck block, for the band's rows
+// plus the one-pixel halo, and the requantized values are written straight into the LDS patch; that convolution's
+// output never reaches memory and its launch disappears.  A lane loads the A fragments of its pixels (rows of K1
+// contiguous bytes) straight from global memory, the 1x1 filters sit in the ring slot that the 3x3 weights need
+// last, and the two operands are swapped in the MFMA so that a lane ends up with four consecutive channels of one
+// pixel: one dword of the patch.  Halo rows are computed by the bands on both sides: (TR + 2) / TR of a cheap
+// convolution.  Pixels outside the image are zeros in the patch (the 3x3 layer's padding is applied to the head's
+// output, not to its input).
 #include <type_traits>
 
 #include "igemm_i8_dma.inc"
@@ -39,6 +49,15 @@ struct HaloParams {
   int tiles_n, nblocks;
   int64_t M;             // N * H * W
   unsigned x_bytes, w_bytes;
+};
+
+// The 1x1 convolution + ReLU + int8 requantization in front of the 3x3 layer (HEAD kernels):
+//   q1[p][c] = sat(rne(relu(float(acc1) * 2^exp2 / div[c] + bias[c]) * 2^-q_position)),  acc1 = sum_k x[p][k] * w[c][k]
+struct HeadDev {
+  const int8_t *w;                 // [CI][K1]
+  const float *div, *rcp, *bias;   // [CI] each; rcp = correctly rounded reciprocals of div
+  int exp2, q_neg_pos;
+  unsigned w_bytes;
 };
 
 // f(integral_constant<int, G>) for G = 0 .. N-1, expanded at compile time (a #pragma unroll over this many large
@@ -68,10 +87,14 @@ __device__ __forceinline__ unsigned halo_key(unsigned prow, unsigned pcol, unsig
   return (prow >> SH) * wo_count + (pcol >> SH);
 }
 
-template <int CI, int TN, int TMW, int S, int EPI, int NW = 4>
+// K1 = 0: the patch is loaded from X [N, Hi, Wi, CI]; K1 > 0: X is the head's input [N, H, W, K1] and the patch
+// is computed (stride 1, band mode, one block over all output channels, four waves, TMA = sub-tiles of the
+// head's rows per wave)
+template <int CI, int TN, int TMW, int S, int EPI, int NW = 4, int K1 = 0, int TMA = 1>
 __global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
-                                                          HaloParams hp, EpiDev e) {
+                                                          HaloParams hp, EpiDev e, HeadDev hd) {
   resolve_exp2(e);
+  constexpr bool HEAD = K1 > 0;
   constexpr int CH = CI / 16;         // 16-byte chunks per pixel
   constexpr int LOG_CI = CI == 64 ? 6 : CI == 128 ? 7 : CI == 256 ? 8 : 9;
   constexpr int BN = 32 * TN;
@@ -117,7 +140,7 @@ __global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__r
   constexpr unsigned OOB = 0x80000000u;
 
   // ---- the input patch: every 16-byte chunk once ------------------------------------------------------------
-  {
+  if constexpr (!HEAD) {
     const int npix = hp.PR * hp.PC;
     const int ninstr = patch_bytes / 1024;
     constexpr int PPI = 64 / CH > 0 ? 64 / CH : 1;  // pixels per DMA instruction (CH <= 32)
@@ -165,14 +188,135 @@ __global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__r
                                                0, 0);
     }
   };
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)lds_dyn;
+  if constexpr (!HEAD) {
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) issue_weights(s, s * B_STAGE);
+    for (int s = 0; s < STAGES - 1; ++s) issue_weights(s, s * B_STAGE);
+  } else {
+    // ---- the head: patch = requantized ReLU of the 1x1 convolution of the block input ------------------------------
+    static_assert(S == 1 && NW == 4 && (K1 == 64 || K1 == 256) && CI * K1 <= B_STAGE, "head shapes");
+    constexpr int KS1 = K1 / 32;   // MFMA K steps of the head
+    constexpr int TN1 = CI / 32;   // its output channel tiles
+    constexpr int CHW = K1 / 16;   // 16-byte chunks per filter row
+    constexpr int NI1 = CI * K1 / 1024 / NW;  // filter DMA instructions per wave
+    static_assert(CI * K1 / 1024 % NW == 0, "the head's filter rows must split evenly over the waves");
+    const unsigned w1_slot = (unsigned)patch_bytes + (STAGES - 1) * B_STAGE;  // the ring slot filled last
+    const unsigned const_off = (unsigned)patch_bytes + STAGES * B_STAGE;      // div', rcp', bias: CI floats each
+    {  // filters -> LDS, chunk index XOR-ed with a row key so that the fragment reads of 16 rows spread over the banks
+      const __amdgpu_buffer_rsrc_t rsrc_w1 = __builtin_amdgcn_make_buffer_rsrc((void *)hd.w, 0, (int)hd.w_bytes, 0x00020000);
+#pragma unroll
+      for (int t = 0; t < NI1; ++t) {
+        const int b = wave * NI1 + t;
+        unsigned row, phys, key;
+        if constexpr (CHW >= 16) { row = (unsigned)b * (64 / CHW) + ((unsigned)lane / CHW); phys = (unsigned)lane % CHW; key = row & 15u; }
+        else { row = (unsigned)b * 16 + ((unsigned)lane >> 2); phys = (unsigned)lane & 3u; key = (row >> 2) & 3u; }
+        const unsigned voff = row * (unsigned)K1 + ((phys ^ key) << 4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w1, (lds_ptr_t)(lds_dyn + w1_slot + b * 1024), 16, (int)voff, 0, 0, 0);
+      }
+    }
+    // the rows of the head: patch rows 0 .. PR-1 of W pixels each (the patch's border columns are zeros), i.e. the
+    // contiguous input pixels base_pix .. base_pix + PR * W; rows above / below the image are not computed
+    const int m_a = hp.PR * hp.W;
+    const int row_lo = (ho0 == 0) ? hp.W : 0;
+    const int rows_in = hp.H - ho0 + 1 < hp.PR ? hp.H - ho0 + 1 : hp.PR;
+    const int row_hi = rows_in * hp.W;
+    const int base_pix = (img0 * hp.H + ho0 - 1) * hp.W;
+    v4i fa[TMA][KS1];
+    bool pvalid[TMA];
+#pragma unroll
+    for (int i = 0; i < TMA; ++i) {
+      const int r_a = (wave + NW * i) * 32 + frow;
+      pvalid[i] = r_a >= row_lo && r_a < row_hi;
+      const int8_t *src = X + (int64_t)(base_pix + r_a) * K1 + fhalf * 16;
+#pragma unroll
+      for (int ks = 0; ks < KS1; ++ks) {
+        fa[i][ks] = v4i{0, 0, 0, 0};
+        if (pvalid[i]) fa[i][ks] = *reinterpret_cast<const v4i *>(src + ks * 32);
+      }
+    }
+    // per-channel constants with the power of two folded in (as epi_lane_setup does), staged once per block
+    if (threadIdx.x < CI) {
+      const int c = threadIdx.x;
+      float *cst = reinterpret_cast<float *>(lds_dyn + const_off);
+      cst[c] = __builtin_ldexpf(hd.div[c], -hd.exp2);
+      cst[CI + c] = __builtin_ldexpf(hd.rcp[c], hd.exp2);
+      cst[2 * CI + c] = hd.bias[c];
+    }
+    // the patch's border columns
+    for (int t = threadIdx.x; t < hp.PR * 2 * CH; t += 64 * NW) {
+      const int pr = t / (2 * CH), rest = t - pr * (2 * CH);
+      const int pc = (rest < CH) ? 0 : hp.PC - 1;
+      *reinterpret_cast<v4i *>(lds_dyn + (pr * hp.PC + pc) * CI + (rest % CH) * 16) = v4i{0, 0, 0, 0};
+    }
+    CATCHQ_VMCNT(0);
+    __syncthreads();  // filters, constants and border columns are in place
+    // the 3x3 layer's first weight stages travel while the head is computed
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue_weights(s, s * B_STAGE);
+
+    // filter fragment of channel tile j, K step ks: row j*32 + frow, logical chunk 2*ks + fhalf
+    unsigned w1_addr[TN1];
+#pragma unroll
+    for (int j = 0; j < TN1; ++j) {
+      const unsigned n = (unsigned)(j * 32 + frow);
+      const unsigned key = (CHW >= 16) ? (n & 15u) : ((n >> 2) & 3u);
+      w1_addr[j] = lds_base + w1_slot + n * (unsigned)K1 + ((((unsigned)fhalf) ^ key) << 4);
+    }
+    const float q_hi = __builtin_ldexpf(127.0f, -hd.q_neg_pos), q_sc = __builtin_ldexpf(1.0f, hd.q_neg_pos);
+#pragma unroll
+    for (int i = 0; i < TMA; ++i) {
+      const int sub = wave + NW * i;
+      if (sub * 32 >= m_a) break;  // wave-uniform
+      v16i acc1[TN1];
+#pragma unroll
+      for (int j = 0; j < TN1; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc1[j][r] = 0;
+      // operands swapped: the 32x32 result has channels down the rows, so a lane holds channels
+      // 8g + 4*fhalf .. + 3 (g = 0 .. 3) of pixel frow
+#pragma unroll
+      for (int ks = 0; ks < KS1; ++ks) {
+        v4i fw[TN1];
+#pragma unroll
+        for (int j = 0; j < TN1; ++j) fw[j] = ds_read_b128<0>(w1_addr[j] ^ (unsigned)(ks << 5));
+#pragma unroll
+        for (int j = 0; j < TN1; ++j) lgkm_wait<0>(fw[j]);
+#pragma unroll
+        for (int j = 0; j < TN1; ++j) acc1[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[j], fa[i][ks], acc1[j], 0, 0, 0);
+      }
+      const int r_a = sub * 32 + frow;
+      const unsigned pr = (unsigned)r_a / (unsigned)hp.W, pc = (unsigned)r_a - pr * (unsigned)hp.W + 1u;
+      const unsigned pix_addr = lds_base + (pr * (unsigned)hp.PC + pc) * (unsigned)CI;
+      const unsigned sw = halo_swz<CH>(halo_key<1>(pr, pc, (unsigned)hp.W));
+#pragma unroll
+      for (int j = 0; j < TN1; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const unsigned c0 = (unsigned)(j * 32 + 8 * g + 4 * fhalf);
+          const unsigned caddr = lds_base + const_off + c0 * 4;
+          v4i dv = ds_read_b128<0>(caddr), rc = ds_read_b128<CI * 4>(caddr), bs = ds_read_b128<CI * 8>(caddr);
+          lgkm_wait<0>(dv, rc, bs);
+          unsigned b[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            float x = div_by_rcp((float)acc1[j][4 * g + t], __int_as_float(dv[t]), __int_as_float(rc[t])) + __int_as_float(bs[t]);
+            x = __builtin_amdgcn_fmed3f(x, 0.0f, q_hi);  // ReLU and the upper clamp; NaN -> 0
+            b[t] = __builtin_bit_cast(unsigned, __builtin_fmaf(x, q_sc, 12582912.0f));
+          }
+          const unsigned lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+          const unsigned hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+          const unsigned packed = pvalid[i] ? (lo | hi2) : 0u;
+          const unsigned dst = pix_addr + (((c0 >> 4) ^ sw) << 4) + (c0 & 15u);
+          if (r_a < m_a) asm volatile("ds_write_b32 %0, %1" ::"v"(dst), "v"(packed) : "memory");
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
 
   // ---- this lane's fragment addresses: one per sub-tile and filter tap ------------------------------------------
   // The A fragment of K step c (32 bytes: chunks 2c and 2c+1, this lane takes chunk 2c + fhalf) of a pixel sits at
   //   pixel * CI + (((2c + fhalf) ^ swz(pixel)) << 4)  =  [pixel * CI + ((fhalf ^ swz(pixel)) << 4)]  ^  (c << 5):
   // the bracket is fixed per (sub-tile, tap), the XOR mask is the same for every lane.
-  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)lds_dyn;
   unsigned a0[TMW][9];
 #pragma unroll
   for (int i = 0; i < TMW; ++i) {
@@ -281,14 +425,15 @@ __global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__r
   }
 }
 
-template <int CI, int TN, int TMW, int S, int EPI, int NW>
-static int launch_halo_epi(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s) {
-  auto kern = conv3x3_halo_kernel<CI, TN, TMW, S, EPI, NW>;
+template <int CI, int TN, int TMW, int S, int EPI, int NW, int K1 = 0, int TMA = 1>
+static int launch_halo_epi(const void *x, const void *w, const HaloParams &hp, const EpiDev &e, int lds_bytes, hipStream_t s,
+                           const HeadDev &hd = HeadDev{}) {
+  auto kern = conv3x3_halo_kernel<CI, TN, TMW, S, EPI, NW, K1, TMA>;
   if (lds_bytes > 64 * 1024) {
     static std::atomic<bool> raised[64];
     if (raise_lds_limit((const void *)kern, 160 * 1024, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
   }
-  kern<<<hp.nblocks, 64 * NW, lds_bytes, s>>>((const int8_t *)x, (const int8_t *)w, hp, e);
+  kern<<<hp.nblocks, 64 * NW, lds_bytes, s>>>((const int8_t *)x, (const int8_t *)w, hp, e, hd);
   return launch_status();
 }
 
@@ -314,31 +459,34 @@ static int launch_halo(const void *x, const void *w, const HaloParams &hp, const
   return tn == 2 ? launch_halo_tm<CI, 2, 2, S>(x, w, hp, e, lds_bytes, s) : launch_halo_tm<CI, 1, 2, S>(x, w, hp, e, lds_bytes, s);
 }
 
-// 3x3, stride 1 or 2 (both directions alike), padding 1, no dilation, Ci in {64, 128, 256, 512} (stride 2: not 64);
-// input [N, Hi, Wi, Ci]; -1: not this kernel's shape
-int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, int Co, int stride, const EpiDev &e,
-                   hipStream_t s) {
-  if (Ci != 64 && Ci != 128 && Ci != 256 && Ci != 512) return -1;
-  if (stride != 1 && !(stride == 2 && Ci != 64)) return -1;
+// Tile choice for a 3x3 layer over input [N, Hi, Wi, Ci]: fills hp, the column tiles per block (tn), the dynamic LDS
+// size and the wave count; false: not this kernel's shape.  force_tn > 0 asks for that many column tiles (one block
+// over all output channels) and for band mode.
+static bool halo_plan(int N, int Hi, int Wi, int Ci, int Co, int stride, HaloParams &hp, int &tn, int &lds_bytes, int &waves,
+                      int force_tn = 0) {
+  if (Ci != 64 && Ci != 128 && Ci != 256 && Ci != 512) return false;
+  if (stride != 1 && !(stride == 2 && Ci != 64)) return false;
   const int H = (Hi - 1) / stride + 1, W = (Wi - 1) / stride + 1;
-  if (Co % 4 != 0 || Wi > 254 || (int64_t)N * Hi * Wi * Ci >= (1ll << 31) || (int64_t)Co * 9 * Ci >= (1ll << 31)) return -1;
-  if ((int64_t)N * Hi >= (1 << 24)) return -1;
-  HaloParams hp = {};
+  if (Co % 4 != 0 || Wi > 254 || (int64_t)N * Hi * Wi * Ci >= (1ll << 31) || (int64_t)Co * 9 * Ci >= (1ll << 31)) return false;
+  if ((int64_t)N * Hi >= (1 << 24)) return false;
+  hp = HaloParams{};
   hp.N = N; hp.H = H; hp.W = W; hp.Co = Co; hp.Hi = Hi; hp.Wi = Wi;
   hp.PC = (W - 1) * stride + 3;
   hp.img_rows = (H - 1) * stride + 3;
   hp.M = (int64_t)N * H * W;
   hp.x_bytes = (unsigned)((int64_t)N * Hi * Wi * Ci);
   hp.w_bytes = (unsigned)((int64_t)Co * 9 * Ci);
-  constexpr int kLdsLimit = 160 * 1024, kMaxP = 256, kRing1 = 3 * 32 * 256;
+  constexpr int kLdsLimit = 160 * 1024, kMaxP = 256;
+  const int kRing1 = 3 * 32 * 256 * (force_tn > 0 ? force_tn : 1);
   // Tile choice.  A tile of P pixels costs ceil(ceil(P / 32) / 4) rounds of MFMA work (four waves, one 32-row
   // sub-tile each per round) plus about half a round of patch loading and synchronisation; the patch must fit
   // beside the smaller weight ring.  Small images go whole, several per tile; larger ones are cut into bands of
   // rows of equal height, the last band of an image possibly shorter.  Twice the cost is compared, in integers.
   auto rounds2 = [](int pixels) { return 2 * (((pixels + 31) / 32 + 3) / 4) + 1; };
-  int best = 0, lds = 0, tn = 2;
+  int best = 0, lds = 0;
+  tn = 2;
   int64_t tiles_m = 0;
-  if (H * W <= kMaxP / 2) {
+  if (H * W <= kMaxP / 2 && force_tn == 0) {
     int g_max = kMaxP / (H * W);
     if (const char *t = tuning_env("CATCHQ_HALO_G")) g_max = atoi(t) < g_max ? atoi(t) : g_max;
     int64_t best_cost = 0;  // cost of `best_g` images' worth of work, cross-multiplied
@@ -349,7 +497,7 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, 
       const int64_t cost = rounds2(g * H * W);  // per g images
       if (!best_g || cost * best_g < best_cost * g) { best_g = g; best_cost = cost; lds = patch; }
     }
-    if (!best_g) return -1;
+    if (!best_g) return false;
     best = best_g * H;
     hp.image_mode = 1;
     hp.PR = best_g * hp.img_rows;
@@ -368,7 +516,7 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, 
       const int64_t cost = (int64_t)bands * rounds2(tr * W);
       if (!best || cost < best_cost) { best = tr; best_cost = cost; lds = patch; hp.bands = bands; }
     }
-    if (!best) return -1;
+    if (!best) return false;
     hp.image_mode = 0;
     hp.PR = (best - 1) * stride + 3;
     tiles_m = (int64_t)N * hp.bands;
@@ -376,31 +524,44 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, 
   hp.TR = best;
   hp.P = best * W;
   hp.nsub = (hp.P + 31) / 32;
-  if (hp.nsub > 8) return -1;
+  if (hp.nsub > 8) return false;
   // tiles that leave waves of the block without a sub-tile are the implicit-GEMM kernel's case
-  if (hp.nsub < 3) return -1;
-  // 64 channels per block while that still gives every compute unit a block and the ring fits
-  int64_t min_blocks = 256;
-  if (const char *t = tuning_env("CATCHQ_HALO_MINBLK")) min_blocks = atoi(t);
-  if (lds + 3 * 64 * 256 > kLdsLimit || tiles_m * ((Co + 63) / 64) < min_blocks) tn = 1;
-  if (const char *t = tuning_env("CATCHQ_HALO_TN")) tn = atoi(t);
-  if (lds + 3 * 32 * tn * 256 > kLdsLimit) tn = 1;
+  if (hp.nsub < 3) return false;
+  if (force_tn > 0) {
+    tn = force_tn;
+  } else {
+    // 64 channels per block while that still gives every compute unit a block and the ring fits
+    int64_t min_blocks = 256;
+    if (const char *t = tuning_env("CATCHQ_HALO_MINBLK")) min_blocks = atoi(t);
+    if (lds + 3 * 64 * 256 > kLdsLimit || tiles_m * ((Co + 63) / 64) < min_blocks) tn = 1;
+    if (const char *t = tuning_env("CATCHQ_HALO_TN")) tn = atoi(t);
+    if (lds + 3 * 32 * tn * 256 > kLdsLimit) tn = 1;
+  }
   hp.tiles_n = (Co + 32 * tn - 1) / (32 * tn);
   const int64_t nb = tiles_m * hp.tiles_n;
-  if (nb > 0x7fffffff) return -1;
+  if (nb > 0x7fffffff) return false;
   // a stride-2 patch is four times its output and leaves room for one block per compute unit: past one round
   // of blocks the implicit-GEMM kernel is faster (measured on the ResNet-50 downsampling layers at 32 and 64 images)
-  if (stride == 2 && nb > 256) return -1;
+  if (stride == 2 && nb > 256) return false;
   hp.nblocks = (int)nb;
-  int lds_bytes = lds + 3 * 32 * tn * 256;
-  int waves = 4;
+  lds_bytes = lds + 3 * 32 * tn * 256;
+  waves = 4;
   // (64-channel layers: K is 18 steps of 32 bytes, too short for a second wave per SIMD to repay its own set-up;
   // measured on ResNet-50's first stage, four waves end to end +0.9 %)
   if (hp.nsub > 4 && Ci >= 128) waves = 8;
   if (const char *t = tuning_env("CATCHQ_HALO_WAVES")) waves = (atoi(t) == 8 && hp.nsub > 4) ? 8 : 4;
   const int epi_bytes = lds + 4 * 32 * (32 * tn + 8) * 4;  // the epilogue's staging area lies where the ring was
   if (epi_bytes > lds_bytes) lds_bytes = epi_bytes;
-  if (lds_bytes > kLdsLimit) return -1;
+  return lds_bytes <= kLdsLimit;
+}
+
+// 3x3, stride 1 or 2 (both directions alike), padding 1, no dilation, Ci in {64, 128, 256, 512} (stride 2: not 64);
+// input [N, Hi, Wi, Ci]; -1: not this kernel's shape
+int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, int Co, int stride, const EpiDev &e,
+                   hipStream_t s) {
+  HaloParams hp;
+  int tn, lds_bytes, waves;
+  if (!halo_plan(N, Hi, Wi, Ci, Co, stride, hp, tn, lds_bytes, waves)) return -1;
   if (stride == 2) {
     switch (Ci) {
       case 128: return launch_halo<128, 2>(x, w, hp, e, tn, lds_bytes, waves, s);
@@ -414,6 +575,44 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, 
     case 256: return launch_halo<256, 1>(x, w, hp, e, tn, lds_bytes, waves, s);
     default: return launch_halo<512, 1>(x, w, hp, e, tn, lds_bytes, waves, s);
   }
+}
+
+// The head's shapes: 1x1 convolution K1 -> 64 channels (+ ReLU, int8 requantization with unit scale) feeding a 3x3
+// layer 64 -> 64, stride 1, padding 1, whose tiles are bands of rows; K1 in {64, 256}.
+bool conv2d_head_halo_i8_ok(int N, int H, int W, int K1, int Cm, int Co) {
+  if (Cm != 64 || Co != 64 || (K1 != 64 && K1 != 256)) return false;
+  if ((int64_t)N * H * W * K1 >= (1ll << 31)) return false;
+  HaloParams hp;
+  int tn, lds_bytes, waves;
+  if (!halo_plan(N, H, W, Cm, Co, 1, hp, tn, lds_bytes, waves, Co / 32)) return false;
+  return hp.image_mode == 0 && waves == 4 && hp.tiles_n == 1 && (hp.PR * hp.W + 31) / 32 <= 12;
+}
+
+// x [N, H, W, K1] int8, head filters [Cm, K1], w [Co, 3, 3, Cm]; -1: not this kernel's shape
+int conv2d_head_halo_i8(const void *x, int K1, const void *w1, const float *div1, const float *rcp1, const float *bias1,
+                        int exp2_1, int q_position1, const void *w, int N, int H, int W, int Cm, int Co, const EpiDev &e,
+                        hipStream_t s) {
+  if (!conv2d_head_halo_i8_ok(N, H, W, K1, Cm, Co)) return -1;
+  if (!div1 || !rcp1 || !bias1 || exp2_1 < -64 || exp2_1 > 64 || !aligned16(x) || !aligned16(w1) || !aligned16(w)) return -1;
+  HaloParams hp;
+  int tn, lds_bytes, waves;
+  halo_plan(N, H, W, Cm, Co, 1, hp, tn, lds_bytes, waves, Co / 32);
+  hp.x_bytes = (unsigned)((int64_t)N * H * W * K1);
+  lds_bytes += 1024;  // the head's per-channel constants behind the ring
+  if (lds_bytes > 160 * 1024) return -1;
+  HeadDev hd = {(const int8_t *)w1, div1, rcp1, bias1, exp2_1, -q_position1, (unsigned)(Cm * K1)};
+  const int epi = pick_epilogue(Co, e);
+  if (epi == EPI_SCALAR) return -1;
+#define CATCHQ_HEAD(K1_, TMW_)                                                                                                  \
+  return epi == EPI_Q8_RELU ? launch_halo_epi<64, 2, TMW_, 1, EPI_Q8_RELU, 4, K1_, 3>(x, w, hp, e, lds_bytes, s, hd)             \
+                            : launch_halo_epi<64, 2, TMW_, 1, EPI_VECTOR, 4, K1_, 3>(x, w, hp, e, lds_bytes, s, hd)
+  if (K1 == 64) {
+    if (hp.nsub <= 4) CATCHQ_HEAD(64, 1);
+    CATCHQ_HEAD(64, 2);
+  }
+  if (hp.nsub <= 4) CATCHQ_HEAD(256, 1);
+  CATCHQ_HEAD(256, 2);
+#undef CATCHQ_HEAD
 }
 
 }  // namespace catchq

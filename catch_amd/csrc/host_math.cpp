@@ -29,21 +29,7 @@ bool range_for(int bitwidth, Range *r) {
 
 }  // namespace
 
-CATCHQ_API int catchq_version(void) { return 103; }
-
-static std::atomic<int> g_launch_sharing{1};
-
-CATCHQ_API int catchq_set_launch_sharing(int launches) {
-  if (launches < 1) return -CATCHQ_ERR_ARG;
-  return g_launch_sharing.exchange(launches);
-}
-
-namespace catchq {
-int planned_cus() {
-  const int cus = 256 / g_launch_sharing.load(std::memory_order_relaxed);
-  return cus < 1 ? 1 : cus;
-}
-}  // namespace catchq
+CATCHQ_API int catchq_version(void) { return 104; }
 
 CATCHQ_API const char *catchq_status_string(int status) {
   switch (status) {

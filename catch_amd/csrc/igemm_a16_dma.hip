@@ -293,7 +293,7 @@ template <int LOAD>
 static int pick_a16_tile(const void *a, const void *b, const IgemmParams &p, const EpiDev &e, int64_t a_bytes,
                          int64_t b_bytes, hipStream_t s) {
   auto blocks = [&](int bm, int bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
-  const int64_t kCUs = planned_cus();
+  const int64_t kCUs = e.cus;
   int tile = forced_tile();
   if (!tile) {
     // Measured on every Darknet-53 layer (bs16, 416x416): the 64x64 tile is the default -- two accumulator

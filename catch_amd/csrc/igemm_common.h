@@ -122,7 +122,7 @@ template <> struct EpiOf<EPI_LK_RESA_Y_Q16> { typedef EpiSpec<0, 1, 2, CATCHQ_AC
 // that has no instance of the variant returned uses the generic EPI_VECTOR
 inline int pick_epilogue(int N, const EpiDev &e) {
   if (!vec_epilogue_ok(N, e)) return EPI_SCALAR;
-  if (e.acc_out || (e.q && e.q_scale != 1.0f) || (e.chan_div && !e.chan_rcp)) return EPI_VECTOR;
+  if (e.acc_out || (e.q && e.q_scale != 1.0f) || (e.chan_div && !e.chan_rcp) || e.half_steps) return EPI_VECTOR;
   const int div = e.chan_rcp ? 1 : 0, bias = e.bias ? 1 : 0;
   const int res = !e.resid ? 0 : (e.resid_after ? 2 : 1);
   const int ym = !e.y ? 0 : (e.y_f16 ? 2 : 1);
@@ -144,7 +144,7 @@ inline int pick_epilogue(int N, const EpiDev &e) {
 // per-channel constants of one lane's four consecutive channels
 struct EpiLane {
   v4f div, rcp, bias;
-  bool use_rcp, use_div, use_bias, use_res, res_after, unit_q;
+  bool use_rcp, use_div, use_bias, use_res, res_after, unit_q, half_steps;
   int act;
 };
 
@@ -155,6 +155,7 @@ __device__ __forceinline__ EpiLane epi_lane_setup(int n, bool n_ok, const EpiDev
   L.res_after = S::resid_after(e);
   L.act = S::act(e);
   L.unit_q = S::kGeneric ? (e.q_scale == 1.0f) : true;
+  L.half_steps = S::kGeneric ? (e.half_steps != 0) : false;
   // Reciprocal form with the power of two folded in:
   //   v = (f*2^e)/d  ==  q = f*(r*2^e); err = fma(-q, d*2^-e, f); fma(err, r*2^e, q)
   // (scaling by 2^e is exact, so every intermediate is the scaled image of the unfolded one)
@@ -178,9 +179,16 @@ __device__ __forceinline__ float epi_dequant1(int a, int t, const EpiLane &L, in
   if (L.use_rcp) x = div_by_rcp(x, L.div[t], L.rcp[t]);
   else {
     x = __builtin_ldexpf(x, exp2);
-    if (L.use_div) x = x / L.div[t];
+    if (L.half_steps) x = round_f16(x);
+    if (L.use_div) {
+      x = x / L.div[t];
+      if (L.half_steps) x = round_f16(x);
+    }
   }
-  if (L.use_bias) x = x + L.bias[t];
+  if (L.use_bias) {
+    x = x + L.bias[t];
+    if (L.half_steps) x = round_f16(x);
+  }
   return x;
 }
 

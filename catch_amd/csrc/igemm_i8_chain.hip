@@ -304,7 +304,7 @@ static int launch_chain(ChainParams &cp, hipStream_t s) {
 // links[0] is the projection shortcut (no activation, nothing added), links[1..] the blocks' last 1x1
 // convolutions in order; -1 when the shapes are not this kernel's
 int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int Wo, int Co, float *y, int8_t *q,
-                     int q_position, hipStream_t s) {
+                     int q_position, int sharing, hipStream_t s) {
   if (nlinks < 2 || nlinks > kChainMaxLinks || Co % 4 != 0) return -1;
   ChainParams cp = {};
   cp.M = (int64_t)N * Ho * Wo;
@@ -316,7 +316,7 @@ int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int W
   cp.y = y;
   cp.q = q;
   cp.q_neg_pos = -q_position;
-  const int64_t kStreamBytes = (64ll << 20) * planned_cus() / 256;
+  const int64_t kStreamBytes = (64ll << 20) * planned_cus(sharing) / 256;
   cp.y_stream = (y && cp.M * Co * 4 >= kStreamBytes) ? 1 : 0;
   if (!aligned16(y) || !aligned16(q)) return -1;
   for (int i = 0; i < nlinks; ++i) {

@@ -225,11 +225,40 @@ struct EpiArgs {
   double q_scale = 1.0;
   double act_slope = 0.0;
   bool resid_after_act = false;
+  bool half_steps = false;  // fp16 output rounded after scaling, division and bias (the reference's half tensor ops)
 };
 
 struct EpiOut {
   Tensor y, acc, q;
 };
+
+// Planning hint of the calling thread: how many launches it expects to run on the device at the same time (a plan
+// that records the parts of a batch on parallel streams sets it around the recording).  Thread-local, so two
+// threads planning at once do not see each other's value; handed to the C ABI per call (catchq_epilogue_t::sharing).
+thread_local int t_launch_sharing = 1;
+
+// whether catchq_conv1x1_conv3x3_nhwc serves (1x1: k1 -> cm, then 3x3 / stride 1 / padding 1: cm -> co) over n images of
+// h x w in one launch (per-channel constants with reciprocals and 16-byte aligned tensors assumed)
+bool head_fuses_op(int64_t n, int64_t h, int64_t w, int64_t k1, int64_t cm, int64_t co) {
+  float one = 1.0f;
+  catchq_pointwise_head_t hd;
+  std::memset(&hd, 0, sizeof(hd));
+  hd.ci = (int)k1;
+  hd.w = &one; hd.chan_div = hd.chan_rcp = hd.bias = &one;  // presence only: nothing is dereferenced
+  catchq_conv_desc_t d = {(int)n, (int)h, (int)w, (int)cm, (int)co, 3, 3, 1, 1, 1, 1, 1, 1, 1};
+  catchq_epilogue_t e;
+  std::memset(&e, 0, sizeof(e));
+  e.q = &one; e.q_bitwidth = 8;
+  size_t bytes = 1;
+  return catchq_conv1x1_conv3x3_workspace_size(&hd, &d, &e, &bytes) == CATCHQ_OK && bytes == 0;
+}
+
+int64_t set_launch_sharing_op(int64_t launches) {
+  TORCH_CHECK(launches >= 1, "set_launch_sharing: at least one launch");
+  const int before = t_launch_sharing;
+  t_launch_sharing = (int)launches;
+  return before;
+}
 
 Tensor as_f32_vec(const c10::optional<Tensor> &t, int64_t n, const char *name) {
   if (!t.has_value() || !t->defined()) return Tensor();
@@ -304,6 +333,8 @@ EpiOut prepare_epilogue(const EpiArgs &a, at::IntArrayRef out_shape, int64_t co,
                 "resid must be a contiguous fp32 tensor of the output's shape");
     e->resid = a.resid->data_ptr<float>();
   }
+  e->sharing = t_launch_sharing;
+  e->half_steps = (a.half_steps && a.y_half) ? 1 : 0;
   e->act = (int)a.act;
   e->act_slope = (float)a.act_slope;
   e->resid_after_act = a.resid_after_act ? 1 : 0;
@@ -467,6 +498,66 @@ std::tuple<Tensor, Tensor> qconv2d_shortcut_op(const Tensor &qx, const Tensor &q
   return std::make_tuple(o.y, o.q);
 }
 
+// First two convolutions of a bottleneck block (catchq_conv1x1_conv3x3_nhwc): qx [N,H,W,K1] int8 NHWC through the
+// 1x1 filters w1 [Cm,K1] (or [Cm,1,1,K1]) + ReLU + int8 requantization at position q_position1, then qw [Co,kh,kw,Cm]
+// with the usual epilogue arguments.
+std::tuple<Tensor, Tensor> qconv2d_head_op(const Tensor &qx, const Tensor &w1, int64_t exp2_1,
+                                           const c10::optional<Tensor> &chan_div1, const c10::optional<Tensor> &bias1,
+                                           int64_t q_position1, const Tensor &qw, int64_t exp2,
+                                           const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias,
+                                           at::IntArrayRef padding, at::IntArrayRef stride, at::IntArrayRef dilation,
+                                           int64_t act, bool want_y, bool y_half, int64_t q_bitwidth, int64_t q_position,
+                                           double q_scale, double act_slope) {
+  c10::DeviceGuard guard(qx.device());
+  TORCH_CHECK(qx.dim() == 4 && qw.dim() == 4 && qx.is_contiguous() && qw.is_contiguous() && w1.is_contiguous(),
+              "qconv2d_head expects contiguous NHWC activations and [Co,kh,kw,Ci] weights");
+  TORCH_CHECK(qx.scalar_type() == at::kChar && qw.scalar_type() == at::kChar && w1.scalar_type() == at::kChar,
+              "qconv2d_head: int8 operands expected");
+  const int64_t cm = qw.size(3), k1 = qx.size(3);
+  TORCH_CHECK(w1.size(0) == cm && w1.numel() == cm * k1, "qconv2d_head: the head's filters must be [", cm, ", ", k1, "]");
+  TORCH_CHECK(w1.device() == qx.device() && qw.device() == qx.device(), "qconv2d_head: operands on different devices");
+  TORCH_CHECK(padding.size() == 2 && stride.size() == 2 && dilation.size() == 2, "2-d conv parameters expected");
+  catchq_conv_desc_t d;
+  d.n = (int)qx.size(0); d.h = (int)qx.size(1); d.w = (int)qx.size(2); d.ci = (int)cm;
+  d.co = (int)qw.size(0); d.kh = (int)qw.size(1); d.kw = (int)qw.size(2);
+  d.pad_h = (int)padding[0]; d.pad_w = (int)padding[1];
+  d.stride_h = (int)stride[0]; d.stride_w = (int)stride[1];
+  d.dil_h = (int)dilation[0]; d.dil_w = (int)dilation[1];
+  d.groups = 1;
+  TORCH_CHECK(d.stride_h > 0 && d.stride_w > 0 && d.pad_h >= 0 && d.pad_w >= 0, "bad stride or padding");
+  const int ho = catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h);
+  const int wo = catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w);
+  TORCH_CHECK(ho > 0 && wo > 0, "Calculated output size is too small");
+  catchq_epilogue_t e;
+  std::vector<Tensor> keep;
+  EpiOut o = prepare_epilogue(make_args(exp2, chan_div, bias, c10::nullopt, act, want_y, y_half, false, q_bitwidth,
+                                        q_position, q_scale, act_slope, false),
+                              {d.n, ho, wo, d.co}, d.co, qx.options(), &e, &keep);
+  catchq_pointwise_head_t hd;
+  std::memset(&hd, 0, sizeof(hd));
+  hd.w = w1.data_ptr();
+  hd.ci = (int)k1;
+  TORCH_CHECK(exp2_1 >= -126 && exp2_1 <= 126, "position sum out of range");
+  hd.exp2 = (int)exp2_1;
+  hd.q_position = (int)q_position1;
+  Tensor cd = as_f32_vec(chan_div1, cm, "head chan_div"), bs = as_f32_vec(bias1, cm, "head bias");
+  if (cd.defined()) {
+    hd.chan_div = cd.data_ptr<float>();
+    keep.push_back(cd);
+    Tensor rcp = reciprocals_for(cd);
+    if (rcp.defined()) { hd.chan_rcp = rcp.data_ptr<float>(); keep.push_back(rcp); }
+  }
+  if (bs.defined()) { hd.bias = bs.data_ptr<float>(); keep.push_back(bs); }
+  if (d.n == 0) return std::make_tuple(o.y, o.q);
+  size_t ws_bytes = 0;
+  check_status(catchq_conv1x1_conv3x3_workspace_size(&hd, &d, &e, &ws_bytes), "torch_mlu::qconv2d_head");
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, qx.options().dtype(at::kChar));
+  check_status(catchq_conv1x1_conv3x3_nhwc(qx.data_ptr(), &hd, qw.data_ptr(), &d, &e, ws.data_ptr(), ws_bytes,
+                                           current_stream()),
+               "torch_mlu::qconv2d_head");
+  return std::make_tuple(o.y, o.q);
+}
+
 // Residual chain (catchq_conv1x1_chain_nhwc): xs[i] [N,Hi,Wi,Ci] int8 NHWC, ws[i] [Co,Ci] or [Co,1,1,Ci] int8;
 // link 0 is the projection shortcut, links 1.. the blocks' last 1x1 convolutions in order.
 std::tuple<Tensor, Tensor> qconv2d_chain_op(at::TensorList xs, at::TensorList ws, at::IntArrayRef strides,
@@ -489,6 +580,9 @@ std::tuple<Tensor, Tensor> qconv2d_chain_op(at::TensorList xs, at::TensorList ws
                 "qconv2d_chain: int8 NHWC activations of one batch expected");
     TORCH_CHECK(w.is_contiguous() && w.scalar_type() == at::kChar && w.size(0) == co && w.numel() == co * x.size(3),
                 "qconv2d_chain: int8 [Co,Ci] filters expected");
+    TORCH_CHECK(x.device() == xs[0].device() && w.device() == xs[0].device() && chan_divs[i].device() == xs[0].device() &&
+                    biases[i].device() == xs[0].device(),
+                "qconv2d_chain: every link's tensors must live on one device");
     const int h = catchq_conv_out_size((int)x.size(1), 1, 0, (int)strides[i], 1);
     const int w_ = catchq_conv_out_size((int)x.size(2), 1, 0, (int)strides[i], 1);
     if (i == 0) { ho = h; wo = w_; }
@@ -508,7 +602,7 @@ std::tuple<Tensor, Tensor> qconv2d_chain_op(at::TensorList xs, at::TensorList ws
   if (q_bitwidth == 8) q = at::empty({n, ho, wo, co}, xs[0].options().dtype(at::kChar));
   if (n == 0) return std::make_tuple(y, q);
   check_status(catchq_conv1x1_chain_nhwc(links, (int)nl, (int)n, ho, wo, (int)co, want_y ? y.data_ptr<float>() : nullptr,
-                                         q.defined() ? q.data_ptr() : nullptr, (int)q_position, current_stream()),
+                                         q.defined() ? q.data_ptr() : nullptr, (int)q_position, t_launch_sharing, current_stream()),
                "torch_mlu::qconv2d_chain");
   return std::make_tuple(y, q);
 }
@@ -588,6 +682,7 @@ struct Prepared {
   c10::StreamId made_on = 0;  // stream that allocated and filled qw / new_scale
   int bw_x = 8, bw_w = 8, pos_x = 0, pos_w = 0;
   bool per_channel = false;
+  bool params_half = false;  // per-channel parameters derived with half tensor ops (half q_scale, int8)
   int variant = 0;   // caller's layout choice for qw (part of the cache key)
   Tensor qw;         // conv: [Co,kh,kw,Ci/g]; linear: [N,K]
   Tensor new_scale;  // device fp32 [Co] when per_channel
@@ -672,7 +767,8 @@ std::shared_ptr<Prepared> prepare(MakeDense make_dense, const Tensor &weight, co
     } else {
       const int64_t co = w_dense.size(0);
       TORCH_CHECK(s_host.numel() == 2 + co, "per-channel q_scale must hold 2 + ", co, " values, got ", s_host.numel());
-      PerChannel pc = half_chain(q_scale, bw)
+      p->params_half = half_chain(q_scale, bw);
+      PerChannel pc = p->params_half
                           ? per_channel_params_half(q_scale.reshape({-1}).slice(0, 2), bw, w_dense.options())
                           : per_channel_params(s + 2, co, bw, w_dense.options());
       p->pos_w = pc.new_pos;
@@ -763,6 +859,9 @@ Tensor conv_prepared(const Tensor &qx, const Prepared &prep, const Tensor &bias,
   if (prep.per_channel) a.chan_div = prep.new_scale;
   if (has_bias(bias)) a.bias = bias;
   a.y_half = half;
+  // per-channel branch on half tensors: the vendor convolution's half output, then `/ new_scale` and `+ bias` as
+  // half tensor ops (quantify_conv_forward.cpp:123-129); where the q-params stayed fp32 (int16), so does this
+  a.half_steps = half && prep.per_channel && prep.params_half;
   return qconv2d_impl(qx, qw, padding, stride, dilation, groups, a).y;
 }
 
@@ -1028,6 +1127,10 @@ TORCH_LIBRARY(torch_mlu, m) {
         "int s_stride, int s_exp2, Tensor? s_chan_div, Tensor? s_bias, int[] padding, int[] stride, int[] dilation, "
         "int act=0, bool want_y=True, bool y_half=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
         "float act_slope=0.0, bool resid_after_act=False) -> (Tensor, Tensor)");
+  m.def("qconv2d_head(Tensor qx, Tensor w1, int exp2_1, Tensor? chan_div1, Tensor? bias1, int q_position1, Tensor qw, "
+        "int exp2, Tensor? chan_div, Tensor? bias, int[] padding, int[] stride, int[] dilation, int act=0, "
+        "bool want_y=True, bool y_half=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
+        "float act_slope=0.0) -> (Tensor, Tensor)");
   m.def("qconv2d_chain(Tensor[] xs, Tensor[] ws, int[] strides, int[] exp2s, Tensor[] chan_divs, Tensor[] biases, "
         "bool want_y=False, int q_bitwidth=8, int q_position=0) -> (Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
@@ -1037,6 +1140,8 @@ TORCH_LIBRARY(torch_mlu, m) {
         "int[] padding, int[] stride, int[] dilation, int groups, int input_bitwidth=8, int weight_bitwidth=8) -> Tensor");
   m.def("maxpool_nhwc(Tensor x, int k, int stride, int pad) -> Tensor");
   m.def("global_avgpool_nhwc(Tensor x, int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> Tensor");
+  m.def("set_launch_sharing(int launches) -> int", &set_launch_sharing_op);
+  m.def("conv1x1_conv3x3_fuses(int n, int h, int w, int k1, int cm, int co) -> bool", &head_fuses_op);
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
   m.def("weight_cache_size() -> int", &cache_size_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
@@ -1059,6 +1164,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("quantize_conv2d", &quantize_conv2d_op);
   m.impl("qconv2d", &qconv2d_op);
   m.impl("qconv2d_shortcut", &qconv2d_shortcut_op);
+  m.impl("qconv2d_head", &qconv2d_head_op);
   m.impl("qconv2d_chain", &qconv2d_chain_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);

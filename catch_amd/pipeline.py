@@ -162,7 +162,7 @@ def _decode(layer, sd, device, ci_dev, co_dev, fractional=False):
 
 class FusedNet(object):
     def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True,
-                 fractional_scale=False, chain_links=None):
+                 fractional_scale=False, chain_links=None, fuse_heads=True):
         """fractional_scale: quantize activations and weights with position and fractional scale -- the
         general form the reference's fused (graph) mode hands to its backend per tensor / per axis
         (jit/utils/utils.cpp:81-167) -- instead of the eager ops' power-of-two steps.
@@ -170,7 +170,10 @@ class FusedNet(object):
         blocks' int8 tensors instead of being stored and read back in fp32: a block whose chain back to the
         stage's projection shortcut has at most this many links (the shortcut counts as one) evaluates the
         whole chain inside its last convolution's launch (torch_mlu::qconv2d_chain); None picks the default
-        rule (_default_chain_links), 0 switches the recomputation off."""
+        rule (_default_chain_links), 0 switches the recomputation off.
+        fuse_heads: a 1x1 convolution + ReLU whose only reader is a 3x3 convolution (the first two layers of a
+        bottleneck block) runs inside that convolution's launch where the kernel library serves the shapes
+        (torch_mlu::qconv2d_head); its int8 output is then never stored."""
         self.layers = list(layers)
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
@@ -235,6 +238,35 @@ class FusedNet(object):
         self._fused_away = set(ds.name for ds in self.shortcut_of.values())
         self._fused_away.update(links[0].name for links in self.chain_of.values()
                                 if links[1].name in self.chain_of or links[1].name in self.shortcut_of)
+        # Heads: head_of[3x3 layer name] = the 1x1 layer in front of it.  Whether a pair runs as one launch also
+        # depends on the image size (head_fuses), known when a batch arrives.
+        self.head_of = {}
+        if fuse_heads:
+            by_name = {l.name: l for l in self.layers}
+            for l in self.layers:
+                h = by_name.get(l.src) if l.kind == "conv" and isinstance(l.src, str) else None
+                if h is None or h.kind != "conv" or l.name in self.chain_of or l.name in self.shortcut_of:
+                    continue
+                readers = [m for m in self.layers
+                           if m.src == h.name or (isinstance(m.src, tuple) and h.name in m.src) or m.add == h.name]
+                lq, hq = self.q[l.name], self.q[h.name]
+                if (l.k == 3 and l.pad == 1 and l.stride == 1 and l.groups == 1 and not l.add
+                        and h.k == 1 and h.pad == 0 and h.stride == 1 and h.groups == 1 and h.act == "relu" and not h.add
+                        and readers == [l] and h.name not in self.outputs and not self.f_demand[h.name]
+                        and self.q_demand[h.name] == [(8, lq.pos_x, 1.0)]
+                        and (lq.bw_x, lq.bw_w, hq.bw_x, hq.bw_w) == (8, 8, 8, 8) and hq.scale_x == 1.0
+                        and hq.chan_div is not None and hq.bias is not None and -64 <= hq.exp2 <= 64
+                        and h.name not in self._fused_away and not (self.stem and self.stem["name"] in (l.name, h.name))):
+                    self.head_of[l.name] = h
+        self._head_names = set(h.name for h in self.head_of.values())
+
+    def head_fuses(self, head, n, h, w):
+        """whether the 1x1 layer `head` and the 3x3 layer behind it run as one launch over n images of h x w"""
+        if head.name not in self._head_names:
+            return False
+        main = next(l for l in self.layers if self.head_of.get(l.name) is head)
+        return bool(torch.ops.torch_mlu.conv1x1_conv3x3_fuses(n, h, w, self.cdev[head.src], self.cdev[head.name],
+                                                             self.cdev[main.name]))
 
     @staticmethod
     def _default_chain_links(co):
@@ -355,9 +387,33 @@ class FusedNet(object):
                                                               w + 2 * sp + self.stem["extra"], sp, sp, d[2])
             else:
                 env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"], d[2])
+        skipped_heads = set()
         for l in self.layers:
             name = l.name
             if l.kind == "conv" and not tracing and name in self._fused_away:
+                continue
+            if l.kind == "conv" and not tracing and name in self._head_names:
+                hx = env[(l.src, 8, self.q[name].pos_x, 1.0)]
+                if self.head_fuses(l, hx.shape[0], hx.shape[1], hx.shape[2]):
+                    skipped_heads.add(name)  # computed inside the launch of the 3x3 layer behind it
+                    continue
+            if l.kind == "conv" and name in self.head_of and self.head_of[name].name in skipped_heads:
+                lq, h = self.q[name], self.head_of[name]
+                hq = self.q[h.name]
+                qd = self.q_demand[name][0] if self.q_demand[name] else None
+                want_y = self.f_demand[name] or qd is None
+                tick(name)
+                y, q = ops.qconv2d_head(env[(h.src, 8, hq.pos_x, 1.0)], hq.qw, hq.exp2, hq.chan_div, hq.bias, lq.pos_x,
+                                        lq.qw, lq.exp2, lq.chan_div, lq.bias, self.padding(l), [1, 1], [1, 1],
+                                        _ACT_CODE[l.act], want_y, self.out_half and name in self.outputs,
+                                        qd[0] if qd else 0, qd[1] if qd else 0, qd[2] if qd else 1.0, LEAKY_SLOPE)
+                tick(name)
+                if want_y:
+                    env[(name, "f")] = y
+                if qd:
+                    env[(name,) + qd] = q
+                for d in self.q_demand[name][1:]:
+                    env[(name,) + d] = ops.quantize(y, d[0], d[1], d[2])
                 continue
             if l.kind == "conv":
                 lq = self.q[name]
@@ -466,15 +522,21 @@ class FusedNet(object):
         parts = max(1, min(int(streams), static_in.shape[0]))
         chunks = list(static_in.chunk(parts))
         side = [torch.cuda.Stream() for _ in chunks]
-        # the launches recorded below will share the device: their tile shapes are chosen for a part of it
-        lib = _native.kernel_lib()
-        before = lib.catchq_set_launch_sharing(len(chunks))
+        # the launches recorded below will share the device: their tile shapes are chosen for a part of it (a hint
+        # of this thread, handed to the kernel library with every call)
+        before = torch.ops.torch_mlu.set_launch_sharing(len(chunks))
         try:
             return self._capture(static_in, chunks, side)
         finally:
-            lib.catchq_set_launch_sharing(max(before, 1))
+            torch.ops.torch_mlu.set_launch_sharing(max(before, 1))
 
     def _capture(self, static_in, chunks, side):
+        """Side streams only ever wait on the capturing stream (fork) and are only ever waited on by it (join).
+        Waits between two side streams in both directions inside one capture ended a capture with a segmentation
+        fault inside the runtime's end-of-capture call; nothing here may introduce such a wait."""
+        cur0 = torch.cuda.current_stream()
+        if len(set(s.cuda_stream for s in side)) != len(side) or any(s.cuda_stream == cur0.cuda_stream for s in side):
+            raise ValueError("capture: every part needs a side stream of its own, distinct from the capturing stream")
         sample = None
         for st, c in zip(side, chunks):  # warm-up outside the capture, on the streams the graph will use
             st.wait_stream(torch.cuda.current_stream())

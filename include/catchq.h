@@ -11,8 +11,7 @@
  *     workspace) is owned by the caller; nothing here allocates or frees;
  *   - all device entry points are asynchronous on `stream` (a hipStream_t passed
  *     as void*; NULL = the null stream).  They are re-entrant and keep no state from call to
- *     call, with two documented exceptions: the planning hint catchq_set_launch_sharing
- *     (process-wide, affects speed only) and the fixed scratch memory of
+ *     call, with one documented exception: the fixed scratch memory of
  *     catchq_quantize_param_noalloc (per device, calls on one device must not overlap);
  *   - the return value is a status (0 = CATCHQ_OK); no exception crosses the
  *     boundary; catchq_status_string() names a status;
@@ -50,13 +49,6 @@ enum { CATCHQ_QUANTIZE_POSITION = 0, CATCHQ_QUANTIZE_POSITION_SCALE = 1, CATCHQ_
 
 int catchq_version(void);
 const char *catchq_status_string(int status);
-
-/* Planning hint: `launches` launches of this library are expected to run on the device at the same time
- * (e.g. the parts of a batch on parallel streams), so each one's tile shapes are chosen for 1/launches of the
- * compute units.  Affects speed only, never a result.  Process-wide, default 1; returns the previous value,
- * or -CATCHQ_ERR_ARG for launches < 1.  (The reference plans per handle, one handle per device re-bound to
- * the calling thread's queue: torch_mlu/csrc/aten/cnnl/cnnlHandle.cpp:41-55; it has no such hint.) */
-int catchq_set_launch_sharing(int launches);
 
 /* ------------------------------------------------------------------ host q-param math */
 
@@ -187,6 +179,18 @@ typedef struct catchq_epilogue {
   int resid_after_act;   /* 0: act(v + resid), otherwise act(v) + resid */
   const int32_t *exp2_dev[2]; /* device-resident positions added to exp2 when non-NULL (no host sync);
                                  the reciprocal form of the division is not used with them */
+  int half_steps;        /* y_dtype CATCHQ_F16 only.  Non-zero: v is rounded to binary16 after the scaling by 2^exp2,
+                            after the division by chan_div[c] and after the addition of bias[c] -- the values the
+                            reference's per-channel branch produces for half tensors, where the vendor convolution
+                            returns half and `output / new_scale` and `output + bias` are half tensor ops
+                            (operators/cnnl/quantify_conv_forward.cpp:123-129); an intermediate beyond 65504 is inf,
+                            as there.  Zero: all steps in fp32, one final conversion. */
+  int sharing;           /* planning hint, per call: this many launches are expected to run on the device at the
+                            same time (e.g. the parts of a batch on parallel streams), so the tile shapes are chosen
+                            for 1/sharing of the compute units; 0 or 1: the launch has the device to itself.
+                            Affects speed only, never a result.  (The reference plans per handle, one handle per
+                            device re-bound to the calling thread's queue: torch_mlu/csrc/aten/cnnl/cnnlHandle.cpp:41-55;
+                            it has no such hint.) */
 } catchq_epilogue_t;
 
 /* cnnl_mm(self, self_position, other, other_position, false, true) -> cnnlMatMul
@@ -261,6 +265,32 @@ int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void *w, int w_
                                 const catchq_epilogue_t *epilogue, const catchq_shortcut_t *shortcut, void *workspace,
                                 size_t workspace_bytes, catchq_stream_t stream);
 
+/* First two convolutions of a bottleneck block in one launch.  In the reference a bottleneck block begins with two
+ * torch_mlu::conv2d calls (cnnl_conv2d, operators/cnnl/quantify_conv_forward.cpp:56-147), each followed by ReLU
+ * (operators/cnnl/activation.cpp): a 1x1 reduction whose output is quantized again for the 3x3 convolution behind
+ * it.  Here `head` is that 1x1 convolution of x [n, h, w, head->ci] (int8) with head->w [desc->ci, head->ci] (int8),
+ *   v1 = float(acc1) * 2^head->exp2 / head->chan_div[c] + head->bias[c]
+ *   q1 = sat(rne(relu(v1) * 2^-head->q_position))                                  (int8, never stored)
+ * and `desc` / `w` / `epilogue` describe the convolution of q1 [n, h, w, desc->ci] exactly as catchq_conv2d_nhwc takes
+ * them (desc->n/h/w are x's; int8 x int8).  The values are those of two catchq_conv2d_nhwc calls, bit for bit.
+ * The fused kernel serves 3x3 / stride 1 / padding 1 / 64 -> 64 channels behind a head of 64 or 256 input channels
+ * on images cut into bands of rows (catchq_conv1x1_conv3x3_workspace_size reports 0 then); any other shape runs as
+ * two launches with q1 in the caller's workspace (n * h * w * desc->ci bytes). */
+typedef struct catchq_pointwise_head {
+  const void *w;         /* device int8 [desc->ci, ci] */
+  int ci;                /* input channels of the 1x1 convolution */
+  int exp2;
+  const float *chan_div; /* device [desc->ci] or NULL */
+  const float *chan_rcp; /* device [desc->ci] or NULL, as in catchq_epilogue_t */
+  const float *bias;     /* device [desc->ci] or NULL */
+  int q_position;
+} catchq_pointwise_head_t;
+int catchq_conv1x1_conv3x3_workspace_size(const catchq_pointwise_head_t *head, const catchq_conv_desc_t *desc,
+                                          const catchq_epilogue_t *epilogue, size_t *bytes);
+int catchq_conv1x1_conv3x3_nhwc(const void *x, const catchq_pointwise_head_t *head, const void *w,
+                                const catchq_conv_desc_t *desc, const catchq_epilogue_t *epilogue, void *workspace,
+                                size_t workspace_bytes, catchq_stream_t stream);
+
 /* Residual chain of a stage of bottleneck blocks, recomputed from its int8 inputs in one launch.
  * In the reference every residual block ends in torch_mlu::conv2d (cnnl_conv2d,
  * operators/cnnl/quantify_conv_forward.cpp:56-147) followed by a float add (cnnl_add, operators/cnnl/add.cpp)
@@ -277,7 +307,8 @@ int catchq_conv2d_shortcut_nhwc(const void *x, int x_bits, const void *w, int w_
  * theirs bit for bit; the blocks' fp32 outputs in between are never stored.
  * Requirements (CATCHQ_ERR_UNSUPPORTED otherwise): 2 <= nlinks <= CATCHQ_CHAIN_MAX_LINKS, ci % 64 == 0,
  * co % 4 == 0, chan_div / chan_rcp / bias given for every link (chan_rcp as in catchq_epilogue_t),
- * -64 <= exp2 <= 64, every tensor below 2 GiB and 16-byte aligned. */
+ * -64 <= exp2 <= 64, every tensor below 2 GiB and 16-byte aligned.  `sharing` is the planning hint of
+ * catchq_epilogue_t::sharing. */
 #define CATCHQ_CHAIN_MAX_LINKS 8
 typedef struct catchq_chain_link {
   const void *x;         /* device int8 [n, in_h, in_w, ci] */
@@ -290,7 +321,7 @@ typedef struct catchq_chain_link {
   const float *bias;     /* device [co] */
 } catchq_chain_link_t;
 int catchq_conv1x1_chain_nhwc(const catchq_chain_link_t *links, int nlinks, int n, int ho, int wo, int co,
-                              float *y, void *q, int q_position, catchq_stream_t stream);
+                              float *y, void *q, int q_position, int sharing, catchq_stream_t stream);
 
 /* ------------------------------------------------------------------ neighbours of the convolutions */
 
@@ -317,6 +348,16 @@ int catchq_global_avgpool_quantize_nhwc(const float *x, void *q, int bitwidth, i
  * "depthwise", ...): for logs and tests; not part of the arithmetic. */
 const char *catchq_conv2d_route(int x_bits, int w_bits, const catchq_conv_desc_t *desc);
 const char *catchq_gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k);
+
+/* ------------------------------------------------------------------ diagnostics */
+
+/* Measurement aid, no counterpart in the reference: `blocks` blocks of four waves each run `iters` rounds of four
+ * independent v_mfma_i32_32x32x32_i8 on operand fragments read once from `operands` (1 MiB of device memory,
+ * 16-byte aligned; its contents decide how many bits toggle, which decides the clock the device sustains) with no
+ * memory access inside the loop: 4 * blocks * iters * 4 * 65536 integer operations per call.  `sink` (one int32
+ * of device memory) is only written if the sums take one improbable value.  Timed by the caller
+ * (bench.py --probe mfma). */
+int catchq_diag_mfma_i8_loop(const void *operands, int iters, int blocks, int32_t *sink, catchq_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 from catch_amd import _native
-from catch_amd._native import ChainLink, ConvDesc, Epilogue, Shortcut, check
+from catch_amd._native import ChainLink, ConvDesc, Epilogue, PointwiseHead, Shortcut, check
 
 F32, F16 = 0, 1
 _INT = {8: torch.int8, 16: torch.int16, 31: torch.int32, 32: torch.int32}
@@ -152,7 +152,26 @@ def conv2d_shortcut_nhwc(x, w, sx, sw, sc_stride, sc_exp2, sc_chan_div=None, sc_
     return out, need.value
 
 
-def conv1x1_chain_nhwc(links, want_y=True, want_q=True, q_pos=0):
+def conv1x1_conv3x3_nhwc(x, w1, exp2_1, div1, rcp1, bias1, q_pos1, w, padding=(1, 1), stride=(1, 1), exp2=0, chan_div=None,
+                         bias=None, act=0, y_dtype=None, q_bw=8, q_pos=0, q_scale=1.0, chan_rcp=None, sharing=0):
+    """x [N,H,W,K1] int8, w1 [Cm,K1] int8 (1x1 + ReLU + requantization at q_pos1), w [Co,kh,kw,Cm] int8
+    -> (outputs, workspace bytes the library asked for)"""
+    d = conv_desc((x.shape[0], x.shape[1], x.shape[2], w.shape[3]), w.shape, padding, stride, (1, 1), 1)
+    ho = lib().catchq_conv_out_size(d.h, d.kh, d.pad_h, d.stride_h, d.dil_h)
+    wo = lib().catchq_conv_out_size(d.w, d.kw, d.pad_w, d.stride_w, d.dil_w)
+    e, out = _epilogue((d.n, ho, wo, d.co), x.device, exp2, chan_div, bias, None, act, y_dtype, False, q_bw, q_pos,
+                       q_scale, chan_rcp)
+    e.sharing = sharing
+    hd = PointwiseHead(ptr(w1), x.shape[3], exp2_1, ptr(div1), ptr(rcp1), ptr(bias1), q_pos1)
+    need = ctypes.c_size_t()
+    check(lib().catchq_conv1x1_conv3x3_workspace_size(ctypes.byref(hd), ctypes.byref(d), ctypes.byref(e), ctypes.byref(need)))
+    ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=x.device)
+    check(lib().catchq_conv1x1_conv3x3_nhwc(ptr(x), ctypes.byref(hd), ptr(w), ctypes.byref(d), ctypes.byref(e), ptr(ws),
+                                            need.value, stream()))
+    return out, need.value
+
+
+def conv1x1_chain_nhwc(links, want_y=True, want_q=True, q_pos=0, sharing=0):
     """links: dicts with x [N,H,W,Ci] int8, w [Co,Ci] int8, stride, exp2, chan_div, chan_rcp, bias (device tensors);
     links[0] is the projection shortcut.  -> {"y": fp32 or None, "q": int8 or None}"""
     n, co = links[0]["x"].shape[0], links[0]["w"].shape[0]
@@ -169,7 +188,7 @@ def conv1x1_chain_nhwc(links, want_y=True, want_q=True, q_pos=0):
     dev_ = links[0]["x"].device
     y = torch.empty((n, ho, wo, co), dtype=torch.float32, device=dev_) if want_y else None
     q = torch.empty((n, ho, wo, co), dtype=torch.int8, device=dev_) if want_q else None
-    check(lib().catchq_conv1x1_chain_nhwc(arr, len(links), n, ho, wo, co, ptr(y), ptr(q), q_pos, stream()))
+    check(lib().catchq_conv1x1_chain_nhwc(arr, len(links), n, ho, wo, co, ptr(y), ptr(q), q_pos, sharing, stream()))
     return {"y": y, "q": q}
 
 

@@ -76,16 +76,15 @@ def test_conv2d_qint_grid(bias, bw, per_channel, half):
     assert (conv.scale.dtype == torch.float16) == (half and bw == "int8")  # int16 q-params stay fp32
     if half and per_channel and conv.scale.dtype == torch.float16:
         # the reference's all-half order (quantify.cpp:55-114 and quantify_conv_forward.cpp:123-129 on half
-        # tensors): same integers bit for bit; the output, rounded once here and three times there, within
-        # 1e-3 of its range
+        # tensors): same integers bit for bit
         r = ref_order.conv2d_per_channel(xin, conv.weight.detach().cpu(), conv.bias.detach().cpu(), (3, 3), (3, 3),
                                          (1, 1), 1, conv.scale.detach().cpu(), conv.quantized_mode.cpu().numpy())
         q, new_pos, new_scale = torch.ops.torch_mlu.quantize_per_channel(conv.weight.detach(), conv.scale.detach()[2:], 8)
         assert same_bits(r["qw"], q.permute(0, 2, 3, 1).contiguous().cpu().numpy())
         assert int(new_pos.item()) == r["new_pos"] and torch.equal(new_scale.cpu(), r["new_scale"])
-        want = r["y"].float().numpy()
-        err = np.abs(got.float().cpu().numpy() - want).max()
-        assert err <= 1e-3 * (want.max() - want.min()), err / (want.max() - want.min())
+        # ... and the output: rounded to half after the scaling, after `/ new_scale` and after `+ bias`
+        assert same_bits(r["y"].contiguous(memory_format=torch.channels_last).numpy(),
+                         got.contiguous(memory_format=torch.channels_last).cpu().numpy())
     else:
         ref = oops.conv2d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), b, (3, 3), (3, 3), (1, 1), 1,
                           conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
@@ -346,8 +345,7 @@ def test_conv1d_module_swap(bw, per_channel, half):
         r = ref_order.conv2d_per_channel(xin[:, :, None, :], conv.weight.detach().cpu()[:, :, None, :],
                                          conv.bias.detach().cpu(), (0, 3), (1, 2), (1, 2), 2, conv.scale.detach().cpu(),
                                          conv.quantized_mode.cpu().numpy())
-        want = r["y"][:, :, 0, :].float().numpy()
-        assert np.abs(got.float().cpu().numpy() - want).max() <= 1e-3 * (want.max() - want.min())
+        assert same_bits(r["y"][:, :, 0, :].contiguous().numpy(), got.cpu().contiguous().numpy())
     else:
         ref = oops.conv1d(xin.numpy(), conv.weight.detach().float().cpu().numpy(), conv.bias.detach().float().cpu().numpy(),
                           (3,), (2,), (2,), 2, conv.scale.detach().float().cpu().numpy(), conv.quantized_mode.cpu().numpy())
@@ -468,14 +466,42 @@ def test_conv2d_first_qint(k, co, h, w):
     # exact: the oracle on the tensor the module hands to the op
     x_norm = ((raw.half().cuda() - conv.input_mean) / conv.input_std)
     assert x_norm.dtype == torch.float16
-    # the all-half model against the reference's half tensor ops: same integers, output within 1e-3 of its range
+    # the all-half model against the reference's half tensor ops: same integers, same output bits
     assert conv.scale.dtype == torch.float16
     r = ref_order.conv2d_per_channel(x_norm.cpu(), conv.weight.detach().cpu(), conv.bias.detach().cpu(), (2, 2), (1, 4),
                                      (1, 1), 1, conv.scale.detach().cpu(), conv.quantized_mode.cpu().numpy())
     q = torch.ops.torch_mlu.quantize_per_channel(conv.weight.detach(), conv.scale.detach()[2:], 8)[0]
     assert same_bits(r["qw"], q.permute(0, 2, 3, 1).contiguous().cpu().numpy())
-    want = r["y"].float().numpy()
-    assert np.abs(got.float().cpu().numpy() - want).max() <= 1e-3 * (want.max() - want.min())
+    assert same_bits(r["y"].contiguous().numpy(), got.cpu().contiguous().numpy())
+
+
+def test_conv2d_half_per_channel_overflows_to_inf_like_the_reference():
+    """all-half per-channel convolution whose scaled integer sum exceeds 65504: the reference's vendor convolution
+    returns half, so the value is inf before `/ new_scale` and `+ bias` see it (quantify_conv_forward.cpp:123-129);
+    the fp32 quotient would have been finite"""
+    note("conv2d half per-channel overflow")
+    torch.manual_seed(5)
+    co, ci = 16, 256
+    # channel 0: one large tap (a wide weight range, so the shared position sits well above the other channels' own);
+    # channels 1..7: 256 small positive taps on a positive input: the sum times new_scale (about 15.6) passes 65504
+    # although the quotient (about 7700) does not; channels 8..15: the same taps with alternating signs, small sums
+    w = torch.zeros(co, ci, 1, 1)
+    w[0, 0] = 60.0
+    w[1:8] = 0.5 + 0.01 * torch.rand(7, ci, 1, 1)
+    sign = torch.tensor([1.0, -1.0]).repeat(ci // 2).reshape(1, ci, 1, 1)
+    w[8:] = (0.5 + 0.01 * torch.rand(8, ci, 1, 1)) * sign
+    w = w.half()
+    x = (torch.rand(2, ci, 5, 5) * 60.0 + 30.0).half()
+    bias = torch.randn(co).half()
+    s_x = 127.0 / x.float().abs().max().item()
+    s_w = 127.0 / w.float().reshape(co, -1).abs().amax(1)
+    q_scale = torch.cat([torch.tensor([s_x, 0.0]), s_w]).half()
+    q_mode = torch.tensor([3], dtype=torch.int32)
+    r = ref_order.conv2d_per_channel(x, w, bias, (0, 0), (1, 1), (1, 1), 1, q_scale, q_mode.numpy())
+    got = torch.ops.torch_mlu.conv2d(x.cuda(), w.cuda(), bias.cuda(), [0, 0], [1, 1], [1, 1], 1, q_scale.cuda(), q_mode.cuda())
+    want = r["y"]
+    assert torch.isinf(want[:, 1:8]).all() and torch.isfinite(want[:, 0]).all() and torch.isfinite(want[:, 8:]).all()
+    assert same_bits(want.contiguous().numpy(), got.cpu().contiguous().numpy())
 
 
 def test_empty_batches():

@@ -97,7 +97,7 @@ def test_quantize_nchw_to_nhwc(shape, cpad, bw):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
-@pytest.mark.parametrize("n", [1, 7, 100000, 4096 * 300 + 3])
+@pytest.mark.parametrize("n", [1, 7, 100000, 4096 * 300 + 3, 4096 * 256 * 4 * 5 + 1029])
 def test_quantize_param(dtype, n):
     note("quantize_param", dtype.__name__, n)
     x = (rng(n).standard_normal(n) * 2.5).astype(dtype)
@@ -144,6 +144,30 @@ def test_dequantize():
         assert same_bits(orc.dequantize(q, -7, 1.7), cabi.dequantize(cabi.dev(q), -7, 1.7).cpu().numpy())
         h = cabi.dequantize(cabi.dev(q), -7, 1.7, half=True).cpu().numpy()
         assert same_bits(orc.dequantize(q, -7, 1.7).astype(np.float16), h)
+
+
+@pytest.mark.parametrize("bits,dtype", [(8, np.int8), (16, np.int16), (32, np.int32)])
+def test_dequantize_vector_paths(bits, dtype):
+    """sizes that run the unrolled vector body several times over plus a ragged tail; every integer of the narrow
+    types; scales that take the reciprocal form of the division (ordinary), the true division (all-ones significand,
+    extreme exponents) and none (1.0); an unaligned view (scalar body)"""
+    note("dequantize vector", bits)
+    r = rng(90 + bits)
+    lim = 2 ** (bits - 1)
+    n = 4096 * 256 * 3 + 11
+    q = r.integers(-lim, lim, n).astype(dtype)
+    if bits <= 16:
+        q[:2 * lim] = np.arange(-lim, lim).astype(dtype)
+    qd = cabi.dev(q)
+    ones = np.frombuffer(np.uint32(0x3fffffff).tobytes(), np.float32)[0]  # 1.9999999: significand all ones
+    for pos, scale in ((-7, 1.0), (3, 1.7), (-20, 0.37), (0, float(ones)), (-7, 3.0e-12), (5, 2.5e11), (-60, 1.25)):
+        want = orc.dequantize(q, pos, scale)
+        assert same_bits(want, cabi.dequantize(qd, pos, scale).cpu().numpy()), (pos, scale)
+        got_h = cabi.dequantize(qd, pos, scale, half=True).cpu().numpy()
+        with np.errstate(over="ignore"):
+            assert same_bits(want.astype(np.float16), got_h), (pos, scale, "half")
+    # views off 16-byte alignment take the scalar body
+    assert same_bits(orc.dequantize(q[1:70001], -3, 1.7), cabi.dequantize(qd[1:70001], -3, 1.7).cpu().numpy())
 
 
 # ------------------------------------------------------------------------------ GEMM
@@ -800,6 +824,51 @@ def test_conv_with_projection_shortcut(case):
     assert same_bits(y, out["y"].cpu().numpy())
 
 
+HEAD_CASES = [
+    # N, H, W, K1 (head input channels), Cm, Co, fused in one launch?
+    (3, 56, 56, 256, 64, 64, True),    # ResNet-50 stage 1, blocks 2 and 3: bands of 4 rows, 11 head sub-tiles
+    (2, 56, 56, 64, 64, 64, True),     # its first block: one K step pair in the head
+    (2, 30, 20, 256, 64, 64, True),    # bands of unequal height (the last one shorter), W not a multiple of 4
+    (5, 17, 33, 64, 64, 64, True),     # odd sizes: ragged sub-tiles in both phases
+    (2, 14, 14, 256, 64, 64, True),    # one band per image: both halo rows lie outside the image
+    (2, 7, 7, 256, 64, 64, False),     # small images go several to a tile: two launches
+    (1, 28, 28, 512, 128, 128, False), # other channel counts: two launches
+    (2, 12, 12, 64, 64, 96, False),
+]
+
+
+@pytest.mark.parametrize("case", HEAD_CASES)
+def test_conv1x1_then_conv3x3(case):
+    """catchq_conv1x1_conv3x3_nhwc against the oracle's two convolutions in sequence: 1x1 (dequant + bias, ReLU,
+    requantized to int8) then 3x3 with padding 1 (the zeros of the padding are zeros of the requantized tensor);
+    int8 and fp32 outputs of the second convolution, bit for bit, with and without planning for a shared device."""
+    n, h, w, k1, cm, co, fused = case
+    note("conv1x1_conv3x3", case)
+    r = rng(sum(case[:6]))
+    x, w1, w2 = _ints(r, (n, h, w, k1), 8), _ints(r, (cm, 1, 1, k1), 8), _ints(r, (co, 3, 3, cm), 8)
+    x[0, 0, :, :] = 127  # the first image row at full scale: what the halo above it must not leak into
+    x[-1, -1, :, :] = -128
+    div1, bias1 = r.uniform(0.6, 3.5, cm).astype(np.float32), r.standard_normal(cm).astype(np.float32) * 4
+    div2, bias2 = r.uniform(0.6, 3.5, co).astype(np.float32), r.standard_normal(co).astype(np.float32)
+    e1, qp1, e2 = {64: -10, 256: -11, 512: -12}[k1], -2, -8
+    acc1, ovf1 = orc.conv2d_nhwc(x, w1, (0, 0), (1, 1), (1, 1), 1)
+    q1 = orc.quantize(orc.epilogue(acc1, e1, div1, bias1, None, 1), 8, qp1)
+    assert ovf1 == 0 and 0 < (q1 == 127).mean() < 0.2 and (q1 == 0).mean() < 0.8  # saturation and ReLU both occur
+    acc2, ovf2 = orc.conv2d_nhwc(q1, w2, (1, 1), (1, 1), (1, 1), 1)
+    assert ovf2 == 0
+    xd, w1d, w2d = cabi.dev(x), cabi.dev(w1.reshape(cm, k1)), cabi.dev(w2)
+    d1, r1, b1 = cabi.dev(div1), cabi.dev(np.float32(1) / div1), cabi.dev(bias1)
+    for act, want_y, sharing in ((1, False, 0), (1, False, 2), (0, True, 0), (2, True, 2)):
+        out, ws_bytes = cabi.conv1x1_conv3x3_nhwc(xd, w1d, e1, d1, r1, b1, qp1, w2d, exp2=e2, chan_div=cabi.dev(div2),
+                                                  bias=cabi.dev(bias2), act=act, y_dtype=torch.float32 if want_y else None,
+                                                  q_bw=8, q_pos=-1, chan_rcp=cabi.dev(np.float32(1) / div2), sharing=sharing)
+        assert (ws_bytes == 0) == fused, ws_bytes
+        y = orc.epilogue(acc2, e2, div2, bias2, None, act)
+        assert same_bits(orc.quantize(y, 8, -1), out["q"].cpu().numpy()), (act, want_y, sharing)
+        if want_y:
+            assert same_bits(y, out["y"].cpu().numpy()), (act, want_y, sharing)
+
+
 CHAIN_CASES = [
     # N, Ho, Wo, Co, shortcut (Cs, stride), main channel counts (one per block)
     (2, 14, 14, 256, (64, 1), (64,)),                  # first block of stage 1: shortcut + one block
@@ -881,6 +950,28 @@ def test_quantize_into_frame():
         want[:, 2:11, 3:14, :3] = orc.quantize(np.transpose(x, (0, 2, 3, 1)), bits, -1)
         got = torch.ops.torch_mlu.quantize_nhwc_frame(cabi.dev(x), bits, -1, cpad, 14, 18, 2, 3)
         assert np.array_equal(want, got.cpu().numpy())
+
+
+@pytest.mark.parametrize("shape,frame", [((3, 3, 10, 12), (2, 3, 1, 4)), ((2, 3, 33, 224), (3, 3, 3, 4)),
+                                         ((5, 1, 7, 260), (0, 1, 2, 0)), ((1, 2, 3, 4), (1, 0, 0, 70)),
+                                         ((2, 3, 224, 224), (3, 3, 3, 4))])
+def test_quantize_into_frame_vector_path(shape, frame):
+    """widths that are multiples of 4 (fp32 -> int8, 4 channels per pixel) take the kernel that moves 4 pixels per
+    lane: rows of more than 64 groups, odd numbers of rows, frames with no border on a side, a border wider than a
+    wave, 1 to 3 channels; the output buffer is pre-filled so that an unwritten border pixel shows"""
+    note("quantize frame vector", shape, frame)
+    n, c, h, w = shape
+    top, left, bottom, right = frame
+    r = rng(sum(shape) + sum(frame))
+    x = (r.standard_normal(shape) * 50).astype(np.float32)
+    x[0, 0, 0, :4] = (np.nan, np.inf, -np.inf, 0.5)
+    oh, ow = h + top + bottom, w + left + right
+    want = np.zeros((n, oh, ow, 4), np.int8)
+    want[:, top:top + h, left:left + w, :c] = orc.quantize(np.transpose(x, (0, 2, 3, 1)), 8, -1)
+    q = torch.full((n, oh, ow, 4), 77, dtype=torch.int8, device="cuda")
+    cabi.check(cabi.lib().catchq_quantize_nchw_to_nhwc_frame(cabi.ptr(cabi.dev(x)), cabi.F32, cabi.ptr(q), 8, n, c, h, w, 4,
+                                                             oh, ow, top, left, -1, 1.0, cabi.stream()))
+    assert np.array_equal(want, q.cpu().numpy())
 
 
 def test_error_statuses():

@@ -37,14 +37,25 @@ def test_library_exports_every_declared_symbol(lib):
     assert lib.catchq_status_string(2) == b"quantify only support input float/half"
 
 
-def test_launch_sharing_hint(lib):
-    """process-wide planning hint: returns the previous value, rejects counts below one, changes the tile a route
-    reports nothing about (results never depend on it: the GPU suite runs graphs recorded with 1, 2, 3 and 4)"""
-    assert lib.catchq_set_launch_sharing(1) >= 1
-    assert lib.catchq_set_launch_sharing(4) == 1
-    assert lib.catchq_set_launch_sharing(2) == 4
-    assert lib.catchq_set_launch_sharing(0) < 0 and lib.catchq_set_launch_sharing(-3) < 0
-    assert lib.catchq_set_launch_sharing(1) == 2  # the rejected calls left it alone
+def test_launch_sharing_hint_is_per_thread():
+    """the planning hint lives in the calling thread (the kernel library takes it per call and keeps nothing):
+    the op returns the previous value, rejects counts below one, and another thread sees its own default
+    (results never depend on it: the GPU suite runs graphs recorded with 1, 2, 3 and 4)"""
+    import threading
+    import catch_amd  # noqa: F401
+    op = torch.ops.torch_mlu.set_launch_sharing
+    assert op(1) >= 1
+    assert op(4) == 1
+    assert op(2) == 4
+    for bad in (0, -3):
+        with pytest.raises(Exception):
+            op(bad)
+    seen = []
+    th = threading.Thread(target=lambda: seen.append((op(3), op(1))))
+    th.start()
+    th.join()
+    assert seen == [(1, 3)]      # the other thread started from the default and changed only its own value
+    assert op(1) == 2            # this thread's value survived the rejected calls and the other thread
 
 
 def test_torch_ops_are_registered():
