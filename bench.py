@@ -309,9 +309,9 @@ def run_probe(args):
     elif what.startswith("gemm:"):
         m, n, k = (int(v) for v in what[5:].split("x"))
         a, b, exp2, div, bias = gaussian_linear_operands(m, n, k)
-        for _ in range(it):
-            ops.qlinear(a, b, exp2, div, bias, 1, True, True, False, 0, 0, 1.0)
-        desc = "int8 GEMM %dx%dx%d, per-channel dequant + bias + ReLU, fp16 out" % (m, n, k)
+        t = event_time(lambda: ops.qlinear(a, b, exp2, div, bias, 1, True, True, False, 0, 0, 1.0), it, 3)
+        desc = "int8 GEMM %dx%dx%d, per-channel dequant + bias + ReLU, fp16 out: %.1f us per launch, %.1f TOPS" % (
+            m, n, k, t * 1e6, 2 * m * n * k / t / 1e12)
     elif what == "mfma":
         print(json.dumps({"probe": what, "mfma_ceiling": mfma_ceiling(seconds=2.0)}))
         return

@@ -13,6 +13,8 @@ int gemm_nt_mfma_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t 
                     hipStream_t s);
 int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph,
                    int pw, int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
+int conv2d_mfma_i8_grouped(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
+                           int sh, int sw, int dh, int dw, int Ho, int Wo, int groups, const EpiDev &e, hipStream_t s);
 int gemm_nt_mfma_a16(const void *a, const void *b, int64_t M, int64_t N, int64_t K, const EpiDev &e, hipStream_t s);
 int conv2d_mfma_a16(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
                     int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -41,7 +43,7 @@ bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
 
-enum Route { kDirect, kMfma, kMfmaA16, kMfmaA16W16, kDepthwise, kBad };
+enum Route { kDirect, kMfma, kMfmaGrouped, kMfmaA16, kMfmaA16W16, kDepthwise, kBad };
 
 static Route gemm_route(int a_bits, int b_bits, int64_t m, int64_t n, int64_t k, const void *a, const void *b) {
   if (a_bits == 8 && b_bits == 8 && k % 16 == 0 && k >= 16 && m > 0 && n > 0 && k < (1ll << 31) &&
@@ -65,6 +67,11 @@ static Route conv_route(int x_bits, int w_bits, const catchq_conv_desc_t *d, con
         dwconv_i8_supported(d->ci, d->kh, d->kw, d->stride_w, d->dil_w) && (!x || aligned16(x)))
       return kDepthwise;
     if (d->groups == 1 && d->ci % 16 == 0 && (!x || aligned16(x)) && (!w || aligned16(w))) return kMfma;
+    // grouped, not depthwise: one implicit GEMM per group when a group's channels fill whole 16-byte K chunks
+    if (d->groups > 1 && d->groups < 65536 && (d->ci / d->groups) % 16 == 0 && (d->co / d->groups) % 4 == 0 &&
+        d->kh * d->kw <= 32 && (int64_t)d->n * d->h * d->w * d->ci < (1ll << 31) &&
+        (int64_t)d->co * d->kh * d->kw * (d->ci / d->groups) < (1ll << 31) && (!x || aligned16(x)) && (!w || aligned16(w)))
+      return kMfmaGrouped;
     // four-channel inputs (an RGB image padded to 4): one pixel per dword
     if (d->groups == 1 && d->ci == 4 && d->dil_w == 1 && (!x || aligned16(x)) && (!w || aligned16(w))) return kMfma;
   }
@@ -82,6 +89,7 @@ static Route conv_route(int x_bits, int w_bits, const catchq_conv_desc_t *d, con
 static const char *route_name(Route r) {
   switch (r) {
     case kMfma: return "mfma";
+    case kMfmaGrouped: return "mfma_grouped";
     case kMfmaA16: return "mfma_a16";
     case kMfmaA16W16: return "mfma_a16w16";
     case kDepthwise: return "depthwise";
@@ -161,6 +169,12 @@ CATCHQ_API int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int 
     case kMfma:
       return conv2d_mfma_i8(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h,
                             d.stride_w, d.dil_h, d.dil_w, ho, wo, e, s);
+    case kMfmaGrouped: {
+      const int st2 = conv2d_mfma_i8_grouped(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h,
+                                             d.stride_w, d.dil_h, d.dil_w, ho, wo, d.groups, e, s);
+      if (st2 >= 0) return st2;
+      break;  // not eligible after all (e.g. 2^31 output pixels): the direct kernel
+    }
     case kMfmaA16: {
       const int st2 = conv2d_mfma_a16(x, w, d.n, d.h, d.w, d.ci, d.co, d.kh, d.kw, d.pad_h, d.pad_w, d.stride_h,
                                       d.stride_w, d.dil_h, d.dil_w, ho, wo, e, s);

@@ -21,18 +21,6 @@
 
 namespace catchq {
 
-// 16 consecutive int16 (two 16-byte chunks) -> their high bytes and their biased low bytes
-__device__ __forceinline__ void split_i16(const v4i c0, const v4i c1, v4i &hi, v4i &lo) {
-  hi[0] = (int)__builtin_amdgcn_perm((unsigned)c0[1], (unsigned)c0[0], 0x07050301u);
-  hi[1] = (int)__builtin_amdgcn_perm((unsigned)c0[3], (unsigned)c0[2], 0x07050301u);
-  hi[2] = (int)__builtin_amdgcn_perm((unsigned)c1[1], (unsigned)c1[0], 0x07050301u);
-  hi[3] = (int)__builtin_amdgcn_perm((unsigned)c1[3], (unsigned)c1[2], 0x07050301u);
-  lo[0] = (int)(__builtin_amdgcn_perm((unsigned)c0[1], (unsigned)c0[0], 0x06040200u) ^ 0x80808080u);
-  lo[1] = (int)(__builtin_amdgcn_perm((unsigned)c0[3], (unsigned)c0[2], 0x06040200u) ^ 0x80808080u);
-  lo[2] = (int)(__builtin_amdgcn_perm((unsigned)c1[1], (unsigned)c1[0], 0x06040200u) ^ 0x80808080u);
-  lo[3] = (int)(__builtin_amdgcn_perm((unsigned)c1[3], (unsigned)c1[2], 0x06040200u) ^ 0x80808080u);
-}
-
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int LOAD, int EPI>
 __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void igemm_a16_dma_kernel(const int16_t *__restrict__ A,
                                                                             const int8_t *__restrict__ B,

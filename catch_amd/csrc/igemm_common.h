@@ -23,7 +23,16 @@ struct IgemmParams {
   // instead of streaming the whole B operand past every row tile.
   int group_m;
   int tiles_m;
+  // Leading dimension of the output matrices (y, q, acc_out, resid); 0 = N.  A grouped convolution runs one GEMM per
+  // group (grid dimension y) whose N is the group's share of the output channels while the rows stay Co apart.
+  int ldc;
+  // groups > 1: per-group offsets -- bytes into the activation tensor (a pixel's channel slice), bytes into the
+  // weights (the group's filters) and output channels (columns of the outputs and entries of the per-channel vectors)
+  int groups, a_group_bytes, n_group;
+  int64_t b_group_bytes;
 };
+
+__device__ __forceinline__ int out_ld(const IgemmParams &p) { return p.ldc ? p.ldc : p.N; }
 
 constexpr int BK = 64;  // bytes of K per pipeline step (one LDS row)
 enum { LOAD_GEMM = 0, LOAD_CONV = 1, LOAD_C4 = 2 };
@@ -329,14 +338,14 @@ __device__ __forceinline__ void igemm_epilogue_vec(v16i (&acc)[TM][TN], int *sta
   constexpr int NIT = 32 / RPI;
   const int cg = lane % CPR, rsub = lane / CPR;
   const bool use_res = L.use_res;
-  const unsigned lane_off0 = (unsigned)rsub * (unsigned)p.N + (unsigned)(cg * 4);
-  const unsigned it_step = (unsigned)RPI * (unsigned)p.N;
+  const unsigned lane_off0 = (unsigned)rsub * (unsigned)out_ld(p) + (unsigned)(cg * 4);
+  const unsigned it_step = (unsigned)RPI * (unsigned)out_ld(p);
   auto tile = [&](auto full_c) {
     constexpr bool FULL = decltype(full_c)::value;
     const bool n_ok = FULL || (n_w + cg * 4 < p.N);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int64_t uni = (m_w + i * 32) * (int64_t)p.N + n_w;
+      const int64_t uni = (m_w + i * 32) * (int64_t)out_ld(p) + n_w;
       const int64_t left = p.M - (m_w + i * 32);
       const int rows = FULL ? 32 : (left < 0 ? 0 : (left > 32 ? 32 : (int)left));  // uniform
       // Opaque copy: a kernel that calls this in a loop would otherwise keep every iteration's byte
@@ -407,8 +416,8 @@ __device__ __forceinline__ void igemm_epilogue_dual(v16i (&acc)[TM][TN], v16i (&
   EpiDev e_sc = {};
   e_sc.exp2 = sc.exp2; e_sc.chan_div = sc.chan_div; e_sc.chan_rcp = sc.chan_rcp; e_sc.bias = sc.bias;
   const EpiLane L_sc = epi_lane_setup<EpiGeneric>(n, n_ok, e_sc);
-  const unsigned lane_off = (unsigned)rsub * (unsigned)p.N + (unsigned)(cg * 4);
-  const unsigned it_step = (unsigned)RPI * (unsigned)p.N;
+  const unsigned lane_off = (unsigned)rsub * (unsigned)out_ld(p) + (unsigned)(cg * 4);
+  const unsigned it_step = (unsigned)RPI * (unsigned)out_ld(p);
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     // shortcut sums -> fp32 residual values in the row-major layout of the stores
@@ -430,7 +439,7 @@ __device__ __forceinline__ void igemm_epilogue_dual(v16i (&acc)[TM][TN], v16i (&
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         stage[(8 * (r >> 2) + 4 * fhalf + (r & 3)) * EPI_STRIDE + j * 32 + frow] = acc[i][j][r];
-    const int64_t uni = (m_w + i * 32) * (int64_t)p.N + n_w;
+    const int64_t uni = (m_w + i * 32) * (int64_t)out_ld(p) + n_w;
     const int64_t left = p.M - (m_w + i * 32);
     const int rows = left < 0 ? 0 : (left > 32 ? 32 : (int)left);
     v4i av[32 / RPI];
@@ -463,7 +472,7 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
         for (int r = 0; r < 16; ++r) {
           const int64_t m = m_w + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
           if (m >= p.M) continue;
-          const int64_t idx = m * p.N + n;
+          const int64_t idx = m * out_ld(p) + n;
           const int a = acc[i][j][r];
           if (e.acc_out) e.acc_out[idx] = a;
           epi_store(epi_value((float)a, idx, n, e), idx, e);
@@ -475,6 +484,18 @@ __device__ __forceinline__ void igemm_epilogue(v16i (&acc)[TM][TN], int *stage, 
     const EpiLane L = epi_lane_setup<S>(n, n < p.N, e);
     igemm_epilogue_vec<TM, TN, EPI, true, BATCHES>(acc, stage, m_w, n_w, lane, p, e, L);
   }
+}
+
+// 16 consecutive int16 (two 16-byte chunks) -> their high bytes and their biased low bytes
+__device__ __forceinline__ void split_i16(const v4i c0, const v4i c1, v4i &hi, v4i &lo) {
+  hi[0] = (int)__builtin_amdgcn_perm((unsigned)c0[1], (unsigned)c0[0], 0x07050301u);
+  hi[1] = (int)__builtin_amdgcn_perm((unsigned)c0[3], (unsigned)c0[2], 0x07050301u);
+  hi[2] = (int)__builtin_amdgcn_perm((unsigned)c1[1], (unsigned)c1[0], 0x07050301u);
+  hi[3] = (int)__builtin_amdgcn_perm((unsigned)c1[3], (unsigned)c1[2], 0x07050301u);
+  lo[0] = (int)(__builtin_amdgcn_perm((unsigned)c0[1], (unsigned)c0[0], 0x06040200u) ^ 0x80808080u);
+  lo[1] = (int)(__builtin_amdgcn_perm((unsigned)c0[3], (unsigned)c0[2], 0x06040200u) ^ 0x80808080u);
+  lo[2] = (int)(__builtin_amdgcn_perm((unsigned)c1[1], (unsigned)c1[0], 0x06040200u) ^ 0x80808080u);
+  lo[3] = (int)(__builtin_amdgcn_perm((unsigned)c1[3], (unsigned)c1[2], 0x06040200u) ^ 0x80808080u);
 }
 
 // launchers of the LDS-DMA pipelined kernel (igemm_i8_dma.hip); return -1 when the shape is not

@@ -327,6 +327,27 @@ int gemm_nt_mfma_i8(const void *a, const void *b, int64_t M, int64_t N, int64_t 
   return pick_tile<LOAD_GEMM>(a, b, p, e, s);
 }
 
+// Grouped convolution (groups > 1, a multiple of 16 input channels and of 4 output channels per group): one implicit
+// GEMM per group, the group index on the grid's second dimension; -1 when the shape is not eligible
+int conv2d_mfma_i8_grouped(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph, int pw,
+                           int sh, int sw, int dh, int dw, int Ho, int Wo, int groups, const EpiDev &e, hipStream_t s) {
+  const int cig = Ci / groups, cog = Co / groups;
+  if (groups < 2 || groups > 65535 || cig % 16 != 0 || cog % 4 != 0 || kh * kw > 32) return -1;
+  IgemmParams p = {};
+  p.M = (int64_t)N * Ho * Wo;
+  p.N = cog;
+  p.H = H; p.W = W; p.Ci = cig; p.Ho = Ho; p.Wo = Wo;
+  p.kh = kh; p.kw = kw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+  p.K = kh * kw * cig;
+  p.img_stride = (unsigned)(H * W * Ci); p.row_stride = (unsigned)(W * Ci); p.pix_stride = (unsigned)Ci;
+  p.ldc = Co;
+  p.groups = groups;
+  p.a_group_bytes = cig;
+  p.b_group_bytes = (int64_t)cog * p.K;
+  p.n_group = cog;
+  return igemm_dma_launch(LOAD_CONV, x, w, p, e, (int64_t)N * H * W * Ci, (int64_t)Co * p.K, s);
+}
+
 int conv2d_mfma_i8(const void *x, const void *w, int N, int H, int W, int Ci, int Co, int kh, int kw, int ph,
                    int pw, int sh, int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s) {
   IgemmParams p = {};

@@ -217,8 +217,10 @@ int catchq_conv_out_size(int in, int k, int pad, int stride, int dil);
  * Depthwise layers (is_depthwise_conv, operators/cnnl/convolution_overrideable.cpp:41-54) run a
  * stencil kernel; dense layers an implicit GEMM on the int8 matrix cores: int8 x int8 with ci % 16 == 0,
  * int16 x int8 and int16 x int16 (the reference's quantized_mode 2 / 4, quantify_conv_forward.cpp:90-101) with
- * ci % 8 == 0 as two resp. four int8 digit products; everything else (grouped non-depthwise, odd channel
- * counts) a direct kernel; the arithmetic is the same in all of them. */
+ * ci % 8 == 0 as two resp. four int8 digit products; grouped int8 layers (cnnlConvolutionForward takes every
+ * group count, convolution_forward_internal.cpp:150-173) as one implicit GEMM per group when (ci / groups) % 16 == 0
+ * and (co / groups) % 4 == 0; everything else (other grouped layers, odd channel counts) a direct kernel; the
+ * arithmetic is the same in all of them. */
 int catchq_conv2d_nhwc(const void *x, int x_bits, const void *w, int w_bits, const catchq_conv_desc_t *desc,
                        const catchq_epilogue_t *epilogue, catchq_stream_t stream);
 

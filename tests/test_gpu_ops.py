@@ -157,7 +157,7 @@ def test_conv2d_cnnl_encoding_int16_act_int8_weight():
     assert rel_rms(want, got.cpu().numpy()) <= 0.02
 
 
-@pytest.mark.parametrize("groups,ci,co", [(2, 4, 16), (8, 8, 8), (32, 32, 32)])
+@pytest.mark.parametrize("groups,ci,co", [(2, 4, 16), (8, 8, 8), (32, 32, 32), (2, 64, 64), (4, 64, 80)])  # the last two: one GEMM per group on the matrix cores
 def test_conv2d_groups_and_layouts(groups, ci, co):
     note("conv2d groups", groups, ci, co)
     torch.manual_seed(groups)

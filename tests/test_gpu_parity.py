@@ -453,6 +453,49 @@ def test_conv_i8_acc_and_epilogue(case):
     assert same_bits(orc.epilogue(acc, -10, None, None, None, 2, np.float16), out["y"].cpu().numpy())
 
 
+GROUPED_CASES = [
+    # N, Ci, H, W, Co, k, pad, stride, dil, groups, route
+    (2, 64, 14, 14, 64, 3, 1, 1, 1, 2, "mfma_grouped"),      # two groups of 32 -> 32
+    (1, 64, 9, 11, 80, 3, 1, 2, 1, 4, "mfma_grouped"),       # 16 -> 20 channels per group, stride 2, ragged tiles
+    (2, 256, 14, 14, 256, 3, 1, 1, 1, 8, "mfma_grouped"),    # a wide-group bottleneck: 32 -> 32 per group
+    (1, 128, 20, 20, 64, 1, 0, 1, 1, 2, "mfma_grouped"),     # grouped pointwise
+    (1, 96, 12, 12, 96, 3, 2, 1, 2, 3, "mfma_grouped"),      # dilation 2, three groups of 32
+    (3, 512, 7, 7, 1024, 3, 1, 1, 1, 32, "mfma_grouped"),    # 32 groups of 16 -> 32 (cardinality 32)
+    (1, 128, 8, 8, 128, 3, 1, 1, 1, 32, "direct"),           # 4 channels per group: not a whole K chunk
+    (1, 64, 8, 8, 36, 3, 1, 1, 1, 2, "direct"),              # 18 outputs per group: not a multiple of 4
+]
+
+
+@pytest.mark.parametrize("case", GROUPED_CASES)
+def test_conv_grouped(case):
+    """grouped (not depthwise) int8 convolutions: groups whose channels fill whole 16-byte K chunks run as one
+    implicit GEMM per group on the matrix cores, the rest on the direct kernel; int32 sums, the generic epilogue with
+    every per-channel vector and a residual, and the ReLU -> int8 instance, all against the oracle"""
+    n, ci, h, w, co, k, pad, stride, dil, g, route = case
+    note("conv_grouped", case)
+    assert cabi.conv_route(8, 8, (n, h, w, ci), (co, k, k, ci // g), (pad, pad), (stride, stride), (dil, dil), g) == route
+    r = rng(sum(case[:10]))
+    x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, k, k, ci // g), 8)
+    acc, ovf = orc.conv2d_nhwc(x, wt, (pad, pad), (stride, stride), (dil, dil), g)
+    assert ovf == 0
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = r.standard_normal(co).astype(np.float32)
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    xd, wd = cabi.dev(x), cabi.dev(wt)
+    args = ((pad, pad), (stride, stride), (dil, dil), g)
+    out = cabi.conv2d_nhwc(xd, wd, *args, exp2=-10, chan_div=cabi.dev(div), bias=cabi.dev(bias), resid=cabi.dev(resid), act=1,
+                           q_bw=8, q_pos=-3, chan_rcp=cabi.dev(np.float32(1) / div))
+    assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
+    y = orc.epilogue(acc, -10, div, bias, resid, 1)
+    assert same_bits(y, out["y"].cpu().numpy())
+    assert same_bits(orc.quantize(y, 8, -3), out["q"].cpu().numpy())
+    q = cabi.conv2d_nhwc(xd, wd, *args, exp2=-10, chan_div=cabi.dev(div), chan_rcp=cabi.dev(np.float32(1) / div),
+                         bias=cabi.dev(bias), act=1, y_dtype=None, want_acc=False, q_bw=8, q_pos=-3)["q"]
+    assert same_bits(orc.quantize(orc.epilogue(acc, -10, div, bias, None, 1), 8, -3), q.cpu().numpy())
+    h16 = cabi.conv2d_nhwc(xd, wd, *args, exp2=-10, bias=cabi.dev(bias), act=2, y_dtype=torch.float16, want_acc=False)["y"]
+    assert same_bits(orc.epilogue(acc, -10, None, bias, None, 2, np.float16), h16.cpu().numpy())
+
+
 @pytest.mark.parametrize("case", [CONV_CASES[4], CONV_CASES[17], CONV_CASES[18], CONV_CASES[3]])
 @pytest.mark.parametrize("after", [False, True])
 def test_conv_leaky_relu_and_residual_order(case, after):
@@ -541,6 +584,53 @@ def test_conv3x3_patch_resident(n, h, w, ci, co, stride):
                          bias=cabi.dev(bias), act=1, y_dtype=None, want_acc=False, q_bw=8, q_pos=-3)["q"]
     want = orc.quantize(orc.epilogue(acc, -14, div, bias, None, 1), 8, -3)
     assert same_bits(want, q.cpu().numpy())
+
+
+@pytest.mark.parametrize("n,h,w,ci,co", [
+    (2, 52, 52, 128, 256),    # Darknet-53's widest 3x3 family
+    (1, 104, 104, 64, 128),
+    (1, 60, 208, 32, 64),     # K = 288
+    (2, 26, 26, 256, 512),
+    (3, 13, 13, 128, 100),    # ragged channel block
+    (5, 7, 7, 64, 32),        # odd batch of small images
+    (2, 9, 31, 32, 68),       # odd width, Co % 32 != 0
+    (1, 1, 1, 64, 64),        # a single pixel
+    (1, 6, 254, 32, 32),      # long rows
+])
+def test_conv3x3_int16_detector_epilogues(n, h, w, ci, co):
+    """3x3 / stride 1 / padding 1 layers of int16 activations x int8 weights at the detector's shapes: int32 sums
+    and the generic epilogue against the oracle (extreme digits in both operands and at the image corners), then the
+    detector's epilogue instances: leaky ReLU -> int16, with the residual behind the activation, with and without fp32"""
+    note("conv3x3 int16", n, h, w, ci, co)
+    r = rng(n * 1000 + h * 10 + ci + co)
+    # values of a few thousand: the int32 sums of 9 * ci products stay exact
+    x = (_ints(r, (n, h, w, ci), 16) // (16 if ci <= 64 else 32)).astype(np.int16)
+    wt = _ints(r, (co, 3, 3, ci), 8)
+    ext = np.array([-1, 0, 127, 128, 255, 256, -128, -129, -256, -257, 1023, -1024], np.int16)
+    x[0, 0, 0, :ext.size] = ext          # every digit pattern at a corner: the padding must contribute nothing
+    x[-1, -1, -1, :ext.size] = ext[::-1]
+    wt[0, :, :, 0] = -128
+    wt[-1, :, :, -1] = 127
+    acc, ovf = orc.conv2d_nhwc(x, wt, (1, 1), (1, 1), (1, 1), 1)
+    assert ovf == 0
+    xd, wd = cabi.dev(x), cabi.dev(wt)
+    assert cabi.conv_route(16, 8, (n, h, w, ci), (co, 3, 3, ci), (1, 1), (1, 1), (1, 1), 1) == "mfma_a16"
+    bias = r.standard_normal(co).astype(np.float32)
+    div = r.uniform(0.5, 2.0, co).astype(np.float32)
+    out = cabi.conv2d_nhwc(xd, wd, (1, 1), (1, 1), exp2=-20, chan_div=cabi.dev(div), bias=cabi.dev(bias))
+    assert same_bits(acc.astype(np.int32), out["acc"].cpu().numpy())
+    assert same_bits(orc.epilogue(acc, -20, div, bias), out["y"].cpu().numpy())
+    resid = r.standard_normal(acc.shape).astype(np.float32)
+    for with_resid, want_y in ((False, False), (True, False), (True, True)):
+        if co % 4:
+            break  # the instances are vector epilogues
+        o = cabi.conv2d_nhwc(xd, wd, (1, 1), (1, 1), exp2=-20, bias=cabi.dev(bias), resid=cabi.dev(resid) if with_resid else None,
+                             act=3, y_dtype=torch.float32 if want_y else None, want_acc=False, q_bw=16, q_pos=-9,
+                             act_slope=0.1, resid_after_act=True)
+        y = orc.epilogue(acc, -20, None, bias, resid if with_resid else None, 3, act_slope=0.1, resid_after_act=True)
+        assert same_bits(orc.quantize(y, 16, -9), o["q"].cpu().numpy()), (with_resid, want_y)
+        if want_y:
+            assert same_bits(y, o["y"].cpu().numpy())
 
 
 @pytest.mark.parametrize("bits", [(8, 8), (16, 8), (16, 16)])
