@@ -245,6 +245,33 @@ def test_standalone_linear_full_size_with_its_epilogue(m, n, k):
     assert torch.equal(torch.relu(y32).half(), y)
 
 
+@pytest.mark.parametrize("m,n,k", [(4096, 2048, 2048), (4000, 2304, 2128), (8192, 8192, 8192)])
+def test_big_gemm_with_the_operands_in_separate_rings(m, n, k):
+    """int8 GEMMs large enough for the 256 x 256 tile with long K, whose operands travel through rings of their own
+    (two A slots, three B slots): the int32 sums and the fp32 epilogue on row blocks at the top, the middle, the
+    ragged bottom and at random against the oracle; K ending inside a 128-byte step; uniformly random bytes (every
+    digit pattern, sums near the int32 limits for the largest K)"""
+    note("big gemm", m, n, k)
+    r = np.random.default_rng(m + n + k)
+    lim = 128 if k <= 4096 else 64  # the int32 sum of 8192 products of full-range bytes could overflow
+    a = r.integers(-lim, lim, (m, k)).astype(np.int8)
+    b = r.integers(-128, 128, (n, k)).astype(np.int8)
+    a[0, :], a[-1, :] = lim - 1, -lim
+    b[0, :], b[-1, :] = 127, -128
+    div = r.uniform(0.6, 3.5, n).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    import cabi
+    out = cabi.gemm_nt(cabi.dev(a), cabi.dev(b), exp2=-12, chan_div=cabi.dev(div), bias=cabi.dev(bias), act=0,
+                       y_dtype=torch.float32, want_acc=True, chan_rcp=cabi.dev(np.float32(1) / div))
+    acc_g, y_g = out["acc"].cpu().numpy(), out["y"].cpu().numpy()
+    starts = [0, m // 2 - 32, m - 64] + [int(v) for v in r.integers(0, m - 64, 2)]
+    for s in starts:
+        rows = slice(s, s + 64)
+        acc, ovf = orc.gemm_nt(a[rows], b)
+        assert ovf == 0 and np.array_equal(acc.astype(np.int32), acc_g[rows]), "rows %d.." % s
+        assert np.array_equal(orc.epilogue(acc, -12, div, bias).view(np.uint32), y_g[rows].view(np.uint32)), "rows %d.." % s
+
+
 def test_darknet53_yolov3_fp16_heads_at_416():
     """Darknet-53 + YOLOv3 heads, one 3 x 416 x 416 U(0,1) image, int16 activations x int8 weights, fp16
     outputs at the 13 / 26 / 52 grids: the heads the plan stores in half precision equal the oracle's fp32 head
