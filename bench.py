@@ -50,6 +50,8 @@ def parse():
                     help="parts the batch is split into inside the HIP graph, each on a stream of its own (1: one launch sequence)")
     ap.add_argument("--chain-links", type=int, default=-1,
                     help="longest residual chain recomputed inside a block's last launch (0: none, -1: the plan's own rule)")
+    ap.add_argument("--fuse-blocks", action="store_true",
+                    help="inverted-residual blocks as one launch each where the kernel serves the shape (A/B runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -92,8 +94,13 @@ def layer_profile(fused, x, iters=20, only=None):
     torch.cuda.synchronize()
     fused_heads = set(h.name for h in fused.head_of.values()
                       if fused.head_fuses(h, *trace[h.name]["qx"].shape[:3]))
+    fused_inner = set()  # expansion and depthwise layers that run inside their block's projection launch
+    for pname, (bx, bd) in fused.block_of.items():
+        if fused.block_fuses(next(l for l in fused.layers if l.name == pname), *trace[bx.name]["qx"].shape[:3]):
+            fused_inner.update((bx.name, bd.name))
     for l in fused.layers:
-        if l.kind not in ("conv", "fc") or l.name in fused._fused_away or l.name in fused_heads or (only and l.name != only):
+        if l.kind not in ("conv", "fc") or l.name in fused._fused_away or l.name in fused_heads or l.name in fused_inner \
+                or (only and l.name != only):
             continue
         lq = fused.q[l.name]
         qx = trace[l.name].get("qx_dev", trace[l.name]["qx"])  # the tensor the kernel reads
@@ -104,7 +111,24 @@ def layer_profile(fused, x, iters=20, only=None):
         chain = fused.chain_of.get(l.name) if l.kind == "conv" else None
         extra_macs = extra_bytes = 0
         head = fused.head_of.get(l.name) if l.kind == "conv" else None
-        if head is not None and head.name in fused_heads:
+        block = fused.block_of.get(l.name) if l.kind == "conv" else None
+        if block is not None and block[0].name in fused_inner:
+            # expansion and depthwise layer run inside this launch: the block input and all three filter sets are read,
+            # neither hidden tensor is stored
+            bx, bd = block
+            xq, dq = fused.q[bx.name], fused.q[bd.name]
+            hx = trace[bx.name]["qx"]
+            resid = torch.zeros_like(trace[l.name]["y"]) if l.add else None
+            extra_macs = trace[bx.name]["y"].numel() * xq.qw.shape[-1] + trace[bd.name]["y"].numel() * 9
+            extra_bytes = hx.numel() + xq.qw.numel() + dq.qw.numel() - qx.numel()
+            code = {"none": 0, "relu": 1, "relu6": 2, "leaky": 3}
+
+            def run(l=l, lq=lq, xq=xq, dq=dq, hx=hx, bx=bx, bd=bd, qd=qd, want_y=want_y, resid=resid):
+                return ops.qconv2d_irb(hx, xq.qw, xq.exp2, xq.chan_div, xq.bias, code[bx.act], dq.pos_x, dq.qw, bd.stride,
+                                       dq.exp2, dq.chan_div, dq.bias, code[bd.act], lq.pos_x, lq.qw, lq.exp2, lq.chan_div,
+                                       lq.bias, resid, want_y, y_half, qd[0] if qd else 0, qd[1] if qd else 0, 1.0)
+            route = "mfma+block"
+        elif head is not None and head.name in fused_heads:
             # the 1x1 layer in front runs inside this launch: its input and filters are read, its output never stored
             hq = fused.q[head.name]
             hx = trace[head.name]["qx"]
@@ -194,6 +218,10 @@ def plan_launches(fused, n, h, w):
             shape[l.name] = (ho, wo)
             if l.name in fused._fused_away or fused.head_fuses(l, n, hi, wi):
                 continue
+            if l.name in fused._block_inner:
+                bp = next(m for m in fused.layers if m.name == fused._block_inner[l.name])
+                if fused.block_fuses(bp, n, *shape[fused.block_of[bp.name][0].src]):
+                    continue
             lq = fused.q[l.name]
             n_out = n * ho * wo * fused.cdev[l.name]
             ih, iw = shape[("input", "q")] if (fused.stem and l.name == fused.stem["name"]) else (hi, wi)
@@ -207,6 +235,13 @@ def plan_launches(fused, n, h, w):
                 hq = fused.q[head.name]
                 macs += n * hi * wi * fused.cdev[head.name] * hq.qw.shape[-1]
                 b += n * hi * wi * (fused.cdev[head.src] - fused.cdev[l.src]) + hq.qw.numel()
+            block = fused.block_of.get(l.name)
+            if block is not None and fused.block_fuses(l, n, *shape[block[0].src]):
+                bx, bd = block
+                xq, dq = fused.q[bx.name], fused.q[bd.name]
+                bh, bw = shape[bx.src]
+                macs += n * bh * bw * fused.cdev[bx.name] * xq.qw.shape[-1] + n * ho * wo * fused.cdev[bd.name] * 9
+                b += n * bh * bw * fused.cdev[bx.src] - n * hi * wi * fused.cdev[l.src] + xq.qw.numel() + dq.qw.numel()
             if chain is not None:
                 # every earlier link of the residual chain is recomputed inside this launch: its int8 input (the
                 # pixels the 1x1 taps touch) and its weights are read, its 2*K operations per output repeated
@@ -449,7 +484,8 @@ def build_workload(args):
             sys.exit("--fractional-scale needs a checkpoint of scales; the detector's holds bit widths and positions")
         what += ", position + fractional scale"
     fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale,
-                              chain_links=None if args.chain_links < 0 else args.chain_links)
+                              chain_links=None if args.chain_links < 0 else args.chain_links,
+                              fuse_blocks=getattr(args, "fuse_blocks", False))
     if args.streams < 1:
         sys.exit("--streams must be at least 1")
     while batch % args.streams:  # the largest number of equal parts not above what was asked for
@@ -506,7 +542,10 @@ def main():
               # blocks whose residual branch is recomputed from int8 tensors inside their last launch: links per launch
               "residual_chains": {n: len(c) for n, c in fused.chain_of.items()},
               # 3x3 layers whose launch also computes the 1x1 layer in front of them
-              "fused_heads": sorted(n for n, h in fused.head_of.items() if fused.head_fuses(h, batch // args.streams, *head_hw(fused, h, side)))}
+              "fused_heads": sorted(n for n, h in fused.head_of.items() if fused.head_fuses(h, batch // args.streams, *head_hw(fused, h, side))),
+              "fused_blocks": sorted(n for n, (bx, bd) in fused.block_of.items()
+                                     if fused.block_fuses(next(l for l in fused.layers if l.name == n), batch // args.streams,
+                                                          *head_hw(fused, bx, side)))}
     metric = ("int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
               else "int8 %s images/sec" % args.workload)
     if args.graph_only:

@@ -31,6 +31,13 @@ class PointwiseHead(ctypes.Structure):
                 ("chan_rcp", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("q_position", ctypes.c_int)]
 
 
+class RequantStage(ctypes.Structure):
+    """struct catchq_requant_stage"""
+    _fields_ = [("w", ctypes.c_void_p), ("exp2", ctypes.c_int), ("chan_div", ctypes.c_void_p),
+                ("chan_rcp", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("act", ctypes.c_int),
+                ("q_position", ctypes.c_int)]
+
+
 class ConvDesc(ctypes.Structure):
     """struct catchq_conv_desc"""
     _fields_ = [(n, ctypes.c_int) for n in ("n", "h", "w", "ci", "co", "kh", "kw", "pad_h", "pad_w", "stride_h",
@@ -88,6 +95,11 @@ SIGNATURES = {
                                                    ctypes.POINTER(Epilogue), ctypes.POINTER(_SZ)]),
     "catchq_conv1x1_conv3x3_nhwc": (_I, [_P, ctypes.POINTER(PointwiseHead), _P, ctypes.POINTER(ConvDesc),
                                          ctypes.POINTER(Epilogue), _P, _SZ, _P]),
+    "catchq_inverted_residual_workspace_size": (_I, [_I, _I, _I, _I, _I, _I, _I, ctypes.POINTER(RequantStage),
+                                                     ctypes.POINTER(RequantStage), ctypes.POINTER(Epilogue),
+                                                     ctypes.POINTER(_SZ)]),
+    "catchq_inverted_residual_nhwc": (_I, [_P, _I, _I, _I, _I, _I, _I, _I, ctypes.POINTER(RequantStage),
+                                           ctypes.POINTER(RequantStage), _P, ctypes.POINTER(Epilogue), _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
     "catchq_diag_mfma_i8_loop": (_I, [_P, _I, _I, _P, _P]),

@@ -39,6 +39,9 @@ bool conv2d_head_halo_i8_ok(int N, int H, int W, int K1, int Cm, int Co);
 int conv2d_head_halo_i8(const void *x, int K1, const void *w1, const float *div1, const float *rcp1, const float *bias1,
                         int exp2_1, int q_position1, const void *w, int N, int H, int W, int Cm, int Co, const EpiDev &e,
                         hipStream_t s);
+bool irb_i8_ok(int N, int H, int W, int Cin, int hid, int Co, int S, int cus);
+int irb_i8(const void *x, int N, int H, int W, int Cin, int hid, int Co, int S, const IrbStageDev &s1, const IrbStageDev &s2,
+           const void *w3, const EpiDev &e, hipStream_t s);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -382,6 +385,95 @@ CATCHQ_API int catchq_conv1x1_conv3x3_nhwc(const void *x, const catchq_pointwise
 }
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+// shapes and constants the inverted-residual kernel serves (pointer alignment and the epilogue are checked at the call)
+static bool irb_fusable(int n, int h, int w, int ci, int hid, int co, int stride, const catchq_requant_stage_t *s1,
+                        const catchq_requant_stage_t *s2, const catchq_epilogue_t *e) {
+  auto stage_ok = [](const catchq_requant_stage_t *s) {
+    return s->chan_div && s->chan_rcp && s->bias && s->exp2 >= -64 && s->exp2 <= 64;
+  };
+  return stage_ok(s1) && stage_ok(s2) && !e->exp2_dev[0] && !e->exp2_dev[1] && !e->acc_out &&
+         irb_i8_ok(n, h, w, ci, hid, co, stride, planned_cus(e->sharing));
+}
+
+static int check_irb(int n, int h, int w, int ci, int hid, int co, int stride, const catchq_requant_stage_t *s1,
+                     const catchq_requant_stage_t *s2, const catchq_epilogue_t *e) {
+  if (!s1 || !s2) return CATCHQ_ERR_ARG;
+  if (n < 0 || h <= 0 || w <= 0 || ci <= 0 || hid <= 0 || co <= 0 || stride <= 0) return CATCHQ_ERR_SHAPE;
+  const int st = check_epi(e);
+  if (st != CATCHQ_OK) return st;
+  for (const catchq_requant_stage_t *s : {s1, s2}) {
+    if (s->act != CATCHQ_ACT_RELU && s->act != CATCHQ_ACT_RELU6) return CATCHQ_ERR_ARG;
+    if (s->exp2 < -126 || s->exp2 > 126 || s->q_position < -126 || s->q_position > 126) return CATCHQ_ERR_ARG;
+  }
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_inverted_residual_workspace_size(int n, int h, int w, int ci, int hid, int co, int stride,
+                                                       const catchq_requant_stage_t *expand,
+                                                       const catchq_requant_stage_t *depthwise,
+                                                       const catchq_epilogue_t *epilogue, size_t *bytes) {
+  const int st = check_irb(n, h, w, ci, hid, co, stride, expand, depthwise, epilogue);
+  if (st != CATCHQ_OK) return st;
+  if (!bytes) return CATCHQ_ERR_ARG;
+  const int ho = catchq_conv_out_size(h, 3, 1, stride, 1), wo = catchq_conv_out_size(w, 3, 1, stride, 1);
+  if (ho <= 0 || wo <= 0) return CATCHQ_ERR_SHAPE;
+  *bytes = irb_fusable(n, h, w, ci, hid, co, stride, expand, depthwise, epilogue)
+               ? 0 : round256((size_t)n * h * w * hid) + round256((size_t)n * ho * wo * hid);
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_inverted_residual_nhwc(const void *x, int n, int h, int w, int ci, int hid, int co, int stride,
+                                             const catchq_requant_stage_t *expand, const catchq_requant_stage_t *depthwise,
+                                             const void *w_project, const catchq_epilogue_t *epilogue, void *workspace,
+                                             size_t workspace_bytes, catchq_stream_t stream) {
+  int st = check_irb(n, h, w, ci, hid, co, stride, expand, depthwise, epilogue);
+  if (st != CATCHQ_OK) return st;
+  const int ho = catchq_conv_out_size(h, 3, 1, stride, 1), wo = catchq_conv_out_size(w, 3, 1, stride, 1);
+  if (ho <= 0 || wo <= 0) return CATCHQ_ERR_SHAPE;
+  if (n == 0) return CATCHQ_OK;
+  if (!x || !w_project || !expand->w || !depthwise->w) return CATCHQ_ERR_ARG;
+  if (irb_fusable(n, h, w, ci, hid, co, stride, expand, depthwise, epilogue) && aligned16(x) && aligned16(expand->w) &&
+      aligned16(depthwise->w) && aligned16(w_project) && aligned16(expand->chan_div) && aligned16(expand->chan_rcp) &&
+      aligned16(expand->bias) && aligned16(depthwise->chan_div) && aligned16(depthwise->chan_rcp) && aligned16(depthwise->bias)) {
+    const EpiDev e = make_epi(epilogue, (int64_t)n * ho * wo * co);
+    const IrbStageDev s1 = {(const int8_t *)expand->w, expand->chan_div, expand->chan_rcp, expand->bias, expand->exp2,
+                            -expand->q_position, expand->act == CATCHQ_ACT_RELU6 ? 1 : 0};
+    const IrbStageDev s2 = {(const int8_t *)depthwise->w, depthwise->chan_div, depthwise->chan_rcp, depthwise->bias,
+                            depthwise->exp2, -depthwise->q_position, depthwise->act == CATCHQ_ACT_RELU6 ? 1 : 0};
+    const int st2 = irb_i8(x, n, h, w, ci, hid, co, stride, s1, s2, w_project, e, as_stream(stream));
+    if (st2 >= 0) return st2;
+  }
+  // three launches: the two hidden tensors go through the workspace
+  const size_t b1 = round256((size_t)n * h * w * hid), b2 = round256((size_t)n * ho * wo * hid);
+  if (!workspace || workspace_bytes < b1 + b2 || !aligned16(workspace)) return CATCHQ_ERR_ARG;
+  void *q1 = workspace, *q2 = (char *)workspace + b1;
+  auto stage_epi = [&](const catchq_requant_stage_t *s, void *q) {
+    catchq_epilogue_t es;
+    memset(&es, 0, sizeof(es));
+    es.exp2 = s->exp2;
+    es.chan_div = s->chan_div;
+    es.chan_rcp = s->chan_rcp;
+    es.bias = s->bias;
+    es.act = s->act;
+    es.q = q;
+    es.q_bitwidth = 8;
+    es.q_position = s->q_position;
+    es.q_scale = 1.0f;
+    es.sharing = epilogue->sharing;
+    return es;
+  };
+  const catchq_conv_desc_t d1 = {n, h, w, ci, hid, 1, 1, 0, 0, 1, 1, 1, 1, 1};
+  const catchq_epilogue_t e1 = stage_epi(expand, q1);
+  st = catchq_conv2d_nhwc(x, 8, expand->w, 8, &d1, &e1, stream);
+  if (st != CATCHQ_OK) return st;
+  const catchq_conv_desc_t d2 = {n, h, w, hid, hid, 3, 3, 1, 1, stride, stride, 1, 1, hid};
+  const catchq_epilogue_t e2 = stage_epi(depthwise, q2);
+  st = catchq_conv2d_nhwc(q1, 8, depthwise->w, 8, &d2, &e2, stream);
+  if (st != CATCHQ_OK) return st;
+  const catchq_conv_desc_t d3 = {n, ho, wo, hid, co, 1, 1, 0, 0, 1, 1, 1, 1, 1};
+  return catchq_conv2d_nhwc(q2, 8, w_project, 8, &d3, epilogue, stream);
+}
 
 CATCHQ_API int catchq_quantize_conv2d_workspace_size(const catchq_conv_desc_t *desc, int x_bits, int w_bits,
                                                      size_t *bytes) {

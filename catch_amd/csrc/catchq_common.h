@@ -147,6 +147,14 @@ struct ShortcutDev {
   const float *chan_div, *chan_rcp, *bias;
 };
 
+// An inner stage of a fused block: an int8 convolution whose ReLU / ReLU6 output is requantized to int8 at once
+//   q = sat(rne(act(float(acc) * 2^exp2 / div[c] + bias[c]) * 2^q_neg_pos)),  rcp = correctly rounded reciprocals of div
+struct IrbStageDev {
+  const int8_t *w;
+  const float *div, *rcp, *bias;
+  int exp2, q_neg_pos, relu6;
+};
+
 // out_elems: elements of the output tensor (0: unknown, nothing is streamed)
 inline EpiDev make_epi(const catchq_epilogue_t *e, int64_t out_elems = 0) {
   EpiDev d;

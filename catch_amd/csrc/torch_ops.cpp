@@ -239,6 +239,21 @@ thread_local int t_launch_sharing = 1;
 
 // whether catchq_conv1x1_conv3x3_nhwc serves (1x1: k1 -> cm, then 3x3 / stride 1 / padding 1: cm -> co) over n images of
 // h x w in one launch (per-channel constants with reciprocals and 16-byte aligned tensors assumed)
+bool irb_fuses_op(int64_t n, int64_t h, int64_t w, int64_t ci, int64_t hid, int64_t co, int64_t stride) {
+  float one = 1.0f;
+  catchq_requant_stage_t st;
+  std::memset(&st, 0, sizeof(st));
+  st.w = &one; st.chan_div = st.chan_rcp = st.bias = &one;  // presence only: nothing is dereferenced
+  st.act = CATCHQ_ACT_RELU6;
+  catchq_epilogue_t e;
+  std::memset(&e, 0, sizeof(e));
+  e.q = &one; e.q_bitwidth = 8;
+  e.sharing = t_launch_sharing;
+  size_t bytes = 1;
+  return catchq_inverted_residual_workspace_size((int)n, (int)h, (int)w, (int)ci, (int)hid, (int)co, (int)stride, &st, &st, &e,
+                                                 &bytes) == CATCHQ_OK && bytes == 0;
+}
+
 bool head_fuses_op(int64_t n, int64_t h, int64_t w, int64_t k1, int64_t cm, int64_t co) {
   float one = 1.0f;
   catchq_pointwise_head_t hd;
@@ -555,6 +570,77 @@ std::tuple<Tensor, Tensor> qconv2d_head_op(const Tensor &qx, const Tensor &w1, i
   check_status(catchq_conv1x1_conv3x3_nhwc(qx.data_ptr(), &hd, qw.data_ptr(), &d, &e, ws.data_ptr(), ws_bytes,
                                            current_stream()),
                "torch_mlu::qconv2d_head");
+  return std::make_tuple(o.y, o.q);
+}
+
+// An inverted-residual block (catchq_inverted_residual_nhwc): qx [N,H,W,Ci] int8 NHWC through the 1x1 expansion w1
+// [hid,Ci] (or [hid,1,1,Ci]), the depthwise 3x3 filters wd [hid,3,3] (or [hid,3,3,1]; padding 1, `stride`), both with
+// act1 / act2 (ReLU or ReLU6) and int8 requantization at q_position1 / q_position2, and the 1x1 projection w3 [Co,hid]
+// with the usual epilogue arguments.
+namespace {
+struct StageKeep {
+  catchq_requant_stage_t st;
+  Tensor cd, rcp, bs;
+};
+void fill_stage(StageKeep *k, const Tensor &w, int64_t exp2, const c10::optional<Tensor> &chan_div,
+                const c10::optional<Tensor> &bias, int64_t act, int64_t q_position, int64_t channels, const char *what) {
+  std::memset(&k->st, 0, sizeof(k->st));
+  TORCH_CHECK(exp2 >= -126 && exp2 <= 126, "position sum out of range");
+  k->st.w = w.data_ptr();
+  k->st.exp2 = (int)exp2;
+  k->st.act = (int)act;
+  k->st.q_position = (int)q_position;
+  k->cd = as_f32_vec(chan_div, channels, what);
+  k->bs = as_f32_vec(bias, channels, what);
+  if (k->cd.defined()) {
+    k->st.chan_div = k->cd.data_ptr<float>();
+    k->rcp = reciprocals_for(k->cd);
+    if (k->rcp.defined()) k->st.chan_rcp = k->rcp.data_ptr<float>();
+  }
+  if (k->bs.defined()) k->st.bias = k->bs.data_ptr<float>();
+}
+}  // namespace
+
+std::tuple<Tensor, Tensor> qconv2d_irb_op(const Tensor &qx, const Tensor &w1, int64_t exp2_1,
+                                          const c10::optional<Tensor> &chan_div1, const c10::optional<Tensor> &bias1,
+                                          int64_t act1, int64_t q_position1, const Tensor &wd, int64_t stride, int64_t exp2_2,
+                                          const c10::optional<Tensor> &chan_div2, const c10::optional<Tensor> &bias2,
+                                          int64_t act2, int64_t q_position2, const Tensor &w3, int64_t exp2,
+                                          const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias,
+                                          const c10::optional<Tensor> &resid, bool want_y, bool y_half, int64_t q_bitwidth,
+                                          int64_t q_position, double q_scale) {
+  c10::DeviceGuard guard(qx.device());
+  TORCH_CHECK(qx.dim() == 4 && qx.is_contiguous() && w1.is_contiguous() && wd.is_contiguous() && w3.is_contiguous(),
+              "qconv2d_irb expects contiguous NHWC activations and contiguous filters");
+  TORCH_CHECK(qx.scalar_type() == at::kChar && w1.scalar_type() == at::kChar && wd.scalar_type() == at::kChar &&
+                  w3.scalar_type() == at::kChar,
+              "qconv2d_irb: int8 operands expected");
+  TORCH_CHECK(w1.device() == qx.device() && wd.device() == qx.device() && w3.device() == qx.device(),
+              "qconv2d_irb: operands on different devices");
+  const int64_t n = qx.size(0), h = qx.size(1), w = qx.size(2), ci = qx.size(3), hid = w1.size(0), co = w3.size(0);
+  TORCH_CHECK(w1.numel() == hid * ci, "qconv2d_irb: the expansion's filters must be [", hid, ", ", ci, "]");
+  TORCH_CHECK(wd.size(0) == hid && wd.numel() == hid * 9, "qconv2d_irb: the depthwise filters must be [", hid, ", 3, 3]");
+  TORCH_CHECK(w3.numel() == co * hid, "qconv2d_irb: the projection's filters must be [", co, ", ", hid, "]");
+  TORCH_CHECK(stride >= 1, "bad stride");
+  const int ho = catchq_conv_out_size((int)h, 3, 1, (int)stride, 1), wo = catchq_conv_out_size((int)w, 3, 1, (int)stride, 1);
+  TORCH_CHECK(ho > 0 && wo > 0, "Calculated output size is too small");
+  catchq_epilogue_t e;
+  std::vector<Tensor> keep;
+  EpiOut o = prepare_epilogue(make_args(exp2, chan_div, bias, resid, 0, want_y, y_half, false, q_bitwidth, q_position,
+                                        q_scale, 0.0, false),
+                              {n, ho, wo, co}, co, qx.options(), &e, &keep);
+  StageKeep k1, k2;
+  fill_stage(&k1, w1, exp2_1, chan_div1, bias1, act1, q_position1, hid, "expansion constants");
+  fill_stage(&k2, wd, exp2_2, chan_div2, bias2, act2, q_position2, hid, "depthwise constants");
+  if (n == 0) return std::make_tuple(o.y, o.q);
+  size_t ws_bytes = 0;
+  check_status(catchq_inverted_residual_workspace_size((int)n, (int)h, (int)w, (int)ci, (int)hid, (int)co, (int)stride,
+                                                       &k1.st, &k2.st, &e, &ws_bytes),
+               "torch_mlu::qconv2d_irb");
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, qx.options().dtype(at::kChar));
+  check_status(catchq_inverted_residual_nhwc(qx.data_ptr(), (int)n, (int)h, (int)w, (int)ci, (int)hid, (int)co, (int)stride,
+                                             &k1.st, &k2.st, w3.data_ptr(), &e, ws.data_ptr(), ws_bytes, current_stream()),
+               "torch_mlu::qconv2d_irb");
   return std::make_tuple(o.y, o.q);
 }
 
@@ -1131,6 +1217,10 @@ TORCH_LIBRARY(torch_mlu, m) {
         "int exp2, Tensor? chan_div, Tensor? bias, int[] padding, int[] stride, int[] dilation, int act=0, "
         "bool want_y=True, bool y_half=False, int q_bitwidth=0, int q_position=0, float q_scale=1.0, "
         "float act_slope=0.0) -> (Tensor, Tensor)");
+  m.def("qconv2d_irb(Tensor qx, Tensor w1, int exp2_1, Tensor? chan_div1, Tensor? bias1, int act1, int q_position1, "
+        "Tensor wd, int stride, int exp2_2, Tensor? chan_div2, Tensor? bias2, int act2, int q_position2, Tensor w3, "
+        "int exp2, Tensor? chan_div, Tensor? bias, Tensor? resid, bool want_y=True, bool y_half=False, "
+        "int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> (Tensor, Tensor)");
   m.def("qconv2d_chain(Tensor[] xs, Tensor[] ws, int[] strides, int[] exp2s, Tensor[] chan_divs, Tensor[] biases, "
         "bool want_y=False, int q_bitwidth=8, int q_position=0) -> (Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
@@ -1142,6 +1232,7 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("global_avgpool_nhwc(Tensor x, int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> Tensor");
   m.def("set_launch_sharing(int launches) -> int", &set_launch_sharing_op);
   m.def("conv1x1_conv3x3_fuses(int n, int h, int w, int k1, int cm, int co) -> bool", &head_fuses_op);
+  m.def("inverted_residual_fuses(int n, int h, int w, int ci, int hid, int co, int stride) -> bool", &irb_fuses_op);
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
   m.def("weight_cache_size() -> int", &cache_size_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
@@ -1165,6 +1256,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("qconv2d", &qconv2d_op);
   m.impl("qconv2d_shortcut", &qconv2d_shortcut_op);
   m.impl("qconv2d_head", &qconv2d_head_op);
+  m.impl("qconv2d_irb", &qconv2d_irb_op);
   m.impl("qconv2d_chain", &qconv2d_chain_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);

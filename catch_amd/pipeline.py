@@ -162,7 +162,7 @@ def _decode(layer, sd, device, ci_dev, co_dev, fractional=False):
 
 class FusedNet(object):
     def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True,
-                 fractional_scale=False, chain_links=None, fuse_heads=True):
+                 fractional_scale=False, chain_links=None, fuse_heads=True, fuse_blocks=False):
         """fractional_scale: quantize activations and weights with position and fractional scale -- the
         general form the reference's fused (graph) mode hands to its backend per tensor / per axis
         (jit/utils/utils.cpp:81-167) -- instead of the eager ops' power-of-two steps.
@@ -173,7 +173,13 @@ class FusedNet(object):
         rule (_default_chain_links), 0 switches the recomputation off.
         fuse_heads: a 1x1 convolution + ReLU whose only reader is a 3x3 convolution (the first two layers of a
         bottleneck block) runs inside that convolution's launch where the kernel library serves the shapes
-        (torch_mlu::qconv2d_head); its int8 output is then never stored."""
+        (torch_mlu::qconv2d_head); its int8 output is then never stored.
+        fuse_blocks: an inverted-residual block (1x1 expansion, 3x3 depthwise, 1x1 linear projection, each hidden
+        tensor read by the next layer only) runs as one launch (torch_mlu::qconv2d_irb) where the library's kernel
+        serves the shape and the image is large enough for it to pay (block_fuses).  Off by default: the one-launch
+        kernel is bound by the same vector arithmetic as the three launches, and with the batch in two parts on
+        parallel streams, where one part's launches already fill the other's start-up gaps, MobileNetV2 at batch 128
+        measured 2 % slower with it (one stream: 1.5 % faster)."""
         self.layers = list(layers)
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
@@ -259,6 +265,54 @@ class FusedNet(object):
                         and h.name not in self._fused_away and not (self.stem and self.stem["name"] in (l.name, h.name))):
                     self.head_of[l.name] = h
         self._head_names = set(h.name for h in self.head_of.values())
+        # Inverted-residual blocks: block_of[projection layer name] = (expansion layer, depthwise layer).
+        self.block_of = {}
+        if fuse_blocks:
+            by_name = {l.name: l for l in self.layers}
+
+            def only_reader(a, b):
+                readers = [m for m in self.layers
+                           if m.src == a.name or (isinstance(m.src, tuple) and a.name in m.src) or m.add == a.name]
+                return (readers == [b] and a.name not in self.outputs and not self.f_demand[a.name]
+                        and self.q_demand[a.name] == [(8, self.q[b.name].pos_x, 1.0)])
+
+            def inner_ok(a):
+                aq = self.q[a.name]
+                return (a.act in ("relu", "relu6") and not a.add and (aq.bw_x, aq.bw_w) == (8, 8) and aq.scale_x == 1.0
+                        and aq.chan_div is not None and aq.bias is not None and -64 <= aq.exp2 <= 64
+                        and a.name not in self._fused_away and a.name not in self._head_names
+                        and not (self.stem and self.stem["name"] == a.name))
+            for pl in self.layers:
+                d = by_name.get(pl.src) if pl.kind == "conv" and isinstance(pl.src, str) else None
+                x = by_name.get(d.src) if d is not None and d.kind == "conv" and isinstance(d.src, str) else None
+                if x is None or x.kind != "conv" or pl.name in self.chain_of or pl.name in self.shortcut_of:
+                    continue
+                pq = self.q[pl.name]
+                if (pl.k == 1 and pl.pad == 0 and pl.stride == 1 and pl.groups == 1 and pl.act == "none"
+                        and not pl.add_after and (pq.bw_x, pq.bw_w) == (8, 8)
+                        and d.k == 3 and d.pad == 1 and d.stride in (1, 2) and d.groups == d.ci == d.co and d.groups > 1
+                        and x.k == 1 and x.pad == 0 and x.stride == 1 and x.groups == 1
+                        and inner_ok(x) and inner_ok(d) and only_reader(x, d) and only_reader(d, pl)
+                        and self.cdev[x.name] == self.cdev[d.name] == x.co):
+                    self.block_of[pl.name] = (x, d)
+        self._block_inner = {}
+        for pname, (x, d) in self.block_of.items():
+            self._block_inner[x.name] = pname
+            self._block_inner[d.name] = pname
+
+    def block_fuses(self, proj, n, h, w):
+        """whether the inverted-residual block that ends in the layer `proj` runs as one launch over n images whose
+        block input is h x w.  The one-launch kernel is bound by the same vector arithmetic as the three launches and
+        saves their start-up and the hidden tensors' traffic: measured on MobileNetV2 it pays from 14 x 14 outputs
+        on; smaller images leave it too few blocks."""
+        if proj.name not in self.block_of:
+            return False
+        x, d = self.block_of[proj.name]
+        ho, wo = (h - 1) // d.stride + 1, (w - 1) // d.stride + 1
+        if ho * wo < 196:
+            return False
+        return bool(torch.ops.torch_mlu.inverted_residual_fuses(n, h, w, self.cdev[x.src], self.cdev[x.name],
+                                                                self.cdev[proj.name], d.stride))
 
     def head_fuses(self, head, n, h, w):
         """whether the 1x1 layer `head` and the 3x3 layer behind it run as one launch over n images of h x w"""
@@ -388,8 +442,41 @@ class FusedNet(object):
             else:
                 env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"], d[2])
         skipped_heads = set()
+        skipped_inner = set()
+        by_name = {l.name: l for l in self.layers}
         for l in self.layers:
             name = l.name
+            if l.kind == "conv" and not tracing and name in self._block_inner:
+                pl = by_name[self._block_inner[name]]
+                x_, d_ = self.block_of[pl.name]
+                if l is x_:
+                    bx = env[(l.src, 8, self.q[name].pos_x, 1.0)]
+                    if self.block_fuses(pl, bx.shape[0], bx.shape[1], bx.shape[2]):
+                        skipped_inner.add(name)  # computed inside the launch of the block's projection
+                        continue
+                elif x_.name in skipped_inner:
+                    skipped_inner.add(name)
+                    continue
+            if l.kind == "conv" and name in self.block_of and self.block_of[name][1].name in skipped_inner:
+                x_, d_ = self.block_of[name]
+                lq, xq, dq = self.q[name], self.q[x_.name], self.q[d_.name]
+                qd = self.q_demand[name][0] if self.q_demand[name] else None
+                want_y = self.f_demand[name] or qd is None
+                resid = env[(l.add, "f")] if l.add else None
+                tick(name)
+                y, q = ops.qconv2d_irb(env[(x_.src, 8, xq.pos_x, 1.0)], xq.qw, xq.exp2, xq.chan_div, xq.bias,
+                                       _ACT_CODE[x_.act], dq.pos_x, dq.qw, d_.stride, dq.exp2, dq.chan_div, dq.bias,
+                                       _ACT_CODE[d_.act], lq.pos_x, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, want_y,
+                                       self.out_half and name in self.outputs, qd[0] if qd else 0, qd[1] if qd else 0,
+                                       qd[2] if qd else 1.0)
+                tick(name)
+                if want_y:
+                    env[(name, "f")] = y
+                if qd:
+                    env[(name,) + qd] = q
+                for dd in self.q_demand[name][1:]:
+                    env[(name,) + dd] = ops.quantize(y, dd[0], dd[1], dd[2])
+                continue
             if l.kind == "conv" and not tracing and name in self._fused_away:
                 continue
             if l.kind == "conv" and not tracing and name in self._head_names:

@@ -293,6 +293,43 @@ int catchq_conv1x1_conv3x3_nhwc(const void *x, const catchq_pointwise_head_t *he
                                 const catchq_conv_desc_t *desc, const catchq_epilogue_t *epilogue, void *workspace,
                                 size_t workspace_bytes, catchq_stream_t stream);
 
+/* An inverted-residual block in one launch: 1x1 expansion, 3x3 depthwise convolution, 1x1 linear projection.
+ * In the reference the block is three torch_mlu::conv2d calls (cnnl_conv2d,
+ * operators/cnnl/quantify_conv_forward.cpp:56-147; the middle one is depthwise by is_depthwise_conv,
+ * operators/cnnl/convolution_overrideable.cpp:41-54), the first two each followed by ReLU6
+ * (operators/cnnl/activation.cpp) and a quantization of the next convolution's input, the last one by the block's
+ * float add (cnnl_add, operators/cnnl/add.cpp) where the block has a shortcut.  Here, for x [n, h, w, ci] (int8):
+ *   q1 = sat(rne(act1(float(acc1) * 2^expand.exp2 / expand.chan_div[c] + expand.bias[c]) * 2^-expand.q_position))
+ *        acc1 = the 1x1 convolution of x with expand.w [hid, ci]                         (int8 [n, h, w, hid], never stored)
+ *   q2 = the same with acc2 = the depthwise 3x3 convolution (padding 1, stride `stride` in both directions) of q1
+ *        with depthwise.w [hid, 3, 3] and depthwise's constants                          (int8 [n, ho, wo, hid], never stored)
+ * and `epilogue` is applied to the 1x1 convolution of q2 with w_project [co, hid] exactly as catchq_conv2d_nhwc
+ * applies it (rows = the pixels of [n, ho, wo]; resid, y, q as there).  act is CATCHQ_ACT_RELU or CATCHQ_ACT_RELU6.
+ * The values are those of three catchq_conv2d_nhwc calls, bit for bit.
+ * The fused kernel serves ci % 32 == 0 (ci <= 160), hid % 32 == 0 (hid >= 128), co % 32 == 0 (co <= 512), w <= 128,
+ * stride 1 or 2, both inner stages with chan_div, chan_rcp and bias (-64 <= exp2 <= 64), no exp2_dev and no acc_out in
+ * the epilogue, on images whose bands of output rows fit its tile (catchq_inverted_residual_workspace_size reports 0
+ * then); any other shape runs as three launches with q1 and q2 in the caller's workspace
+ * (n * (h * w + ho * wo) * hid bytes, each part rounded up to 256).  The one-launch kernel does the vector arithmetic of
+ * the three launches and saves their start-up and the hidden tensors' traffic: it is the faster route for a lone
+ * stream of launches from 14 x 14 outputs on, not for small images or beside other launches that fill the gaps. */
+typedef struct catchq_requant_stage {
+  const void *w;         /* device int8 */
+  int exp2;
+  const float *chan_div; /* device [hid] or NULL */
+  const float *chan_rcp; /* device [hid] or NULL, as in catchq_epilogue_t */
+  const float *bias;     /* device [hid] or NULL */
+  int act;               /* CATCHQ_ACT_RELU or CATCHQ_ACT_RELU6 */
+  int q_position;
+} catchq_requant_stage_t;
+int catchq_inverted_residual_workspace_size(int n, int h, int w, int ci, int hid, int co, int stride,
+                                            const catchq_requant_stage_t *expand, const catchq_requant_stage_t *depthwise,
+                                            const catchq_epilogue_t *epilogue, size_t *bytes);
+int catchq_inverted_residual_nhwc(const void *x, int n, int h, int w, int ci, int hid, int co, int stride,
+                                  const catchq_requant_stage_t *expand, const catchq_requant_stage_t *depthwise,
+                                  const void *w_project, const catchq_epilogue_t *epilogue, void *workspace,
+                                  size_t workspace_bytes, catchq_stream_t stream);
+
 /* Residual chain of a stage of bottleneck blocks, recomputed from its int8 inputs in one launch.
  * In the reference every residual block ends in torch_mlu::conv2d (cnnl_conv2d,
  * operators/cnnl/quantify_conv_forward.cpp:56-147) followed by a float add (cnnl_add, operators/cnnl/add.cpp)

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 from catch_amd import _native
-from catch_amd._native import ChainLink, ConvDesc, Epilogue, PointwiseHead, Shortcut, check
+from catch_amd._native import ChainLink, ConvDesc, Epilogue, PointwiseHead, RequantStage, Shortcut, check
 
 F32, F16 = 0, 1
 _INT = {8: torch.int8, 16: torch.int16, 31: torch.int32, 32: torch.int32}
@@ -168,6 +168,28 @@ def conv1x1_conv3x3_nhwc(x, w1, exp2_1, div1, rcp1, bias1, q_pos1, w, padding=(1
     ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=x.device)
     check(lib().catchq_conv1x1_conv3x3_nhwc(ptr(x), ctypes.byref(hd), ptr(w), ctypes.byref(d), ctypes.byref(e), ptr(ws),
                                             need.value, stream()))
+    return out, need.value
+
+
+def inverted_residual_nhwc(x, expand, depthwise, w3, stride=1, exp2=0, chan_div=None, bias=None, resid=None, act=0,
+                           y_dtype=None, q_bw=8, q_pos=0, chan_rcp=None, sharing=0):
+    """x [N,H,W,Ci] int8; expand / depthwise: dicts with w (int8 [hid,Ci] / [hid,3,3]), exp2, chan_div, chan_rcp, bias,
+    act, q_pos (device tensors); w3 [Co,hid] int8 -> (outputs of the projection, workspace bytes the library asked for)"""
+    n, h, w, ci = x.shape
+    hid, co = expand["w"].shape[0], w3.shape[0]
+    ho = lib().catchq_conv_out_size(h, 3, 1, stride, 1)
+    wo = lib().catchq_conv_out_size(w, 3, 1, stride, 1)
+    e, out = _epilogue((n, ho, wo, co), x.device, exp2, chan_div, bias, resid, act, y_dtype, False, q_bw, q_pos, 1.0,
+                       chan_rcp)
+    e.sharing = sharing
+    st = [RequantStage(ptr(s["w"]), s["exp2"], ptr(s["chan_div"]), ptr(s.get("chan_rcp")), ptr(s["bias"]), s["act"],
+                       s["q_pos"]) for s in (expand, depthwise)]
+    need = ctypes.c_size_t()
+    check(lib().catchq_inverted_residual_workspace_size(n, h, w, ci, hid, co, stride, ctypes.byref(st[0]),
+                                                        ctypes.byref(st[1]), ctypes.byref(e), ctypes.byref(need)))
+    ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=x.device)
+    check(lib().catchq_inverted_residual_nhwc(ptr(x), n, h, w, ci, hid, co, stride, ctypes.byref(st[0]), ctypes.byref(st[1]),
+                                              ptr(w3), ctypes.byref(e), ptr(ws), need.value, stream()))
     return out, need.value
 
 

@@ -959,6 +959,72 @@ def test_conv1x1_then_conv3x3(case):
             assert same_bits(y, out["y"].cpu().numpy()), (act, want_y, sharing)
 
 
+IRB_CASES = [
+    # N, H, W, Ci, hidden, Co, stride, shortcut?, fused in one launch?
+    (3, 14, 14, 64, 384, 64, 1, True, True),     # MobileNetV2 at 14 x 14: two bands of 7 rows, two chunks of hidden channels
+    (2, 14, 14, 64, 384, 96, 1, False, True),    # three column tiles on two wave columns
+    (2, 14, 14, 96, 576, 96, 1, True, True),     # three K steps in the expansion, three chunks
+    (2, 14, 14, 96, 576, 160, 2, False, True),   # stride 2: 7 x 7 out of a 15-row patch
+    (2, 7, 7, 160, 960, 160, 1, True, True),     # whole 7 x 7 images, five chunks
+    (1, 7, 7, 160, 960, 320, 1, False, True),    # ten column tiles: three per wave
+    (2, 28, 28, 32, 192, 32, 1, True, True),     # one chunk, bands of 28 x 28 images
+    (2, 28, 28, 32, 192, 64, 2, False, True),    # stride 2 from 28 x 28: bands of two output rows
+    (2, 12, 20, 32, 192, 32, 1, True, True),     # W not a multiple of 4: ragged stencil groups
+    (1, 9, 11, 64, 192, 64, 2, False, True),     # odd sizes with stride 2
+    (2, 10, 10, 16, 96, 32, 1, False, False),    # channel counts outside the fused kernel: three launches
+    (1, 6, 6, 32, 192, 24, 1, False, False),
+]
+
+
+@pytest.mark.parametrize("case", IRB_CASES)
+def test_inverted_residual_block(case):
+    """catchq_inverted_residual_nhwc against the oracle's three convolutions in sequence: 1x1 expansion and 3x3 depthwise
+    convolution (padding 1), each dequantized, biased, sent through ReLU6 and requantized to int8, then the 1x1 projection
+    with its own epilogue (no activation, optional fp32 shortcut); int8 and fp32 outputs, bit for bit."""
+    n, h, w, ci, hid, co, stride, shortcut, fused = case
+    note("inverted_residual", case)
+    r = rng(sum(case[:7]))
+    x, w1 = _ints(r, (n, h, w, ci), 8), _ints(r, (hid, 1, 1, ci), 8)
+    wd, w3 = _ints(r, (hid, 3, 3, 1), 8), _ints(r, (co, 1, 1, hid), 8)
+    x[0, 0, :, :] = 127  # full-scale border rows: what the zero padding of the hidden tensor must not be replaced by
+    x[-1, -1, :, :] = -128
+
+    def consts(c, spread):
+        return r.uniform(0.6, 3.5, c).astype(np.float32), (r.standard_normal(c) * spread).astype(np.float32)
+
+    (div1, bias1), (div2, bias2), (div3, bias3) = consts(hid, 1.5), consts(hid, 1.5), consts(co, 1.0)
+    e1 = -12 - int(np.log2(ci / 32) / 2 + 0.5)
+    e2, e3, qp1, qp2, qp3 = -11, -10, -4, -4, -1
+    acc1, ovf1 = orc.conv2d_nhwc(x, w1, (0, 0), (1, 1), (1, 1), 1)
+    q1 = orc.quantize(orc.epilogue(acc1, e1, div1, bias1, None, 2), 8, qp1)
+    assert ovf1 == 0 and 0.02 < (q1 == 96).mean() < 0.5 and (q1 == 0).mean() < 0.8  # ReLU6's 6 and ReLU's 0 both occur
+    acc2, ovf2 = orc.conv2d_nhwc(q1, wd, (1, 1), (stride, stride), (1, 1), hid)
+    q2 = orc.quantize(orc.epilogue(acc2, e2, div2, bias2, None, 2), 8, qp2)
+    assert ovf2 == 0 and 0.005 < (q2 == 96).mean() < 0.6 and (q2 == 0).mean() < 0.8
+    acc3, ovf3 = orc.conv2d_nhwc(q2, w3, (0, 0), (1, 1), (1, 1), 1)
+    assert ovf3 == 0
+    resid = (r.standard_normal(acc3.shape) * 8).astype(np.float32) if shortcut else None
+    y = orc.epilogue(acc3, e3, div3, bias3, resid, 0)
+    q = orc.quantize(y, 8, qp3)
+    assert 0 < (np.abs(q.astype(np.int32)) >= 127).mean() < 0.4
+
+    dv = cabi.dev
+    st1 = dict(w=dv(w1.reshape(hid, ci)), exp2=e1, chan_div=dv(div1), chan_rcp=dv(np.float32(1) / div1), bias=dv(bias1),
+               act=2, q_pos=qp1)
+    st2 = dict(w=dv(wd.reshape(hid, 3, 3)), exp2=e2, chan_div=dv(div2), chan_rcp=dv(np.float32(1) / div2), bias=dv(bias2),
+               act=2, q_pos=qp2)
+    xd, w3d, d3, r3, b3 = dv(x), dv(w3.reshape(co, hid)), dv(div3), dv(np.float32(1) / div3), dv(bias3)
+    rd = dv(resid) if shortcut else None
+    for want_y, sharing in ((False, 0), (True, 2)):
+        out, ws_bytes = cabi.inverted_residual_nhwc(xd, st1, st2, w3d, stride=stride, exp2=e3, chan_div=d3, bias=b3, resid=rd,
+                                                    act=0, y_dtype=torch.float32 if want_y else None, q_bw=8, q_pos=qp3,
+                                                    chan_rcp=r3, sharing=sharing)
+        assert (ws_bytes == 0) == fused, ws_bytes
+        assert same_bits(q, out["q"].cpu().numpy()), (want_y, sharing)
+        if want_y:
+            assert same_bits(y, out["y"].cpu().numpy()), (want_y, sharing)
+
+
 CHAIN_CASES = [
     # N, Ho, Wo, Co, shortcut (Cs, stride), main channel counts (one per block)
     (2, 14, 14, 256, (64, 1), (64,)),                  # first block of stage 1: shortcut + one block

@@ -234,6 +234,32 @@ def test_mobilenet_v2_small():
     check_against_oracle(layers, sd, x, fused)
 
 
+def test_mobilenet_v2_blocks_in_one_launch():
+    """fuse_blocks: inverted-residual blocks as one launch each (torch_mlu::qconv2d_irb).  At 224 x 224 the blocks
+    with 28 x 28 and 14 x 14 outputs and hidden channel counts the kernel serves run fused; every tensor the plan still
+    produces, and the logits, equal the layer-by-layer plan's bit for bit, and that plan equals the oracle."""
+    note("mobilenet_v2 bs2 224x224, fused blocks")
+    layers = nets.mobilenet_v2()
+    net = nets.FloatNet(layers, seed=5, weight_std=0.2).eval()
+    x = torch.randn(2, 3, 224, 224, generator=torch.Generator().manual_seed(6))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd, fuse_blocks=True)
+    plain = pipeline.FusedNet(layers, sd)
+    assert sorted(fused.block_of) == sorted("b%d.proj" % b for b in range(1, 17)) and not plain.block_of
+    ka, kb, timers = {}, {}, {}
+    a = fused.forward(x.cuda(), keep=ka, timers=timers)
+    b = plain.forward(x.cuda(), keep=kb)
+    torch.cuda.synchronize()
+    one_launch = sorted(int(n[1:].split(".")[0]) for n in fused.block_of if n[:-4] + "dw" not in timers)
+    assert one_launch == list(range(4, 13)), one_launch  # b4 .. b12: hidden channels a multiple of 32, 196 outputs and more
+    for bnum in one_launch:
+        assert "b%d.exp" % bnum not in timers and ("b%d.exp" % bnum, 8) not in [k[:2] for k in ka]
+    assert torch.equal(a, b)
+    for key, t in ka.items():
+        assert torch.equal(t, kb[key]), key
+    check_against_oracle(layers, sd, x, plain)
+
+
 def test_darknet53_yolov3_int16_activations():
     """Darknet-53 + three YOLOv3 heads with int16 activations x int8 weights in the reference's
     [bitwidths],[positions] q-param encoding: leaky ReLU, shortcut adds after the activation,
