@@ -292,9 +292,10 @@ def plan_launches(fused, n, h, w):
         elif l.kind == "upsample":
             hi, wi = shape[l.src]
             shape[l.name] = (hi * 2, wi * 2)
-            for form in fused._forms(l.name):  # torch's repeat_interleave, twice
+            for form in fused._forms(l.name):  # torch's repeat_interleave, twice: rows doubled, then columns
                 e = 4 if form == ("f",) else form[0] // 8
-                rows.append(dict(name=l.name, kind="upsample", ops=0, bytes=n * fused.cdev[l.src] * e * hi * wi * 9))
+                rows.append(dict(name=l.name, kind="upsample", ops=0, bytes=n * fused.cdev[l.src] * e * hi * wi * 3))
+                rows.append(dict(name=l.name, kind="upsample", ops=0, bytes=n * fused.cdev[l.src] * e * hi * wi * 6))
         elif l.kind == "concat":
             shape[l.name] = shape[l.src[0]]
             hi, wi = shape[l.name]
