@@ -301,3 +301,39 @@ def test_darknet53_yolov3_fp16_heads_at_416():
             got = trace[l.name]["acc"].cpu().numpy()
             want = rec[l.name]["acc"].astype(np.int32)
             assert np.array_equal(want, got[..., :want.shape[-1]]), l.name
+
+
+@pytest.mark.parametrize("arch,batch,side", [("mobilenet_v2", 128, 224), ("darknet53_yolov3", 16, 416), ("resnet50", 64, 224)])
+def test_full_batch_graph_equals_its_images_alone(arch, batch, side):
+    """The benchmark's whole batch through the graph the benchmark replays (two parts on two streams, tiles planned
+    for a shared device): every output row of the first and last image of either part equals what the same plan
+    returns for that image alone, bit for bit, and the first image alone equals the oracle's whole network.  The
+    images are independent, so this carries the oracle's check to every batch position that the tile and band
+    rules place differently (first / last tile of a launch, either stream)."""
+    note("full batch", arch, batch, side)
+    layers = nets.NETS[arch]()
+    detector = arch == "darknet53_yolov3"
+    net = nets.FloatNet(layers, seed=7 if detector else 5, weight_std="he" if detector else (0.2 if arch == "mobilenet_v2" else 0.05)).eval()
+    g = torch.Generator().manual_seed(8)
+    x = torch.rand(batch, 3, side, side, generator=g) if detector else torch.randn(batch, 3, side, side, generator=g)
+    if detector:
+        sd = pipeline.to_position_encoding(pipeline.calibrate(net, x[:1], "int16", False), 16, 8)
+    else:
+        sd = pipeline.calibrate(net, x[:4], "int8", True)
+    fused = pipeline.FusedNet(layers, sd, out_half=detector)
+    static_in, replay = fused.capture(x.cuda(), streams=2)
+    out = replay()
+    outs = out if isinstance(out, tuple) else (out,)
+    half = batch // 2
+    for n in (0, half - 1, half, batch - 1):
+        alone = fused.forward(x[n:n + 1].cuda())
+        alone = alone if isinstance(alone, tuple) else (alone,)
+        for a, b in zip(alone, outs):
+            assert torch.equal(a[0], b[n]), (arch, n)
+    t, rec = netref.run(layers, {k: v.detach().cpu().numpy() for k, v in sd.items()}, x[:1].numpy(), record=False)
+    for name, o in zip(fused.outputs, outs):
+        got = o[:1].float().cpu().numpy()
+        want = t[name]
+        got = np.transpose(got, (0, 2, 3, 1)) if got.ndim == 4 else got.reshape(want.shape)
+        want = want.astype(np.float16).astype(np.float32) if detector else want
+        assert np.array_equal(want, got), name
