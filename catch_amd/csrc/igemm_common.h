@@ -256,10 +256,12 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     v[t] = x;
   }
   if (S::y16(e)) {
-    __half2 h[2] = {__halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1])),
-                    __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]))};
-    store_stream(reinterpret_cast<v2i *>(where.at(reinterpret_cast<__half *>(e.y))), *reinterpret_cast<v2i *>(h),
-                 e.y_stream != 0);
+    // two values per conversion instruction (v_cvt_pk_f16_f32: round to nearest even, like the single conversion)
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 h01 = __builtin_convertvector(f32x2{v[0], v[1]}, f16x2), h23 = __builtin_convertvector(f32x2{v[2], v[3]}, f16x2);
+    const v2i packed = {__builtin_bit_cast(int, h01), __builtin_bit_cast(int, h23)};
+    store_stream(reinterpret_cast<v2i *>(where.at(reinterpret_cast<__half *>(e.y))), packed, e.y_stream != 0);
   } else if (S::y32(e)) {
     v4f o = {v[0], v[1], v[2], v[3]};
     store_stream(reinterpret_cast<v4f *>(where.at(reinterpret_cast<float *>(e.y))), o, e.y_stream != 0);
