@@ -70,6 +70,11 @@ struct EpiSpec {
   // quantizer, 0 <= x <= min(6, 127 * 2^pos)
   static constexpr bool kFoldAct = DIV >= 0 && QM == 8 && YM == 0 && ACC == 0 && RESID != 2 &&
                                    (ACT == CATCHQ_ACT_RELU || ACT == CATCHQ_ACT_RELU6);
+  // ... and with the reciprocal form and no residual the requantization's power of two folds into the per-channel
+  // constants as well (scaling by 2^k is exact, so every intermediate is the scaled image of the unfolded one): the
+  // value arrives in units of the output's step, and one instruction (v_cvt_pk_u8_f32: round to nearest even,
+  // saturate to 0 .. 255, insert the byte) rounds and packs it
+  static constexpr bool kFoldScale = kFoldAct && DIV == 1 && RESID == 0;
   static __device__ __forceinline__ bool rcp(const EpiDev &e) { return DIV < 0 ? e.chan_rcp != nullptr : DIV == 1; }
   static __device__ __forceinline__ bool truediv(const EpiDev &e) {
     return DIV < 0 ? (e.chan_div != nullptr && e.chan_rcp == nullptr) : DIV == 2;
@@ -132,6 +137,8 @@ template <> struct EpiOf<EPI_LK_RESA_Y_Q16> { typedef EpiSpec<0, 1, 2, CATCHQ_AC
 inline int pick_epilogue(int N, const EpiDev &e) {
   if (!vec_epilogue_ok(N, e)) return EPI_SCALAR;
   if (e.acc_out || (e.q && e.q_scale != 1.0f) || (e.chan_div && !e.chan_rcp) || e.half_steps) return EPI_VECTOR;
+  // (the instances that fold the requantization's power of two into the per-channel constants keep those in range)
+  if (e.q && (e.q_neg_pos < -40 || e.q_neg_pos > 40)) return EPI_VECTOR;
   const int div = e.chan_rcp ? 1 : 0, bias = e.bias ? 1 : 0;
   const int res = !e.resid ? 0 : (e.resid_after ? 2 : 1);
   const int ym = !e.y ? 0 : (e.y_f16 ? 2 : 1);
@@ -174,11 +181,17 @@ __device__ __forceinline__ EpiLane epi_lane_setup(int n, bool n_ok, const EpiDev
     L.rcp = *reinterpret_cast<const v4f *>(e.chan_rcp + n);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      L.rcp[t] = __builtin_ldexpf(L.rcp[t], e.exp2);
-      L.div[t] = __builtin_ldexpf(L.div[t], -e.exp2);
+      L.rcp[t] = __builtin_ldexpf(L.rcp[t], e.exp2 + (S::kFoldScale ? e.q_neg_pos : 0));
+      L.div[t] = __builtin_ldexpf(L.div[t], -e.exp2 - (S::kFoldScale ? e.q_neg_pos : 0));
     }
   }
-  if (n_ok && L.use_bias) L.bias = *reinterpret_cast<const v4f *>(e.bias + n);
+  if (n_ok && L.use_bias) {
+    L.bias = *reinterpret_cast<const v4f *>(e.bias + n);
+    if constexpr (S::kFoldScale) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) L.bias[t] = __builtin_ldexpf(L.bias[t], e.q_neg_pos);
+    }
+  }
   return L;
 }
 
@@ -266,7 +279,20 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     v4f o = {v[0], v[1], v[2], v[3]};
     store_stream(reinterpret_cast<v4f *>(where.at(reinterpret_cast<float *>(e.y))), o, e.y_stream != 0);
   }
-  if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
+  if constexpr (S::kFoldScale) {
+    // v is already in units of the output's step: clamp to 0 .. min(127, 6 / step) (the median maps a NaN to 0, as
+    // ReLU does), then round, saturate and insert byte by byte
+    float hi = 127.0f;
+    if constexpr (S::kAct == CATCHQ_ACT_RELU6) {
+      const float six = __builtin_ldexpf(6.0f, e.q_neg_pos);
+      hi = (six < hi) ? six : hi;
+    }
+    unsigned packed = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(v[t], 0.0f, hi), (unsigned)t, packed);
+    *reinterpret_cast<unsigned *>(where.at(reinterpret_cast<int8_t *>(e.q))) = packed;
+  } else if constexpr (!S::kGeneric && S::kQ == 8 && (S::kAct == CATCHQ_ACT_RELU || S::kAct == CATCHQ_ACT_RELU6)) {
     // values are >= 0 and never NaN here (or, with the activation folded in, are made so by the median:
     // for a NaN operand it returns the smallest of the other two, 0, which is what ReLU makes of a NaN);
     // the requantization scale is 1:
