@@ -326,13 +326,17 @@ __device__ __forceinline__ void epi_vec4(const v4i a, const v4f res, const EpiLa
     const unsigned hi = __builtin_amdgcn_perm((unsigned)b[3], (unsigned)b[2], 0x04000c0cu);
     *reinterpret_cast<unsigned *>(where.at(reinterpret_cast<int8_t *>(e.q))) = lo | hi;
   } else if (S::q16(e)) {
-    v2i pk;
-    unsigned h[4];
+    // rounded to an integer and converted (NaN -> 0, out-of-range values saturate to the int32 range), then
+    // v_cvt_pk_i16_i32 saturates two of them to int16 and packs them: no clamp, mask or shift of our own
+    int i32[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-      h[t] = (unsigned)(L.unit_q ? quant1_unit<16>(v[t], e.q_neg_pos) : quant1<16>(v[t], e.q_scale, e.q_neg_pos)) & 0xffffu;
-    pk[0] = (int)(h[0] | (h[1] << 16));
-    pk[1] = (int)(h[2] | (h[3] << 16));
+    for (int t = 0; t < 4; ++t) {
+      const float x = L.unit_q ? v[t] : v[t] * e.q_scale;
+      i32[t] = cvt_i32_sat(__builtin_rintf(__builtin_ldexpf(x, e.q_neg_pos)));
+    }
+    v2i pk;
+    pk[0] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(i32[0], i32[1]));
+    pk[1] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(i32[2], i32[3]));
     *reinterpret_cast<v2i *>(where.at(reinterpret_cast<int16_t *>(e.q))) = pk;
   }
 }
