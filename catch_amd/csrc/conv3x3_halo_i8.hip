@@ -151,12 +151,12 @@ __global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__r
     for (int s = 0; s < STAGES - 1; ++s) issue_weights(s, s * B_STAGE);
   } else {
     // ---- the head: patch = requantized ReLU of the 1x1 convolution of the block input ------------------------------
-    static_assert(S == 1 && NW == 4 && (K1 == 64 || K1 == 256) && CI * K1 <= B_STAGE, "head shapes");
+    static_assert(S == 1 && (NW == 4 || NW == 8) && (K1 == 64 || K1 == 256) && CI * K1 <= B_STAGE, "head shapes");
     constexpr int KS1 = K1 / 32;   // MFMA K steps of the head
     constexpr int TN1 = CI / 32;   // its output channel tiles
     constexpr int CHW = K1 / 16;   // 16-byte chunks per filter row
-    constexpr int NI1 = CI * K1 / 1024 / NW;  // filter DMA instructions per wave
-    static_assert(CI * K1 / 1024 % NW == 0, "the head's filter rows must split evenly over the waves");
+    constexpr int W1_INSTR = CI * K1 / 1024;             // filter DMA instructions of the block
+    constexpr int NI1 = (W1_INSTR + NW - 1) / NW;        // ... per wave (the last waves may have none)
     const unsigned w1_slot = (unsigned)patch_bytes + (STAGES - 1) * B_STAGE;  // the ring slot filled last
     const unsigned const_off = (unsigned)patch_bytes + STAGES * B_STAGE;      // div', rcp', bias: CI floats each
     {  // filters -> LDS, chunk index XOR-ed with a row key so that the fragment reads of 16 rows spread over the banks
@@ -164,6 +164,7 @@ __global__ __launch_bounds__(64 * NW) void conv3x3_halo_kernel(const int8_t *__r
 #pragma unroll
       for (int t = 0; t < NI1; ++t) {
         const int b = wave * NI1 + t;
+        if (b >= W1_INSTR) break;  // wave-uniform
         unsigned row, phys, key;
         if constexpr (CHW >= 16) { row = (unsigned)b * (64 / CHW) + ((unsigned)lane / CHW); phys = (unsigned)lane % CHW; key = row & 15u; }
         else { row = (unsigned)b * 16 + ((unsigned)lane >> 2); phys = (unsigned)lane & 3u; key = (row >> 2) & 3u; }
@@ -467,6 +468,19 @@ int conv2d_head_halo_i8(const void *x, int K1, const void *w1, const float *div1
 #define CATCHQ_HEAD(K1_, TMW_)                                                                                                  \
   return epi == EPI_Q8_RELU ? launch_halo_epi<64, 2, TMW_, 1, EPI_Q8_RELU, 4, K1_, 3>(x, w, hp, e, lds_bytes, s, hd)             \
                             : launch_halo_epi<64, 2, TMW_, 1, EPI_VECTOR, 4, K1_, 3>(x, w, hp, e, lds_bytes, s, hd)
+#define CATCHQ_HEAD8(K1_)                                                                                                       \
+  return epi == EPI_Q8_RELU ? launch_halo_epi<64, 2, 1, 1, EPI_Q8_RELU, 8, K1_, 2>(x, w, hp, e, lds_bytes, s, hd)                \
+                            : launch_halo_epi<64, 2, 1, 1, EPI_VECTOR, 8, K1_, 2>(x, w, hp, e, lds_bytes, s, hd)
+  // Five to eight sub-tiles behind a head of 256 channels run on eight waves: the head's eleven or twelve sub-tiles of
+  // matrix and epilogue work spread over twice the waves and need two thirds of the fragment registers (measured on
+  // ResNet-50's first stage, 32 images: 20.7 -> 18.7 us per launch, +0.6 % end to end; the 64-channel head gains nothing)
+  int head_waves = (K1 == 256 && hp.nsub > 4 && hp.nsub <= 8) ? 8 : 4;
+  if (const char *t = tuning_env("CATCHQ_HEAD_WAVES")) head_waves = (atoi(t) == 8 && hp.nsub <= 8) ? 8 : 4;
+  if (head_waves == 8) {
+    if (K1 == 64) CATCHQ_HEAD8(64);
+    CATCHQ_HEAD8(256);
+  }
+#undef CATCHQ_HEAD8
   if (K1 == 64) {
     if (hp.nsub <= 4) CATCHQ_HEAD(64, 1);
     CATCHQ_HEAD(64, 2);
