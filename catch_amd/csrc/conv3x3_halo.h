@@ -52,9 +52,9 @@ __device__ __forceinline__ unsigned halo_key(unsigned prow, unsigned pcol, unsig
 
 // Tile choice for a 3x3 layer over input [N, Hi, Wi, Ci] of elem_bytes-wide integers: fills hp, the column tiles per block (tn), the dynamic LDS
 // size and the wave count; false: not this kernel's shape.  force_tn > 0 asks for that many column tiles (one block
-// over all output channels) and for band mode.
+// over all output channels) and for band mode; cus: the compute units the launch plans for.
 inline bool halo_plan(int N, int Hi, int Wi, int Ci, int Co, int stride, HaloParams &hp, int &tn, int &lds_bytes, int &waves,
-                      int force_tn = 0, int elem_bytes = 1) {
+                      int force_tn = 0, int elem_bytes = 1, int cus = 256) {
   const int Cb = Ci * elem_bytes;  // bytes per input pixel
   if (Cb != 64 && Cb != 128 && Cb != 256 && Cb != 512) return false;
   if (stride != 1 && !(stride == 2 && Cb != 64)) return false;
@@ -122,8 +122,10 @@ inline bool halo_plan(int N, int Hi, int Wi, int Ci, int Co, int stride, HaloPar
   if (force_tn > 0) {
     tn = force_tn;
   } else {
-    // 64 channels per block while that still gives every compute unit a block and the ring fits
-    int64_t min_blocks = 256;
+    // 64 channels per block while that still gives every compute unit the launch plans for a block and the ring fits
+    // (a launch that shares the device with another one plans for its share: measured on ResNet-50 as two parts,
+    // 64-channel blocks in stages 3 and 4 are worth +0.5 % end to end)
+    int64_t min_blocks = cus;
     if (const char *t = tuning_env("CATCHQ_HALO_MINBLK")) min_blocks = atoi(t);
     if (lds + 3 * 64 * 256 > kLdsLimit || tiles_m * ((Co + 63) / 64) < min_blocks) tn = 1;
     if (const char *t = tuning_env("CATCHQ_HALO_TN")) tn = atoi(t);

@@ -423,7 +423,7 @@ int conv2d_halo_i8(const void *x, const void *w, int N, int Hi, int Wi, int Ci, 
                    hipStream_t s) {
   HaloParams hp;
   int tn, lds_bytes, waves;
-  if (!halo_plan(N, Hi, Wi, Ci, Co, stride, hp, tn, lds_bytes, waves)) return -1;
+  if (!halo_plan(N, Hi, Wi, Ci, Co, stride, hp, tn, lds_bytes, waves, 0, 1, e.cus)) return -1;
   if (stride == 2) {
     switch (Ci) {
       case 128: return launch_halo<128, 2>(x, w, hp, e, tn, lds_bytes, waves, s);
