@@ -155,14 +155,24 @@ struct IrbStageDev {
   int exp2, q_neg_pos, relu6;
 };
 
+// From which size on a floating output is written, and a residual read, with the non-temporal hint, for a launch that
+// plans for `cus` of the 256 compute units.  Such a tensor is next used three launches later; kept in the caches it
+// pushes out the int8 operands and the filters of the launches in between.  Measured end to end (same box,
+// alternating): a residual read gains from the hint from 16 MiB on with the device to itself and from 8 MiB on as
+// one of two parts (ResNet-50 two parts +0.9-1.5 %, MobileNetV2 +0.3 %); an output of 25 MB written by one of two
+// parts gains as well (ResNet-50 +0.3-0.9 %, MobileNetV2 +1 %), while one of 51 MB written with the device to itself
+// loses (MobileNetV2 on one stream -1.6 %): the output's limit falls with the square of the share -- a part has its
+// share of the cache, and the other parts' traffic runs through that share too.
+inline int64_t stream_limit_y(int cus) { return (64ll << 20) * cus / 256 * cus / 256; }
+inline int64_t stream_limit_resid(int cus) { return (16ll << 20) * cus / 256; }
+
 // out_elems: elements of the output tensor (0: unknown, nothing is streamed)
 inline EpiDev make_epi(const catchq_epilogue_t *e, int64_t out_elems = 0) {
   EpiDev d;
-  // a quarter of the 256 MB last-level cache, of this launch's share of it
   d.cus = planned_cus(e->sharing);
-  const int64_t kStreamBytes = (64ll << 20) * d.cus / 256;
-  d.y_stream = (e->y && out_elems * (e->y_dtype == CATCHQ_F16 ? 2 : 4) >= kStreamBytes) ? 1 : 0;
-  d.resid_stream = (e->resid && out_elems * 4 >= kStreamBytes) ? 1 : 0;
+  const int64_t y_limit = stream_limit_y(d.cus), r_limit = stream_limit_resid(d.cus);
+  d.y_stream = (e->y && out_elems * (e->y_dtype == CATCHQ_F16 ? 2 : 4) >= y_limit) ? 1 : 0;
+  d.resid_stream = (e->resid && out_elems * 4 >= r_limit) ? 1 : 0;
   d.exp2 = e->exp2;
   d.chan_div = e->chan_div;
   const bool dev_exp = e->exp2_dev[0] || e->exp2_dev[1];

@@ -316,8 +316,7 @@ int conv1x1_chain_i8(const ChainLinkDev *links, int nlinks, int N, int Ho, int W
   cp.y = y;
   cp.q = q;
   cp.q_neg_pos = -q_position;
-  const int64_t kStreamBytes = (64ll << 20) * planned_cus(sharing) / 256;
-  cp.y_stream = (y && cp.M * Co * 4 >= kStreamBytes) ? 1 : 0;
+  cp.y_stream = (y && cp.M * Co * 4 >= stream_limit_y(planned_cus(sharing))) ? 1 : 0;
   if (!aligned16(y) || !aligned16(q)) return -1;
   for (int i = 0; i < nlinks; ++i) {
     const ChainLinkDev &ln = links[i];
