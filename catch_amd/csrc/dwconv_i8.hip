@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(const int8_t *__restrict__ x
       if (wo >= p.Wo) continue;
       const EpiAtSplit at = {(int64_t)img * p.Ho * p.Wo * p.C, (unsigned)((ho * p.Wo + wo) * p.C + c)};
       v4f res = {0.f, 0.f, 0.f, 0.f};
-      if (L.use_res) res = *reinterpret_cast<const v4f *>(at.at(e.resid));
+      if (L.use_res) res = load_stream(reinterpret_cast<const v4f *>(at.at(e.resid)), e.resid_stream != 0);
       const v4i a = {acc[py][px][0], acc[py][px][1], acc[py][px][2], acc[py][px][3]};
       epi_vec4<Sp>(a, res, L, at, e);
     }

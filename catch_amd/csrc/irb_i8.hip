@@ -386,7 +386,7 @@ __global__ __launch_bounds__(64 * IRB_NW) void irb_kernel(const int8_t *__restri
       L.bias = *reinterpret_cast<const v4f *>(c3 + 2 * p.Co + n);
       const int64_t idx = (m0 + pix) * p.Co + n;
       v4f res = {0.f, 0.f, 0.f, 0.f};
-      if (L.use_res) res = *reinterpret_cast<const v4f *>(e.resid + idx);
+      if (L.use_res) res = load_stream(reinterpret_cast<const v4f *>(e.resid + idx), e.resid_stream != 0);
       epi_vec4<EpiGeneric>(a, res, L, idx, e);
     }
   }
