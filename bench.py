@@ -52,6 +52,8 @@ def parse():
                     help="longest residual chain recomputed inside a block's last launch (0: none, -1: the plan's own rule)")
     ap.add_argument("--fuse-blocks", action="store_true",
                     help="inverted-residual blocks as one launch each where the kernel serves the shape (A/B runs)")
+    ap.add_argument("--no-fuse-first", action="store_true",
+                    help="input quantizer, first convolution and max pooling as three launches (A/B runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -98,9 +100,24 @@ def layer_profile(fused, x, iters=20, only=None):
     for pname, (bx, bd) in fused.block_of.items():
         if fused.block_fuses(next(l for l in fused.layers if l.name == pname), *trace[bx.name]["qx"].shape[:3]):
             fused_inner.update((bx.name, bd.name))
+    first = fused.first_layers_fuse(*x.shape)  # quantizer, first convolution and pooling in one launch
     for l in fused.layers:
         if l.kind not in ("conv", "fc") or l.name in fused._fused_away or l.name in fused_heads or l.name in fused_inner \
                 or (only and l.name != only):
+            continue
+        if first and l is fused.layers[0]:
+            lq, pool, d = fused.q[l.name], fused.first_pool, fused.q_demand["input"][0]
+            qd = fused.q_demand[pool.name][0]
+            code = {"relu": 1, "relu6": 2}[l.act]
+
+            def run(l=l, lq=lq, pool=pool, d=d, qd=qd, code=code):
+                return ops.qconv2d_first_layers(x, d[1], d[2], lq.qw, lq.exp2, lq.chan_div, lq.bias, code, qd[1], l.k, l.stride,
+                                                l.pad, pool.k, pool.stride, pool.pad)
+            pooled = run()
+            macs = trace[l.name]["y"].numel() * (lq.qw.numel() // lq.qw.shape[0])
+            t = event_time(run, iters)
+            rows.append(dict(name=l.name, route="mfma+first", t=t, ops=2 * macs,
+                             bytes=x.numel() * 4 + lq.qw.numel() + pooled.numel()))
             continue
         lq = fused.q[l.name]
         qx = trace[l.name].get("qx_dev", trace[l.name]["qx"])  # the tensor the kernel reads
@@ -202,7 +219,8 @@ def plan_launches(fused, n, h, w):
     integer outputs written) and integer operations, from the layer shapes alone (nothing is launched)."""
     rows, shape = [], {}
     cin = fused.cdev["input"]
-    for d in fused.q_demand["input"]:
+    first = fused.first_layers_fuse(n, fused.chan["input"], h, w)  # quantizer, first convolution and pooling in one launch
+    for d in fused.q_demand["input"] if not first else ():
         if fused.stem:
             sp = fused.stem["pad"]
             oh, ow = h + 2 * sp, w + 2 * sp + fused.stem["extra"]
@@ -217,6 +235,13 @@ def plan_launches(fused, n, h, w):
             ho, wo = (hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1
             shape[l.name] = (ho, wo)
             if l.name in fused._fused_away or fused.head_fuses(l, n, hi, wi):
+                continue
+            if first and l is fused.layers[0]:
+                lq, pool = fused.q[l.name], fused.first_pool
+                hp, wp = (ho + 2 * pool.pad - pool.k) // pool.stride + 1, (wo + 2 * pool.pad - pool.k) // pool.stride + 1
+                rows.append(dict(name=l.name, kind="conv", ops=2 * n * ho * wo * fused.cdev[l.name] * (lq.qw.numel() // lq.qw.shape[0]),
+                                 bytes=n * fused.chan["input"] * h * w * 4 + lq.qw.numel() + n * hp * wp * fused.cdev[l.name],
+                                 m=n * ho * wo, n=fused.cdev[l.name], k=lq.qw.numel() // lq.qw.shape[0]))
                 continue
             if l.name in fused._block_inner:
                 bp = next(m for m in fused.layers if m.name == fused._block_inner[l.name])
@@ -275,7 +300,7 @@ def plan_launches(fused, n, h, w):
             hi, wi = shape[l.src]
             ho, wo = (hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1
             shape[l.name] = (ho, wo)
-            for form in fused._forms(l.name):
+            for form in fused._forms(l.name) if not (first and l is fused.first_pool) else ():
                 e = 4 if form == ("f",) else form[0] // 8
                 rows.append(dict(name=l.name, kind="maxpool", ops=0, bytes=n * fused.cdev[l.src] * e * (hi * wi + ho * wo)))
         elif l.kind == "gap":
@@ -486,7 +511,8 @@ def build_workload(args):
         what += ", position + fractional scale"
     fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale,
                               chain_links=None if args.chain_links < 0 else args.chain_links,
-                              fuse_blocks=getattr(args, "fuse_blocks", False))
+                              fuse_blocks=getattr(args, "fuse_blocks", False),
+                              fuse_first_layers=not getattr(args, "no_fuse_first", False))
     if args.streams < 1:
         sys.exit("--streams must be at least 1")
     while batch % args.streams:  # the largest number of equal parts not above what was asked for
@@ -546,7 +572,9 @@ def main():
               "fused_heads": sorted(n for n, h in fused.head_of.items() if fused.head_fuses(h, batch // args.streams, *head_hw(fused, h, side))),
               "fused_blocks": sorted(n for n, (bx, bd) in fused.block_of.items()
                                      if fused.block_fuses(next(l for l in fused.layers if l.name == n), batch // args.streams,
-                                                          *head_hw(fused, bx, side)))}
+                                                          *head_hw(fused, bx, side))),
+              # input quantizer, first convolution and max pooling in one launch
+              "fused_first_layers": fused.first_layers_fuse(batch // args.streams, fused.chan["input"], side, side)}
     metric = ("int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
               else "int8 %s images/sec" % args.workload)
     if args.graph_only:

@@ -100,6 +100,10 @@ SIGNATURES = {
                                                      ctypes.POINTER(_SZ)]),
     "catchq_inverted_residual_nhwc": (_I, [_P, _I, _I, _I, _I, _I, _I, _I, ctypes.POINTER(RequantStage),
                                            ctypes.POINTER(RequantStage), _P, ctypes.POINTER(Epilogue), _P, _SZ, _P]),
+    "catchq_first_layers_workspace_size": (_I, [_I, _I, _I, _I, _I, _I, _I, _I, _I, ctypes.POINTER(RequantStage), _I, _I, _I,
+                                                _I, ctypes.POINTER(_SZ)]),
+    "catchq_first_layers_nchw": (_I, [_P, _I, _I, _I, _I, _I, ctypes.c_float, _I, _I, _I, _I, _I,
+                                      ctypes.POINTER(RequantStage), _I, _I, _I, _P, _I, _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
     "catchq_diag_mfma_i8_loop": (_I, [_P, _I, _I, _P, _P]),

@@ -42,6 +42,9 @@ int conv2d_head_halo_i8(const void *x, int K1, const void *w1, const float *div1
 bool irb_i8_ok(int N, int H, int W, int Cin, int hid, int Co, int S, int cus);
 int irb_i8(const void *x, int N, int H, int W, int Cin, int hid, int Co, int S, const IrbStageDev &s1, const IrbStageDev &s2,
            const void *w3, const EpiDev &e, hipStream_t s);
+bool stem_pool_i8_ok(int N, int C, int H, int W, int Co, int cus);
+int stem_pool_i8(const void *x, int N, int C, int H, int W, int x_pos, float x_scale, const IrbStageDev &s, int Co,
+                 void *q, int cus, hipStream_t st);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -473,6 +476,95 @@ CATCHQ_API int catchq_inverted_residual_nhwc(const void *x, int n, int h, int w,
   if (st != CATCHQ_OK) return st;
   const catchq_conv_desc_t d3 = {n, ho, wo, hid, co, 1, 1, 0, 0, 1, 1, 1, 1, 1};
   return catchq_conv2d_nhwc(q2, 8, w_project, 8, &d3, epilogue, stream);
+}
+
+// ---- first layers: quantizer + few-channel convolution + max pooling ------------------------------------------------
+struct FirstLayersShape {
+  int kw4, fh, fw, hc, wc, hp, wp;
+};
+
+static int check_first_layers(int n, int c, int h, int w, int co, int kh, int kw, int stride, int pad,
+                              const catchq_requant_stage_t *conv, int pool_k, int pool_stride, int pool_pad,
+                              FirstLayersShape *sh) {
+  if (!conv) return CATCHQ_ERR_ARG;
+  if (n < 0 || c <= 0 || c > 4 || h <= 0 || w <= 0 || co <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || pad < 0 ||
+      pool_k <= 0 || pool_stride <= 0 || pool_pad < 0 || 2 * pool_pad > pool_k)
+    return CATCHQ_ERR_SHAPE;
+  if (conv->act != CATCHQ_ACT_RELU && conv->act != CATCHQ_ACT_RELU6) return CATCHQ_ERR_ARG;
+  if (conv->exp2 < -126 || conv->exp2 > 126 || conv->q_position < -126 || conv->q_position > 126) return CATCHQ_ERR_ARG;
+  sh->kw4 = (kw + 3) / 4 * 4;
+  sh->fh = h + 2 * pad;
+  sh->fw = w + 2 * pad + sh->kw4 - kw;
+  sh->hc = catchq_conv_out_size(h, kh, pad, stride, 1);
+  sh->wc = catchq_conv_out_size(w, kw, pad, stride, 1);
+  if (sh->hc <= 0 || sh->wc <= 0) return CATCHQ_ERR_SHAPE;
+  sh->hp = catchq_conv_out_size(sh->hc, pool_k, pool_pad, pool_stride, 1);
+  sh->wp = catchq_conv_out_size(sh->wc, pool_k, pool_pad, pool_stride, 1);
+  if (sh->hp <= 0 || sh->wp <= 0) return CATCHQ_ERR_SHAPE;
+  return CATCHQ_OK;
+}
+
+static bool first_layers_fusable(int n, int c, int h, int w, int co, int kh, int kw, int stride, int pad,
+                                 const catchq_requant_stage_t *conv, int pool_k, int pool_stride, int pool_pad,
+                                 int sharing) {
+  return kh == 7 && kw == 7 && stride == 2 && pad == 3 && pool_k == 3 && pool_stride == 2 && pool_pad == 1 &&
+         conv->chan_div && conv->chan_rcp && conv->bias && conv->exp2 >= -64 && conv->exp2 <= 64 &&
+         stem_pool_i8_ok(n, c, h, w, co, planned_cus(sharing));
+}
+
+CATCHQ_API int catchq_first_layers_workspace_size(int n, int c, int h, int w, int co, int kh, int kw, int stride,
+                                                  int pad, const catchq_requant_stage_t *conv, int pool_k,
+                                                  int pool_stride, int pool_pad, int sharing, size_t *bytes) {
+  FirstLayersShape sh;
+  const int st = check_first_layers(n, c, h, w, co, kh, kw, stride, pad, conv, pool_k, pool_stride, pool_pad, &sh);
+  if (st != CATCHQ_OK) return st;
+  if (!bytes) return CATCHQ_ERR_ARG;
+  *bytes = first_layers_fusable(n, c, h, w, co, kh, kw, stride, pad, conv, pool_k, pool_stride, pool_pad, sharing)
+               ? 0 : round256((size_t)n * sh.fh * sh.fw * 4) + round256((size_t)n * sh.hc * sh.wc * co);
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_first_layers_nchw(const float *x, int n, int c, int h, int w, int x_position, float x_scale,
+                                        int co, int kh, int kw, int stride, int pad,
+                                        const catchq_requant_stage_t *conv, int pool_k, int pool_stride, int pool_pad,
+                                        void *q, int sharing, void *workspace, size_t workspace_bytes,
+                                        catchq_stream_t stream) {
+  FirstLayersShape sh;
+  int st = check_first_layers(n, c, h, w, co, kh, kw, stride, pad, conv, pool_k, pool_stride, pool_pad, &sh);
+  if (st != CATCHQ_OK) return st;
+  if (x_position < -126 || x_position > 126) return CATCHQ_ERR_ARG;
+  if (n == 0) return CATCHQ_OK;
+  if (!x || !q || !conv->w) return CATCHQ_ERR_ARG;
+  if (first_layers_fusable(n, c, h, w, co, kh, kw, stride, pad, conv, pool_k, pool_stride, pool_pad, sharing) &&
+      aligned16(x) && aligned16(conv->w) && aligned16(q)) {
+    const IrbStageDev s = {(const int8_t *)conv->w, conv->chan_div, conv->chan_rcp, conv->bias, conv->exp2,
+                           -conv->q_position, conv->act == CATCHQ_ACT_RELU6 ? 1 : 0};
+    const int st2 = stem_pool_i8(x, n, c, h, w, x_position, x_scale, s, co, q, planned_cus(sharing), as_stream(stream));
+    if (st2 >= 0) return st2;
+  }
+  // three launches: the framed int8 image and the convolution's output go through the workspace
+  const size_t b1 = round256((size_t)n * sh.fh * sh.fw * 4), b2 = round256((size_t)n * sh.hc * sh.wc * co);
+  if (!workspace || workspace_bytes < b1 + b2 || !aligned16(workspace)) return CATCHQ_ERR_ARG;
+  void *qx = workspace, *q1 = (char *)workspace + b1;
+  st = catchq_quantize_nchw_to_nhwc_frame(x, CATCHQ_F32, qx, 8, n, c, h, w, 4, sh.fh, sh.fw, pad, pad, x_position, x_scale,
+                                          stream);
+  if (st != CATCHQ_OK) return st;
+  catchq_epilogue_t es;
+  memset(&es, 0, sizeof(es));
+  es.exp2 = conv->exp2;
+  es.chan_div = conv->chan_div;
+  es.chan_rcp = conv->chan_rcp;
+  es.bias = conv->bias;
+  es.act = conv->act;
+  es.q = q1;
+  es.q_bitwidth = 8;
+  es.q_position = conv->q_position;
+  es.q_scale = 1.0f;
+  es.sharing = sharing;
+  const catchq_conv_desc_t d = {n, sh.fh, sh.fw, 4, co, kh, sh.kw4, 0, 0, stride, stride, 1, 1, 1};
+  st = catchq_conv2d_nhwc(qx, 8, conv->w, 8, &d, &es, stream);
+  if (st != CATCHQ_OK) return st;
+  return catchq_maxpool_nhwc(q1, q, 8, n, sh.hc, sh.wc, co, pool_k, pool_stride, pool_pad, stream);
 }
 
 CATCHQ_API int catchq_quantize_conv2d_workspace_size(const catchq_conv_desc_t *desc, int x_bits, int w_bits,

@@ -254,6 +254,19 @@ bool irb_fuses_op(int64_t n, int64_t h, int64_t w, int64_t ci, int64_t hid, int6
                                                  &bytes) == CATCHQ_OK && bytes == 0;
 }
 
+bool first_layers_fuse_op(int64_t n, int64_t c, int64_t h, int64_t w, int64_t co, int64_t k, int64_t stride, int64_t pad,
+                          int64_t pool_k, int64_t pool_stride, int64_t pool_pad) {
+  float one = 1.0f;
+  catchq_requant_stage_t st;
+  std::memset(&st, 0, sizeof(st));
+  st.w = &one; st.chan_div = st.chan_rcp = st.bias = &one;  // presence only: nothing is dereferenced
+  st.act = CATCHQ_ACT_RELU;
+  size_t bytes = 1;
+  return catchq_first_layers_workspace_size((int)n, (int)c, (int)h, (int)w, (int)co, (int)k, (int)k, (int)stride, (int)pad, &st,
+                                            (int)pool_k, (int)pool_stride, (int)pool_pad, t_launch_sharing,
+                                            &bytes) == CATCHQ_OK && bytes == 0;
+}
+
 bool head_fuses_op(int64_t n, int64_t h, int64_t w, int64_t k1, int64_t cm, int64_t co) {
   float one = 1.0f;
   catchq_pointwise_head_t hd;
@@ -642,6 +655,43 @@ std::tuple<Tensor, Tensor> qconv2d_irb_op(const Tensor &qx, const Tensor &w1, in
                                              &k1.st, &k2.st, w3.data_ptr(), &e, ws.data_ptr(), ws_bytes, current_stream()),
                "torch_mlu::qconv2d_irb");
   return std::make_tuple(o.y, o.q);
+}
+
+// The first layers in one call (catchq_first_layers_nchw): x [N,C,H,W] fp32, w [Co,kh,kw4,4] int8 (filter rows padded
+// with zero taps to a multiple of 4, and to 4 channels) -> the pooled int8 tensor [N,Hp,Wp,Co].
+Tensor qconv2d_first_layers_op(const Tensor &x, int64_t x_position, double x_scale, const Tensor &w, int64_t exp2,
+                               const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias, int64_t act,
+                               int64_t q_position, int64_t kw, int64_t stride, int64_t pad, int64_t pool_k,
+                               int64_t pool_stride, int64_t pool_pad) {
+  c10::DeviceGuard guard(x.device());
+  TORCH_CHECK(x.dim() == 4 && x.is_contiguous() && x.scalar_type() == at::kFloat,
+              "qconv2d_first_layers expects a contiguous fp32 NCHW input");
+  TORCH_CHECK(w.dim() == 4 && w.is_contiguous() && w.scalar_type() == at::kChar && w.device() == x.device(),
+              "qconv2d_first_layers expects int8 filters [Co, kh, kw4, 4] on the input's device");
+  const int64_t n = x.size(0), c = x.size(1), h = x.size(2), wd = x.size(3), co = w.size(0), kh = w.size(1);
+  TORCH_CHECK(w.size(3) == 4 && w.size(2) == (kw + 3) / 4 * 4 && c <= 4,
+              "qconv2d_first_layers: filter rows of ", (kw + 3) / 4 * 4, " taps x 4 channels expected");
+  TORCH_CHECK(x_position >= -126 && x_position <= 126, "input position out of range");
+  StageKeep k;
+  fill_stage(&k, w, exp2, chan_div, bias, act, q_position, co, "first-layer constants");
+  size_t ws_bytes = 0;
+  check_status(catchq_first_layers_workspace_size((int)n, (int)c, (int)h, (int)wd, (int)co, (int)kh, (int)kw, (int)stride,
+                                                  (int)pad, &k.st, (int)pool_k, (int)pool_stride, (int)pool_pad,
+                                                  t_launch_sharing, &ws_bytes),
+               "torch_mlu::qconv2d_first_layers");
+  const int hc = catchq_conv_out_size((int)h, (int)kh, (int)pad, (int)stride, 1);
+  const int wc = catchq_conv_out_size((int)wd, (int)kw, (int)pad, (int)stride, 1);
+  const int hp = catchq_conv_out_size(hc, (int)pool_k, (int)pool_pad, (int)pool_stride, 1);
+  const int wp = catchq_conv_out_size(wc, (int)pool_k, (int)pool_pad, (int)pool_stride, 1);
+  Tensor q = at::empty({n, hp, wp, co}, x.options().dtype(at::kChar));
+  if (n == 0) return q;
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, x.options().dtype(at::kChar));
+  check_status(catchq_first_layers_nchw(x.data_ptr<float>(), (int)n, (int)c, (int)h, (int)wd, (int)x_position, (float)x_scale,
+                                        (int)co, (int)kh, (int)kw, (int)stride, (int)pad, &k.st, (int)pool_k,
+                                        (int)pool_stride, (int)pool_pad, q.data_ptr(), t_launch_sharing, ws.data_ptr(), ws_bytes,
+                                        current_stream()),
+               "torch_mlu::qconv2d_first_layers");
+  return q;
 }
 
 // Residual chain (catchq_conv1x1_chain_nhwc): xs[i] [N,Hi,Wi,Ci] int8 NHWC, ws[i] [Co,Ci] or [Co,1,1,Ci] int8;
@@ -1221,6 +1271,8 @@ TORCH_LIBRARY(torch_mlu, m) {
         "Tensor wd, int stride, int exp2_2, Tensor? chan_div2, Tensor? bias2, int act2, int q_position2, Tensor w3, "
         "int exp2, Tensor? chan_div, Tensor? bias, Tensor? resid, bool want_y=True, bool y_half=False, "
         "int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> (Tensor, Tensor)");
+  m.def("qconv2d_first_layers(Tensor x, int x_position, float x_scale, Tensor w, int exp2, Tensor? chan_div, Tensor? bias, "
+        "int act, int q_position, int kw, int stride, int pad, int pool_k, int pool_stride, int pool_pad) -> Tensor");
   m.def("qconv2d_chain(Tensor[] xs, Tensor[] ws, int[] strides, int[] exp2s, Tensor[] chan_divs, Tensor[] biases, "
         "bool want_y=False, int q_bitwidth=8, int q_position=0) -> (Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
@@ -1233,6 +1285,8 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("set_launch_sharing(int launches) -> int", &set_launch_sharing_op);
   m.def("conv1x1_conv3x3_fuses(int n, int h, int w, int k1, int cm, int co) -> bool", &head_fuses_op);
   m.def("inverted_residual_fuses(int n, int h, int w, int ci, int hid, int co, int stride) -> bool", &irb_fuses_op);
+  m.def("first_layers_fuse(int n, int c, int h, int w, int co, int k, int stride, int pad, int pool_k, int pool_stride, "
+        "int pool_pad) -> bool", &first_layers_fuse_op);
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
   m.def("weight_cache_size() -> int", &cache_size_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
@@ -1257,6 +1311,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("qconv2d_shortcut", &qconv2d_shortcut_op);
   m.impl("qconv2d_head", &qconv2d_head_op);
   m.impl("qconv2d_irb", &qconv2d_irb_op);
+  m.impl("qconv2d_first_layers", &qconv2d_first_layers_op);
   m.impl("qconv2d_chain", &qconv2d_chain_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);

@@ -162,7 +162,8 @@ def _decode(layer, sd, device, ci_dev, co_dev, fractional=False):
 
 class FusedNet(object):
     def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True,
-                 fractional_scale=False, chain_links=None, fuse_heads=True, fuse_blocks=False):
+                 fractional_scale=False, chain_links=None, fuse_heads=True, fuse_blocks=False,
+                 fuse_first_layers=True):
         """fractional_scale: quantize activations and weights with position and fractional scale -- the
         general form the reference's fused (graph) mode hands to its backend per tensor / per axis
         (jit/utils/utils.cpp:81-167) -- instead of the eager ops' power-of-two steps.
@@ -179,7 +180,10 @@ class FusedNet(object):
         serves the shape and the image is large enough for it to pay (block_fuses).  Off by default: the one-launch
         kernel is bound by the same vector arithmetic as the three launches, and with the batch in two parts on
         parallel streams, where one part's launches already fill the other's start-up gaps, MobileNetV2 at batch 128
-        measured 2 % slower with it (one stream: 1.5 % faster)."""
+        measured 2 % slower with it (one stream: 1.5 % faster).
+        fuse_first_layers: the input quantizer, a few-channel first convolution + ReLU and the max pooling that is its
+        only reader run as one launch (torch_mlu::qconv2d_first_layers) where the library's kernel serves the shape;
+        neither the quantized image nor the convolution's output is then stored."""
         self.layers = list(layers)
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
@@ -295,6 +299,23 @@ class FusedNet(object):
                         and inner_ok(x) and inner_ok(d) and only_reader(x, d) and only_reader(d, pl)
                         and self.cdev[x.name] == self.cdev[d.name] == x.co):
                     self.block_of[pl.name] = (x, d)
+        # First layers: first_pool = the max-pooling layer behind the few-channel first convolution, when the pooled
+        # int8 tensor is all that anything reads of the two.
+        self.first_pool = None
+        if fuse_first_layers and self.stem:
+            l0 = self.layers[0]
+            lq = self.q[l0.name]
+            readers = [m for m in self.layers
+                       if m.src == l0.name or (isinstance(m.src, tuple) and l0.name in m.src) or m.add == l0.name]
+            pool = readers[0] if len(readers) == 1 and readers[0].kind == "maxpool" else None
+            if (pool is not None and l0.act in ("relu", "relu6") and not l0.add and (lq.bw_x, lq.bw_w) == (8, 8)
+                    and lq.chan_div is not None and lq.bias is not None and -64 <= lq.exp2 <= 64
+                    and self.cdev["input"] == 4 and len(self.q_demand["input"]) == 1
+                    and not ({l0.name, pool.name} & set(self.outputs))
+                    and not self.f_demand[l0.name] and not self.f_demand[pool.name]
+                    and len(self.q_demand[pool.name]) == 1 and self.q_demand[pool.name][0][0] == 8
+                    and self.q_demand[pool.name][0][2] == 1.0 and self.q_demand[l0.name] == self.q_demand[pool.name]):
+                self.first_pool = pool
         self._block_inner = {}
         for pname, (x, d) in self.block_of.items():
             self._block_inner[x.name] = pname
@@ -313,6 +334,14 @@ class FusedNet(object):
             return False
         return bool(torch.ops.torch_mlu.inverted_residual_fuses(n, h, w, self.cdev[x.src], self.cdev[x.name],
                                                                 self.cdev[proj.name], d.stride))
+
+    def first_layers_fuse(self, n, c, h, w):
+        """whether quantizer, first convolution and pooling run as one launch on a contiguous fp32 batch [n, c, h, w]"""
+        if self.first_pool is None:
+            return False
+        l0, pool = self.layers[0], self.first_pool
+        return bool(torch.ops.torch_mlu.first_layers_fuse(n, c, h, w, self.cdev[l0.name], l0.k, l0.stride, l0.pad, pool.k,
+                                                          pool.stride, pool.pad))
 
     def head_fuses(self, head, n, h, w):
         """whether the 1x1 layer `head` and the 3x3 layer behind it run as one launch over n images of h x w"""
@@ -434,7 +463,17 @@ class FusedNet(object):
             ev.record()
             timers.setdefault(name, []).append(ev)
             return ev
-        for d in self.q_demand["input"]:
+        first_fused = set()
+        if not tracing and x.dtype == torch.float32 and x.is_contiguous() and self.first_layers_fuse(*x.shape):
+            l0, pool, d = self.layers[0], self.first_pool, self.q_demand["input"][0]
+            lq, qd = self.q[l0.name], self.q_demand[self.first_pool.name][0]
+            tick(l0.name)
+            env[(pool.name,) + qd] = ops.qconv2d_first_layers(x, d[1], d[2], lq.qw, lq.exp2, lq.chan_div, lq.bias,
+                                                              _ACT_CODE[l0.act], qd[1], l0.k, l0.stride, l0.pad, pool.k,
+                                                              pool.stride, pool.pad)
+            tick(l0.name)
+            first_fused = {l0.name, pool.name}
+        for d in self.q_demand["input"] if not first_fused else ():
             if self.stem:
                 sp, h, w = self.stem["pad"], x.shape[2], x.shape[3]
                 env[("input",) + d] = ops.quantize_nhwc_frame(x, d[0], d[1], self.cdev["input"], h + 2 * sp,
@@ -446,6 +485,8 @@ class FusedNet(object):
         by_name = {l.name: l for l in self.layers}
         for l in self.layers:
             name = l.name
+            if name in first_fused:
+                continue
             if l.kind == "conv" and not tracing and name in self._block_inner:
                 pl = by_name[self._block_inner[name]]
                 x_, d_ = self.block_of[pl.name]

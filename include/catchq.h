@@ -330,6 +330,31 @@ int catchq_inverted_residual_nhwc(const void *x, int n, int h, int w, int ci, in
                                   const void *w_project, const catchq_epilogue_t *epilogue, void *workspace,
                                   size_t workspace_bytes, catchq_stream_t stream);
 
+/* The first layers of an image network in one launch: input quantization, k x k convolution over a few channels,
+ * ReLU / ReLU6, requantization, max pooling.  In the reference these are cnnl_quantify_offline on the channels-last
+ * input (operators/cnnl/quantify_conv_forward.cpp:62-63,97), torch_mlu::conv2d (cnnl_conv2d,
+ * operators/cnnl/quantify_conv_forward.cpp:56-147), ReLU (operators/cnnl/activation.cpp), the quantization of the
+ * next convolution's input and cnnl_max_pool2d (operators/cnnl/pooling.cpp).  For x [n, c, h, w] (fp32, contiguous,
+ * c <= 4):
+ *   qx = sat(rne(x * x_scale * 2^-x_position))                  int8, inside the convolution's zero padding; never stored
+ *   q1 = sat(rne(act(float(acc) * 2^conv.exp2 / conv.chan_div[o] + conv.bias[o]) * 2^-conv.q_position))
+ *        acc = the kh x kw convolution (stride `stride`, padding `pad`, both directions) of qx with conv.w
+ *        [co][kh][kw4][4] -- filter rows padded with zero taps to kw4 = kw rounded up to a multiple of 4, and to 4
+ *        channels, the layout catchq_conv2d_nhwc takes for a framed 4-channel input          int8 [n, hc, wc, co]; never stored
+ *   q  = max of q1 over windows pool_k x pool_k, stride pool_stride, padding pool_pad       int8 [n, hp, wp, co]
+ * The values are those of catchq_quantize_nchw_to_nhwc_frame, catchq_conv2d_nhwc and catchq_maxpool_nhwc called one
+ * after the other, bit for bit.  The fused kernel serves 7x7 / 2 / 3 convolutions of c <= 3 channels into 32, 64 or
+ * 128 channels followed by 3x3 / 2 / 1 pooling, w % 4 == 0, x 16-byte aligned, the stage with chan_div, chan_rcp and
+ * bias (-64 <= exp2 <= 64) (catchq_first_layers_workspace_size reports 0 then); anything else runs as the three
+ * launches with qx and q1 in the caller's workspace.  `sharing` is the planning hint of catchq_epilogue_t::sharing. */
+int catchq_first_layers_workspace_size(int n, int c, int h, int w, int co, int kh, int kw, int stride, int pad,
+                                       const catchq_requant_stage_t *conv, int pool_k, int pool_stride, int pool_pad,
+                                       int sharing, size_t *bytes);
+int catchq_first_layers_nchw(const float *x, int n, int c, int h, int w, int x_position, float x_scale, int co,
+                             int kh, int kw, int stride, int pad, const catchq_requant_stage_t *conv, int pool_k,
+                             int pool_stride, int pool_pad, void *q, int sharing, void *workspace,
+                             size_t workspace_bytes, catchq_stream_t stream);
+
 /* Residual chain of a stage of bottleneck blocks, recomputed from its int8 inputs in one launch.
  * In the reference every residual block ends in torch_mlu::conv2d (cnnl_conv2d,
  * operators/cnnl/quantify_conv_forward.cpp:56-147) followed by a float add (cnnl_add, operators/cnnl/add.cpp)

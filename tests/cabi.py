@@ -193,6 +193,26 @@ def inverted_residual_nhwc(x, expand, depthwise, w3, stride=1, exp2=0, chan_div=
     return out, need.value
 
 
+def first_layers_nchw(x, x_pos, conv, k, stride=2, pad=3, pool=(3, 2, 1), x_scale=1.0, sharing=0):
+    """x [N,C,H,W] fp32; conv: dict with w (int8 [Co,k,kw4,4], zero taps and channels included), exp2, chan_div, chan_rcp,
+    bias, act, q_pos (device tensors) -> (pooled int8 [N,Hp,Wp,Co], workspace bytes the library asked for)"""
+    n, c, h, w = x.shape
+    co = conv["w"].shape[0]
+    L = lib()
+    hc, wc = L.catchq_conv_out_size(h, k, pad, stride, 1), L.catchq_conv_out_size(w, k, pad, stride, 1)
+    hp, wp = L.catchq_conv_out_size(hc, pool[0], pool[2], pool[1], 1), L.catchq_conv_out_size(wc, pool[0], pool[2], pool[1], 1)
+    st = RequantStage(ptr(conv["w"]), conv["exp2"], ptr(conv["chan_div"]), ptr(conv.get("chan_rcp")), ptr(conv["bias"]),
+                      conv["act"], conv["q_pos"])
+    need = ctypes.c_size_t()
+    check(L.catchq_first_layers_workspace_size(n, c, h, w, co, k, k, stride, pad, ctypes.byref(st), pool[0], pool[1], pool[2],
+                                               sharing, ctypes.byref(need)))
+    ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=x.device)
+    q = torch.empty((n, hp, wp, co), dtype=torch.int8, device=x.device)
+    check(L.catchq_first_layers_nchw(ptr(x), n, c, h, w, x_pos, x_scale, co, k, k, stride, pad, ctypes.byref(st), pool[0],
+                                     pool[1], pool[2], ptr(q), sharing, ptr(ws), need.value, stream()))
+    return q, need.value
+
+
 def conv1x1_chain_nhwc(links, want_y=True, want_q=True, q_pos=0, sharing=0):
     """links: dicts with x [N,H,W,Ci] int8, w [Co,Ci] int8, stride, exp2, chan_div, chan_rcp, bias (device tensors);
     links[0] is the projection shortcut.  -> {"y": fp32 or None, "q": int8 or None}"""

@@ -62,6 +62,21 @@ def check_plan_rows(fused, x, images, rows_per_layer=3):
             if l.name in fused._fused_away:
                 continue  # evaluated inside its consumer's launch: covered there
             lq = fused.q[l.name]
+            if l is fused.layers[0] and fused.first_pool is not None and ("input",) + tuple(fused.q_demand["input"][0]) not in keep:
+                # quantizer, first convolution and pooling ran as one launch: the pooled tensor of the sampled images
+                # against the oracle's four steps on the whole image
+                d, pool = fused.q_demand["input"][0], fused.first_pool
+                qd = fused.q_demand[pool.name][0]
+                got = keep[(pool.name,) + tuple(qd)]
+                for n in images:
+                    qx = orc.quantize_nchw_to_nhwc(x[n:n + 1].cpu().numpy(), d[0], d[1], d[2], cpad=fused.cdev["input"])
+                    acc, ovf = orc.conv2d_nhwc(qx, lq.qw.cpu().numpy()[:, :, :l.k], (l.pad, l.pad), (l.stride, l.stride), (1, 1), 1)
+                    assert ovf == 0
+                    q1 = orc.quantize(orc.epilogue(acc, lq.exp2, _np(lq.chan_div), _np(lq.bias), None, _ACT[l.act]), 8, qd[1])
+                    want = orc.maxpool_nhwc(q1.astype(np.float32), pool.k, pool.stride, pool.pad).astype(np.int8)
+                    assert np.array_equal(want, got[n:n + 1].cpu().numpy()), "first layers: image %d" % n
+                    checked += 1
+                continue
             if l.name in fused._head_names and (l.name, 8, fused.q_demand[l.name][0][1], 1.0) not in keep:
                 continue  # a 1x1 head computed inside the launch of the 3x3 layer behind it: covered there
             head = fused.head_of.get(l.name)
@@ -130,6 +145,8 @@ def check_plan_rows(fused, x, images, rows_per_layer=3):
             checked += 1
         elif l.kind == "maxpool":
             for form in fused._forms(l.name):
+                if l is fused.first_pool and (l.src,) + form not in keep:
+                    continue  # pooled inside the first convolution's launch: covered there
                 src, got = keep[(l.src,) + form], keep[(l.name,) + form]
                 for n in images:
                     want = orc.maxpool_nhwc(src[n:n + 1].float().cpu().numpy(), l.k, l.stride, l.pad)
@@ -148,6 +165,9 @@ def check_plan_rows(fused, x, images, rows_per_layer=3):
             raise AssertionError("layer kind %s is not covered by this check" % l.kind)
     # the network input's quantized forms
     for d in fused.q_demand["input"]:
+        if ("input",) + tuple(d) not in keep:
+            assert fused.first_pool is not None  # quantized inside the first convolution's launch
+            continue
         got = keep[("input",) + tuple(d)]
         for n in images:
             want = orc.quantize_nchw_to_nhwc(x[n:n + 1].cpu().numpy(), d[0], d[1], d[2], cpad=fused.cdev["input"])

@@ -1025,6 +1025,57 @@ def test_inverted_residual_block(case):
             assert same_bits(y, out["y"].cpu().numpy()), (want_y, sharing)
 
 
+FIRST_LAYER_CASES = [
+    # N, C, H, W, Co, k, stride, pad, pool (k, stride, pad), activation, planning hint, fused in one launch?
+    (2, 3, 64, 64, 64, 7, 2, 3, (3, 2, 1), 1, 0, True),       # bands of one pooled row
+    (32, 3, 64, 64, 64, 7, 2, 3, (3, 2, 1), 1, 4, True),      # bands of five pooled rows, the last one shorter
+    (4, 3, 224, 224, 64, 7, 2, 3, (3, 2, 1), 1, 16, True),    # the ImageNet shape: bands of three pooled rows, 19 per image
+    (2, 3, 50, 36, 64, 7, 2, 3, (3, 2, 1), 2, 8, True),       # odd convolution height: the last window is cut by the image
+    (3, 1, 32, 40, 32, 7, 2, 3, (3, 2, 1), 1, 0, True),       # one input channel, 32 output channels
+    (1, 2, 40, 32, 128, 7, 2, 3, (3, 2, 1), 2, 0, True),      # 128 output channels: four channel groups
+    (2, 3, 30, 30, 64, 7, 2, 3, (3, 2, 1), 1, 0, False),      # width not a multiple of 4: three launches
+    (1, 4, 32, 32, 64, 7, 2, 3, (3, 2, 1), 1, 0, False),      # four input channels
+    (2, 3, 24, 24, 32, 3, 1, 1, (2, 2, 0), 2, 0, False),      # another filter and window
+]
+
+
+@pytest.mark.parametrize("case", FIRST_LAYER_CASES)
+def test_first_layers(case):
+    """catchq_first_layers_nchw against the oracle's quantizer, convolution, epilogue + requantization and max pooling in
+    sequence, bit for bit; full-scale pixels on the image's border show a wrong frame or a wrong window."""
+    n, c, h, w, co, k, stride, pad, pool, act, sharing, fused = case
+    note("first_layers", case)
+    r = rng(n + c + h + w + co + k)
+    x = (r.standard_normal((n, c, h, w)) * 1.5).astype(np.float32)
+    x[:, :, 0, :] = 5.0
+    x[:, :, -1, :] = -5.0
+    x[:, :, :, 0] = 4.5
+    x[:, :, :, -1] = -4.5
+    x_pos, x_scale = -5, 1.0 if n % 2 else 0.9371
+    wt = _ints(r, (co, k, k, 4), 8)
+    wt[..., c:] = 0
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = (r.standard_normal(co) * 2.0).astype(np.float32)
+    e1 = -11 - int(np.log2(k * k * c / 49.0) / 2 + 0.5)
+    qp = -3
+    qx = orc.quantize_nchw_to_nhwc(x, 8, x_pos, x_scale, cpad=4)
+    assert 0 < (np.abs(qx.astype(np.int32)) >= 127).mean() < 0.2
+    acc, ovf = orc.conv2d_nhwc(qx, wt, (pad, pad), (stride, stride), (1, 1), 1)
+    assert ovf == 0
+    q1 = orc.quantize(orc.epilogue(acc, e1, div, bias, None, act), 8, qp)
+    assert 0.02 < (q1 == (48 if act == 2 else 127)).mean() < 0.6 and 0.1 < (q1 == 0).mean() < 0.8
+    want = orc.maxpool_nhwc(q1.astype(np.float32), *pool).astype(np.int8)  # the oracle pools floats; int8 values survive the trip
+
+    kw4 = (k + 3) // 4 * 4
+    wdev = np.zeros((co, k, kw4, 4), np.int8)
+    wdev[:, :, :k] = wt
+    dv = cabi.dev
+    conv = dict(w=dv(wdev), exp2=e1, chan_div=dv(div), chan_rcp=dv(np.float32(1) / div), bias=dv(bias), act=act, q_pos=qp)
+    got, ws_bytes = cabi.first_layers_nchw(dv(x), x_pos, conv, k, stride, pad, pool, x_scale, sharing)
+    assert (ws_bytes == 0) == fused, ws_bytes
+    assert same_bits(want, got.cpu().numpy())
+
+
 CHAIN_CASES = [
     # N, Ho, Wo, Co, shortcut (Cs, stride), main channel counts (one per block)
     (2, 14, 14, 256, (64, 1), (64,)),                  # first block of stage 1: shortcut + one block

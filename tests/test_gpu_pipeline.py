@@ -260,6 +260,41 @@ def test_mobilenet_v2_blocks_in_one_launch():
     check_against_oracle(layers, sd, x, plain)
 
 
+def test_resnet50_first_layers_in_one_launch():
+    """fuse_first_layers (the default): input quantizer, 7x7 convolution + ReLU and 3x3 max pooling as one launch
+    (torch_mlu::qconv2d_first_layers).  Neither the quantized image nor the convolution's output is produced; every other
+    tensor of the plan, and the logits, equal those of the plan that runs the three launches, bit for bit, eagerly and
+    from a captured graph, and that plan equals the oracle."""
+    note("resnet50 bs3 96x96, first layers in one launch")
+    layers = nets.resnet(50)
+    net = nets.FloatNet(layers, seed=11, weight_std=0.05).eval()
+    x = torch.randn(3, 3, 96, 96, generator=torch.Generator().manual_seed(12))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd)
+    plain = pipeline.FusedNet(layers, sd, fuse_first_layers=False)
+    assert fused.first_pool is not None and fused.first_pool.name == "pool1" and plain.first_pool is None
+    assert fused.first_layers_fuse(3, 3, 96, 96) and not fused.first_layers_fuse(3, 3, 96, 98)
+    ka, kb, timers = {}, {}, {}
+    a = fused.forward(x.cuda(), keep=ka, timers=timers)
+    b = plain.forward(x.cuda(), keep=kb)
+    torch.cuda.synchronize()
+    missing = sorted(set(kb) - set(ka))
+    assert [k[0] for k in missing] == ["conv1", "input"] and set(ka) <= set(kb), missing
+    assert torch.equal(a, b)
+    for key, t in ka.items():
+        assert torch.equal(t, kb[key]), key
+    static_in, replay = fused.capture(x.cuda())
+    for i in range(2):
+        static_in.copy_(x.cuda())
+        assert torch.equal(replay(), b), "replay %d" % i
+        _ = fused.forward(torch.randn(3, 3, 96, 96, device="cuda"))  # eager work between the replays
+        torch.cuda.synchronize()
+    # a width the one-launch kernel does not take: the same plan falls back to the three launches
+    x2 = torch.randn(2, 3, 64, 62, generator=torch.Generator().manual_seed(13)).cuda()
+    assert torch.equal(fused.forward(x2), plain.forward(x2))
+    check_against_oracle(layers, sd, x, plain)
+
+
 def test_darknet53_yolov3_int16_activations():
     """Darknet-53 + three YOLOv3 heads with int16 activations x int8 weights in the reference's
     [bitwidths],[positions] q-param encoding: leaky ReLU, shortcut adds after the activation,
