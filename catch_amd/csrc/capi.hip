@@ -42,9 +42,9 @@ int conv2d_head_halo_i8(const void *x, int K1, const void *w1, const float *div1
 bool irb_i8_ok(int N, int H, int W, int Cin, int hid, int Co, int S, int cus);
 int irb_i8(const void *x, int N, int H, int W, int Cin, int hid, int Co, int S, const IrbStageDev &s1, const IrbStageDev &s2,
            const void *w3, const EpiDev &e, hipStream_t s);
-bool stem_pool_i8_ok(int N, int C, int H, int W, int Co, int cus);
+bool stem_pool_i8_ok(int N, int C, int H, int W, int Co);
 int stem_pool_i8(const void *x, int N, int C, int H, int W, int x_pos, float x_scale, const IrbStageDev &s, int Co,
-                 void *q, int cus, hipStream_t st);
+                 void *q, hipStream_t st);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -509,7 +509,7 @@ static bool first_layers_fusable(int n, int c, int h, int w, int co, int kh, int
                                  int sharing) {
   return kh == 7 && kw == 7 && stride == 2 && pad == 3 && pool_k == 3 && pool_stride == 2 && pool_pad == 1 &&
          conv->chan_div && conv->chan_rcp && conv->bias && conv->exp2 >= -64 && conv->exp2 <= 64 &&
-         stem_pool_i8_ok(n, c, h, w, co, planned_cus(sharing));
+         stem_pool_i8_ok(n, c, h, w, co);
 }
 
 CATCHQ_API int catchq_first_layers_workspace_size(int n, int c, int h, int w, int co, int kh, int kw, int stride,
@@ -539,7 +539,7 @@ CATCHQ_API int catchq_first_layers_nchw(const float *x, int n, int c, int h, int
       aligned16(x) && aligned16(conv->w) && aligned16(q)) {
     const IrbStageDev s = {(const int8_t *)conv->w, conv->chan_div, conv->chan_rcp, conv->bias, conv->exp2,
                            -conv->q_position, conv->act == CATCHQ_ACT_RELU6 ? 1 : 0};
-    const int st2 = stem_pool_i8(x, n, c, h, w, x_position, x_scale, s, co, q, planned_cus(sharing), as_stream(stream));
+    const int st2 = stem_pool_i8(x, n, c, h, w, x_position, x_scale, s, co, q, as_stream(stream));
     if (st2 >= 0) return st2;
   }
   // three launches: the framed int8 image and the convolution's output go through the workspace

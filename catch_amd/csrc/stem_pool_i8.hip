@@ -215,9 +215,14 @@ __global__ __launch_bounds__(64 * NW) void stem_pool_kernel(const float *__restr
 }
 
 // 7x7 / 2 / pad 3 convolution of up to three channels followed by 3x3 / 2 / pad 1 max pooling; 32, 64 or 128 output
-// channels; fp32 planes of a width that is a multiple of 4.  The band height is the largest that leaves two blocks
-// room in a compute unit's LDS, never more than gives every planned compute unit a block.
-static bool stem_pool_plan(int N, int C, int H, int W, int Co, int cus, StemPoolParams &p, int &lds_bytes) {
+// channels; fp32 planes of a width that is a multiple of 4.
+// Band height: a block's work grows with its 2 * PR + 1 convolution rows plus a fixed part (set-up, barriers, the
+// latency of its input rows), the launch takes as many rounds of blocks as the busiest compute unit gets, and a
+// compute unit that holds one block at a time (more than 80 KiB of LDS) cannot hide one block's input latency behind
+// another's arithmetic.  Measured on 32 x 3 x 224 x 224 (us): PR 1 34.8, 2 29.1, 3 30.2, 4 31.6, 5 36.7, 6 40.8 and,
+// with one block of sixteen waves per compute unit, 7 24.1 -- the estimate below ranks them in that order.  Blocks that
+// are alone on their compute unit run sixteen waves.
+static bool stem_pool_plan(int N, int C, int H, int W, int Co, StemPoolParams &p, int &lds_bytes, int &waves) {
   if (N <= 0 || C < 1 || C > 3 || H < 7 || W < 8 || W % 4 != 0 || W > 2048) return false;
   if (Co != 32 && Co != 64 && Co != 128) return false;
   p = StemPoolParams{};
@@ -235,12 +240,16 @@ static bool stem_pool_plan(int N, int C, int H, int W, int Co, int cus, StemPool
   };
   int want = 0;
   if (const char *t = tuning_env("CATCHQ_STEM_PR")) want = atoi(t);
+  constexpr int kDeviceCUs = 256;
   int best = 0;
+  int64_t best_cost = 0;
   for (int pr = 1; pr <= p.Hp && pr <= 16; ++pr) {
     const int lds = lds_of(pr);
     if (lds > 160 * 1024) break;
     const int bands = (p.Hp + pr - 1) / pr;
-    if (want > 0 ? (pr == want || !best) : (!best || (lds <= 80 * 1024 && (int64_t)N * bands >= 2 * cus))) best = pr;
+    const int64_t rounds = ((int64_t)N * bands + kDeviceCUs - 1) / kDeviceCUs;
+    const int64_t cost = rounds * (4 * pr + 5) * (lds > 80 * 1024 ? 150 : 115);
+    if (want > 0 ? (pr == want || !best) : (!best || cost < best_cost)) { best = pr; best_cost = cost; }
   }
   if (!best) return false;
   p.PR = best;
@@ -249,31 +258,35 @@ static bool stem_pool_plan(int N, int C, int H, int W, int Co, int cus, StemPool
   p.off_in = up(Co * 12);
   p.off_tile = p.off_in + up((4 * best + SP_KH) * p.in_pitch);
   lds_bytes = lds_of(best);
+  waves = lds_bytes > 80 * 1024 ? 16 : 8;
+  if (const char *t = tuning_env("CATCHQ_STEM_NW")) waves = atoi(t) == 16 ? 16 : 8;
   return true;
 }
 
-bool stem_pool_i8_ok(int N, int C, int H, int W, int Co, int cus) {
+bool stem_pool_i8_ok(int N, int C, int H, int W, int Co) {
   StemPoolParams p;
-  int lds;
-  return stem_pool_plan(N, C, H, W, Co, cus, p, lds);
+  int lds, waves;
+  return stem_pool_plan(N, C, H, W, Co, p, lds, waves);
 }
 
 // x fp32 [N, C, H, W]; s.w the filters [Co][7][8][4] (the eighth tap and the channels from C on zero); q int8
 // [N, Hp, Wp, Co].  -1: not this kernel's shape.
 int stem_pool_i8(const void *x, int N, int C, int H, int W, int x_pos, float x_scale, const IrbStageDev &s, int Co,
-                 void *q, int cus, hipStream_t st) {
+                 void *q, hipStream_t st) {
   StemPoolParams p;
-  int lds_bytes;
-  if (!stem_pool_plan(N, C, H, W, Co, cus, p, lds_bytes)) return -1;
+  int lds_bytes, waves;
+  if (!stem_pool_plan(N, C, H, W, Co, p, lds_bytes, waves)) return -1;
   p.x_neg_pos = -x_pos;
   p.x_scale = x_scale;
-  auto kern = stem_pool_kernel<8>;
-  if (lds_bytes > 64 * 1024) {
-    static std::atomic<bool> raised[64];
-    if (raise_lds_limit((const void *)kern, 160 * 1024, raised) != CATCHQ_OK) return CATCHQ_ERR_LAUNCH;
-  }
-  kern<<<N * p.bands, 64 * 8, lds_bytes, st>>>((const float *)x, s, (int8_t *)q, p);
-  return launch_status();
+  auto launch = [&](auto kern, int nw) {
+    if (lds_bytes > 64 * 1024) {
+      static std::atomic<bool> raised[64];
+      if (raise_lds_limit((const void *)kern, 160 * 1024, raised) != CATCHQ_OK) return (int)CATCHQ_ERR_LAUNCH;
+    }
+    kern<<<N * p.bands, 64 * nw, lds_bytes, st>>>((const float *)x, s, (int8_t *)q, p);
+    return launch_status();
+  };
+  return waves == 16 ? launch(stem_pool_kernel<16>, 16) : launch(stem_pool_kernel<8>, 8);
 }
 
 }  // namespace catchq

@@ -1027,9 +1027,11 @@ def test_inverted_residual_block(case):
 
 FIRST_LAYER_CASES = [
     # N, C, H, W, Co, k, stride, pad, pool (k, stride, pad), activation, planning hint, fused in one launch?
-    (2, 3, 64, 64, 64, 7, 2, 3, (3, 2, 1), 1, 0, True),       # bands of one pooled row
-    (32, 3, 64, 64, 64, 7, 2, 3, (3, 2, 1), 1, 4, True),      # bands of five pooled rows, the last one shorter
-    (4, 3, 224, 224, 64, 7, 2, 3, (3, 2, 1), 1, 16, True),    # the ImageNet shape: bands of three pooled rows, 19 per image
+    (2, 3, 64, 64, 64, 7, 2, 3, (3, 2, 1), 1, 0, True),       # few images: bands of one pooled row
+    (32, 3, 64, 64, 64, 7, 2, 3, (3, 2, 1), 1, 4, True),      # bands of two pooled rows
+    (48, 3, 52, 52, 64, 7, 2, 3, (3, 2, 1), 1, 0, True),      # bands of three pooled rows, the last band one row
+    (96, 3, 44, 44, 64, 7, 2, 3, (3, 2, 1), 2, 2, True),      # bands of six pooled rows, the last band five
+    (32, 3, 224, 224, 64, 7, 2, 3, (3, 2, 1), 1, 2, True),    # the ImageNet shape: seven pooled rows per block of sixteen waves
     (2, 3, 50, 36, 64, 7, 2, 3, (3, 2, 1), 2, 8, True),       # odd convolution height: the last window is cut by the image
     (3, 1, 32, 40, 32, 7, 2, 3, (3, 2, 1), 1, 0, True),       # one input channel, 32 output channels
     (1, 2, 40, 32, 128, 7, 2, 3, (3, 2, 1), 2, 0, True),      # 128 output channels: four channel groups
@@ -1063,7 +1065,7 @@ def test_first_layers(case):
     acc, ovf = orc.conv2d_nhwc(qx, wt, (pad, pad), (stride, stride), (1, 1), 1)
     assert ovf == 0
     q1 = orc.quantize(orc.epilogue(acc, e1, div, bias, None, act), 8, qp)
-    assert 0.02 < (q1 == (48 if act == 2 else 127)).mean() < 0.6 and 0.1 < (q1 == 0).mean() < 0.8
+    assert 0.005 < (q1 == (48 if act == 2 else 127)).mean() < 0.6 and 0.1 < (q1 == 0).mean() < 0.8
     want = orc.maxpool_nhwc(q1.astype(np.float32), *pool).astype(np.int8)  # the oracle pools floats; int8 values survive the trip
 
     kw4 = (k + 3) // 4 * 4
