@@ -54,6 +54,8 @@ def parse():
                     help="inverted-residual blocks as one launch each where the kernel serves the shape (A/B runs)")
     ap.add_argument("--no-fuse-first", action="store_true",
                     help="input quantizer, first convolution and max pooling as three launches (A/B runs)")
+    ap.add_argument("--no-fuse-avgpool", action="store_true",
+                    help="the last 1x1 convolution and the global average pooling as two launches (A/B runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -129,6 +131,26 @@ def layer_profile(fused, x, iters=20, only=None):
         extra_macs = extra_bytes = 0
         head = fused.head_of.get(l.name) if l.kind == "conv" else None
         block = fused.block_of.get(l.name) if l.kind == "conv" else None
+        gap = next((g for g in fused.layers if fused.pooled_conv.get(g.name) is l), None)
+        if gap is not None and fused.avgpool_fuses(gap, *qx.shape[:3]):
+            # the convolution runs inside the launch of the global average pooling behind it: its fp32 output is never
+            # stored, the launch writes the pooled values only
+            qds = fused.q_demand[gap.name]
+            want_mean = fused.f_demand[gap.name] or len(qds) != 1
+            gd = qds[0] if qds else None
+            resid = torch.zeros_like(trace[l.name]["y"]) if l.add else None
+            code = {"none": 0, "relu": 1, "relu6": 2}[l.act]
+
+            def run(lq=lq, qx=qx, resid=resid, code=code, want_mean=want_mean, gd=gd):
+                return ops.qconv2d_avgpool(qx, lq.qw, lq.exp2, lq.chan_div, lq.bias, resid, code, want_mean,
+                                           gd[0] if gd else 0, gd[1] if gd else 0, gd[2] if gd else 1.0)
+            y = trace[l.name]["y"]
+            pooled = y.shape[0] * y.shape[-1]
+            t = event_time(run, iters)
+            rows.append(dict(name=l.name, route="mfma+avgpool", t=t, ops=2 * y.numel() * (lq.qw.numel() // lq.qw.shape[0]),
+                             bytes=qx.numel() + lq.qw.numel() + (4 * y.numel() if resid is not None else 0)
+                             + pooled * ((4 if want_mean else 0) + (gd[0] // 8 if gd else 0))))
+            continue
         if block is not None and block[0].name in fused_inner:
             # expansion and depthwise layer run inside this launch: the block input and all three filter sets are read,
             # neither hidden tensor is stored
@@ -218,6 +240,7 @@ def plan_launches(fused, n, h, w):
     bytes (the tensors the fused plan moves: integer inputs and weights, fp32 residual read, fp32 / fp16 and
     integer outputs written) and integer operations, from the layer shapes alone (nothing is launched)."""
     rows, shape = [], {}
+    pooled_inside = set()  # 1x1 convolutions that run inside the launch of the global average pooling behind them
     cin = fused.cdev["input"]
     first = fused.first_layers_fuse(n, fused.chan["input"], h, w)  # quantizer, first convolution and pooling in one launch
     for d in fused.q_demand["input"] if not first else ():
@@ -235,6 +258,17 @@ def plan_launches(fused, n, h, w):
             ho, wo = (hi + 2 * l.pad - l.k) // l.stride + 1, (wi + 2 * l.pad - l.k) // l.stride + 1
             shape[l.name] = (ho, wo)
             if l.name in fused._fused_away or fused.head_fuses(l, n, hi, wi):
+                continue
+            gap = next((g for g in fused.layers if fused.pooled_conv.get(g.name) is l), None)
+            if gap is not None and fused.avgpool_fuses(gap, n, hi, wi):
+                lq, qds = fused.q[l.name], fused.q_demand[gap.name]
+                n_out = n * ho * wo * fused.cdev[l.name]
+                k = lq.qw.numel() // lq.qw.shape[0]
+                pooled_bytes = n * fused.cdev[l.name] * ((4 if (fused.f_demand[gap.name] or len(qds) != 1) else 0)
+                                                          + (qds[0][0] // 8 if qds else 0))
+                rows.append(dict(name=l.name, kind="conv", ops=2 * n_out * k, m=n * ho * wo, n=fused.cdev[l.name], k=k,
+                                 bytes=n * hi * wi * fused.cdev[l.src] + lq.qw.numel() + (4 * n_out if l.add else 0) + pooled_bytes))
+                pooled_inside.add(l.name)
                 continue
             if first and l is fused.layers[0]:
                 lq, pool = fused.q[l.name], fused.first_pool
@@ -307,7 +341,10 @@ def plan_launches(fused, n, h, w):
             hi, wi = shape[l.src]
             shape[l.name] = (1, 1)
             c = fused.cdev[l.src]
-            if fused.f_demand[l.name] or not fused.q_demand[l.name]:
+            if l.src in pooled_inside:
+                for d in fused.q_demand[l.name][1:]:
+                    rows.append(dict(name=l.name, kind="quantize", ops=0, bytes=n * c * (4 + d[0] // 8)))
+            elif fused.f_demand[l.name] or not fused.q_demand[l.name]:
                 rows.append(dict(name=l.name, kind="avgpool", ops=0, bytes=n * c * 4 * (hi * wi + 1)))
                 for d in fused.q_demand[l.name]:
                     rows.append(dict(name=l.name, kind="quantize", ops=0, bytes=n * c * (4 + d[0] // 8)))
@@ -512,7 +549,8 @@ def build_workload(args):
     fused = pipeline.FusedNet(layers, sd, out_half=detector, fractional_scale=args.fractional_scale,
                               chain_links=None if args.chain_links < 0 else args.chain_links,
                               fuse_blocks=getattr(args, "fuse_blocks", False),
-                              fuse_first_layers=not getattr(args, "no_fuse_first", False))
+                              fuse_first_layers=not getattr(args, "no_fuse_first", False),
+                              fuse_avgpool=not getattr(args, "no_fuse_avgpool", False))
     if args.streams < 1:
         sys.exit("--streams must be at least 1")
     while batch % args.streams:  # the largest number of equal parts not above what was asked for
@@ -574,7 +612,11 @@ def main():
                                      if fused.block_fuses(next(l for l in fused.layers if l.name == n), batch // args.streams,
                                                           *head_hw(fused, bx, side))),
               # input quantizer, first convolution and max pooling in one launch
-              "fused_first_layers": fused.first_layers_fuse(batch // args.streams, fused.chan["input"], side, side)}
+              "fused_first_layers": fused.first_layers_fuse(batch // args.streams, fused.chan["input"], side, side),
+              # 1x1 convolutions that run inside the launch of the global average pooling behind them
+              "fused_avgpool": sorted(c.name for g, c in fused.pooled_conv.items()
+                                      if fused.avgpool_fuses(next(l for l in fused.layers if l.name == g), batch // args.streams,
+                                                             *head_hw(fused, c, side)))}
     metric = ("int8 ResNet-50 images/sec bs64 + int8 GEMM TOPS (% MFMA peak), 1 GPU" if args.workload == "resnet50"
               else "int8 %s images/sec" % args.workload)
     if args.graph_only:

@@ -104,6 +104,9 @@ SIGNATURES = {
                                                 _I, ctypes.POINTER(_SZ)]),
     "catchq_first_layers_nchw": (_I, [_P, _I, _I, _I, _I, _I, ctypes.c_float, _I, _I, _I, _I, _I,
                                       ctypes.POINTER(RequantStage), _I, _I, _I, _P, _I, _P, _SZ, _P]),
+    "catchq_conv1x1_avgpool_workspace_size": (_I, [_I, _I, _I, _I, ctypes.POINTER(Epilogue), ctypes.POINTER(_SZ)]),
+    "catchq_conv1x1_avgpool_nhwc": (_I, [_P, _P, _I, _I, _I, _I, ctypes.POINTER(Epilogue), _P, _P, _I, _I, ctypes.c_float,
+                                         _P, _SZ, _P]),
     "catchq_conv2d_route": (ctypes.c_char_p, [_I, _I, ctypes.POINTER(ConvDesc)]),
     "catchq_gemm_route": (ctypes.c_char_p, [_I, _I, _I64, _I64, _I64]),
     "catchq_diag_mfma_i8_loop": (_I, [_P, _I, _I, _P, _P]),

@@ -19,7 +19,7 @@ INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
-KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "igemm_i8_dma_gemm.hip", "igemm_i8_dma_conv.hip", "igemm_i8_dual.hip", "igemm_i8_chain.hip", "conv3x3_halo_i8.hip", "igemm_a16_dma.hip", "pw_i8.hip", "dwconv_i8.hip", "irb_i8.hip", "stem_pool_i8.hip", "pool.hip", "diag.hip", "capi.hip",
+KERNEL_SOURCES = ["quantize.hip", "contract_direct.hip", "igemm_i8.hip", "igemm_i8_dma_gemm.hip", "igemm_i8_dma_conv.hip", "igemm_i8_dual.hip", "igemm_i8_chain.hip", "conv3x3_halo_i8.hip", "igemm_a16_dma.hip", "pw_i8.hip", "dwconv_i8.hip", "irb_i8.hip", "stem_pool_i8.hip", "conv1x1_gap_i8.hip", "pool.hip", "diag.hip", "capi.hip",
                   "host_math.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from the fp32 epilogue math.

@@ -45,6 +45,16 @@ int irb_i8(const void *x, int N, int H, int W, int Cin, int hid, int Co, int S, 
 bool stem_pool_i8_ok(int N, int C, int H, int W, int Co);
 int stem_pool_i8(const void *x, int N, int C, int H, int W, int x_pos, float x_scale, const IrbStageDev &s, int Co,
                  void *q, hipStream_t st);
+struct GapConvDev {
+  const float *div, *rcp, *bias, *resid;
+  int exp2, act;
+  float *mean;
+  void *q;
+  int q_bw, q_neg_pos;
+  float q_scale;
+};
+bool conv1x1_gap_i8_ok(int N, int HW, int K, int Co);
+int conv1x1_gap_i8(const void *x, const void *w, int N, int HW, int K, int Co, const GapConvDev &e, hipStream_t st);
 bool dwconv_i8_supported(int C, int kh, int kw, int sw, int dw);
 int dwconv_i8(const void *x, const void *w, int N, int H, int W, int C, int kh, int kw, int ph, int pw, int sh,
               int sw, int dh, int dw, int Ho, int Wo, const EpiDev &e, hipStream_t s);
@@ -565,6 +575,65 @@ CATCHQ_API int catchq_first_layers_nchw(const float *x, int n, int c, int h, int
   st = catchq_conv2d_nhwc(qx, 8, conv->w, 8, &d, &es, stream);
   if (st != CATCHQ_OK) return st;
   return catchq_maxpool_nhwc(q1, q, 8, n, sh.hc, sh.wc, co, pool_k, pool_stride, pool_pad, stream);
+}
+
+// ---- 1x1 convolution + global average pooling ---------------------------------------------------------------------------
+static int check_conv_avgpool(int n, int hw, int ci, int co, const catchq_epilogue_t *e) {
+  if (n < 0 || hw <= 0 || ci <= 0 || co <= 0) return CATCHQ_ERR_SHAPE;
+  if (!e || e->y || e->q || e->acc_out || (e->resid && e->resid_after_act)) return CATCHQ_ERR_ARG;  // the output is not stored
+  if (e->act < CATCHQ_ACT_NONE || e->act > CATCHQ_ACT_LEAKY || e->exp2 < -126 || e->exp2 > 126 || e->sharing < 0)
+    return CATCHQ_ERR_ARG;
+  return CATCHQ_OK;
+}
+
+static bool conv_avgpool_fusable(int n, int hw, int ci, int co, const catchq_epilogue_t *e) {
+  return e->chan_div && e->chan_rcp && e->bias && e->exp2 >= -64 && e->exp2 <= 64 && !e->exp2_dev[0] && !e->exp2_dev[1] &&
+         !e->half_steps && (e->act == CATCHQ_ACT_NONE || e->act == CATCHQ_ACT_RELU || e->act == CATCHQ_ACT_RELU6) &&
+         conv1x1_gap_i8_ok(n, hw, ci, co);
+}
+
+CATCHQ_API int catchq_conv1x1_avgpool_workspace_size(int n, int hw, int ci, int co, const catchq_epilogue_t *epilogue,
+                                                     size_t *bytes) {
+  const int st = check_conv_avgpool(n, hw, ci, co, epilogue);
+  if (st != CATCHQ_OK) return st;
+  if (!bytes) return CATCHQ_ERR_ARG;
+  *bytes = conv_avgpool_fusable(n, hw, ci, co, epilogue) ? 0 : (size_t)n * hw * co * 4;
+  return CATCHQ_OK;
+}
+
+CATCHQ_API int catchq_conv1x1_avgpool_nhwc(const void *x, const void *w, int n, int hw, int ci, int co,
+                                           const catchq_epilogue_t *epilogue, float *mean, void *q, int q_bitwidth,
+                                           int q_position, float q_scale, void *workspace, size_t workspace_bytes,
+                                           catchq_stream_t stream) {
+  int st = check_conv_avgpool(n, hw, ci, co, epilogue);
+  if (st != CATCHQ_OK) return st;
+  if (q && q_bitwidth != 8 && q_bitwidth != 16) return CATCHQ_ERR_BITWIDTH;
+  if (q_position < -126 || q_position > 126) return CATCHQ_ERR_ARG;
+  if (!mean && !q) return CATCHQ_ERR_ARG;
+  if (n == 0) return CATCHQ_OK;
+  if (!x || !w) return CATCHQ_ERR_ARG;
+  if (conv_avgpool_fusable(n, hw, ci, co, epilogue) && aligned16(x) && aligned16(w) && aligned16(epilogue->chan_div) &&
+      aligned16(epilogue->chan_rcp) && aligned16(epilogue->bias) && aligned16(epilogue->resid)) {
+    const GapConvDev e = {epilogue->chan_div, epilogue->chan_rcp, epilogue->bias, epilogue->resid, epilogue->exp2,
+                          epilogue->act, mean, q, q_bitwidth, -q_position, q_scale};
+    const int st2 = conv1x1_gap_i8(x, w, n, hw, ci, co, e, as_stream(stream));
+    if (st2 >= 0) return st2;
+  }
+  // two launches: the convolution's fp32 output goes through the workspace
+  const size_t need = (size_t)n * hw * co * 4;
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return CATCHQ_ERR_ARG;
+  catchq_epilogue_t ec = *epilogue;
+  ec.y = workspace;
+  ec.y_dtype = CATCHQ_F32;
+  const catchq_conv_desc_t d = {n, hw, 1, ci, co, 1, 1, 0, 0, 1, 1, 1, 1, 1};
+  st = catchq_conv2d_nhwc(x, 8, w, 8, &d, &ec, stream);
+  if (st != CATCHQ_OK) return st;
+  if (mean) {
+    st = catchq_global_avgpool_nhwc((const float *)workspace, mean, n, hw, co, stream);
+    if (st != CATCHQ_OK) return st;
+  }
+  if (q) return catchq_global_avgpool_quantize_nhwc((const float *)workspace, q, q_bitwidth, n, hw, co, q_position, q_scale, stream);
+  return CATCHQ_OK;
 }
 
 CATCHQ_API int catchq_quantize_conv2d_workspace_size(const catchq_conv_desc_t *desc, int x_bits, int w_bits,

@@ -267,6 +267,16 @@ bool first_layers_fuse_op(int64_t n, int64_t c, int64_t h, int64_t w, int64_t co
                                             &bytes) == CATCHQ_OK && bytes == 0;
 }
 
+bool conv_avgpool_fuses_op(int64_t n, int64_t hw, int64_t ci, int64_t co) {
+  float one = 1.0f;
+  catchq_epilogue_t e;
+  std::memset(&e, 0, sizeof(e));
+  e.chan_div = e.chan_rcp = e.bias = &one;  // presence only: nothing is dereferenced
+  e.act = CATCHQ_ACT_RELU;
+  size_t bytes = 1;
+  return catchq_conv1x1_avgpool_workspace_size((int)n, (int)hw, (int)ci, (int)co, &e, &bytes) == CATCHQ_OK && bytes == 0;
+}
+
 bool head_fuses_op(int64_t n, int64_t h, int64_t w, int64_t k1, int64_t cm, int64_t co) {
   float one = 1.0f;
   catchq_pointwise_head_t hd;
@@ -692,6 +702,55 @@ Tensor qconv2d_first_layers_op(const Tensor &x, int64_t x_position, double x_sca
                                         current_stream()),
                "torch_mlu::qconv2d_first_layers");
   return q;
+}
+
+// A 1x1 convolution and the global average pooling behind it (catchq_conv1x1_avgpool_nhwc): qx [N,H,W,Ci] int8 NHWC,
+// qw [Co,Ci] or [Co,1,1,Ci] int8, resid [N,H,W,Co] fp32 -> (fp32 means [N,Co] or an undefined tensor,
+// means quantized at (q_position, q_scale) [N,Co] or an undefined tensor)
+std::tuple<Tensor, Tensor> qconv2d_avgpool_op(const Tensor &qx, const Tensor &qw, int64_t exp2,
+                                              const c10::optional<Tensor> &chan_div, const c10::optional<Tensor> &bias,
+                                              const c10::optional<Tensor> &resid, int64_t act, bool want_mean,
+                                              int64_t q_bitwidth, int64_t q_position, double q_scale) {
+  c10::DeviceGuard guard(qx.device());
+  TORCH_CHECK(qx.dim() == 4 && qx.is_contiguous() && qw.is_contiguous() && qx.scalar_type() == at::kChar &&
+                  qw.scalar_type() == at::kChar && qw.device() == qx.device(),
+              "qconv2d_avgpool expects contiguous int8 NHWC activations and int8 filters on one device");
+  const int64_t n = qx.size(0), hw = qx.size(1) * qx.size(2), ci = qx.size(3), co = qw.size(0);
+  TORCH_CHECK(qw.numel() == co * ci, "qconv2d_avgpool: the filters must be [", co, ", ", ci, "]");
+  TORCH_CHECK(want_mean || q_bitwidth != 0, "qconv2d_avgpool: no output requested");
+  TORCH_CHECK(q_bitwidth == 0 || q_bitwidth == 8 || q_bitwidth == 16, "bitwidth not support");
+  TORCH_CHECK(exp2 >= -126 && exp2 <= 126, "position sum out of range");
+  catchq_epilogue_t e;
+  std::memset(&e, 0, sizeof(e));
+  e.exp2 = (int)exp2;
+  e.act = (int)act;
+  e.sharing = t_launch_sharing;
+  Tensor cd = as_f32_vec(chan_div, co, "qconv2d_avgpool constants"), bs = as_f32_vec(bias, co, "qconv2d_avgpool constants"), rcp, rs;
+  if (cd.defined()) {
+    e.chan_div = cd.data_ptr<float>();
+    rcp = reciprocals_for(cd);
+    if (rcp.defined()) e.chan_rcp = rcp.data_ptr<float>();
+  }
+  if (bs.defined()) e.bias = bs.data_ptr<float>();
+  if (resid.has_value() && resid->defined()) {
+    rs = *resid;
+    TORCH_CHECK(rs.scalar_type() == at::kFloat && rs.is_contiguous() && rs.numel() == n * hw * co && rs.device() == qx.device(),
+                "qconv2d_avgpool: the residual must be a contiguous fp32 [N,H,W,Co] tensor on the input's device");
+    e.resid = rs.data_ptr<float>();
+  }
+  Tensor mean, q;
+  if (want_mean) mean = at::empty({n, co}, qx.options().dtype(at::kFloat));
+  if (q_bitwidth) q = at::empty({n, co}, qx.options().dtype(int_type((int)q_bitwidth)));
+  if (n == 0) return std::make_tuple(mean, q);
+  size_t ws_bytes = 0;
+  check_status(catchq_conv1x1_avgpool_workspace_size((int)n, (int)hw, (int)ci, (int)co, &e, &ws_bytes), "torch_mlu::qconv2d_avgpool");
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, qx.options().dtype(at::kChar));
+  check_status(catchq_conv1x1_avgpool_nhwc(qx.data_ptr(), qw.data_ptr(), (int)n, (int)hw, (int)ci, (int)co, &e,
+                                           mean.defined() ? mean.data_ptr<float>() : nullptr,
+                                           q.defined() ? q.data_ptr() : nullptr, (int)q_bitwidth, (int)q_position,
+                                           (float)q_scale, ws.data_ptr(), ws_bytes, current_stream()),
+               "torch_mlu::qconv2d_avgpool");
+  return std::make_tuple(mean, q);
 }
 
 // Residual chain (catchq_conv1x1_chain_nhwc): xs[i] [N,Hi,Wi,Ci] int8 NHWC, ws[i] [Co,Ci] or [Co,1,1,Ci] int8;
@@ -1273,6 +1332,8 @@ TORCH_LIBRARY(torch_mlu, m) {
         "int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> (Tensor, Tensor)");
   m.def("qconv2d_first_layers(Tensor x, int x_position, float x_scale, Tensor w, int exp2, Tensor? chan_div, Tensor? bias, "
         "int act, int q_position, int kw, int stride, int pad, int pool_k, int pool_stride, int pool_pad) -> Tensor");
+  m.def("qconv2d_avgpool(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, Tensor? resid, int act, "
+        "bool want_mean=True, int q_bitwidth=0, int q_position=0, float q_scale=1.0) -> (Tensor, Tensor)");
   m.def("qconv2d_chain(Tensor[] xs, Tensor[] ws, int[] strides, int[] exp2s, Tensor[] chan_divs, Tensor[] biases, "
         "bool want_y=False, int q_bitwidth=8, int q_position=0) -> (Tensor, Tensor)");
   m.def("qlinear(Tensor qx, Tensor qw, int exp2, Tensor? chan_div, Tensor? bias, int act=0, "
@@ -1287,6 +1348,7 @@ TORCH_LIBRARY(torch_mlu, m) {
   m.def("inverted_residual_fuses(int n, int h, int w, int ci, int hid, int co, int stride) -> bool", &irb_fuses_op);
   m.def("first_layers_fuse(int n, int c, int h, int w, int co, int k, int stride, int pad, int pool_k, int pool_stride, "
         "int pool_pad) -> bool", &first_layers_fuse_op);
+  m.def("conv1x1_avgpool_fuses(int n, int hw, int ci, int co) -> bool", &conv_avgpool_fuses_op);
   m.def("clear_weight_cache() -> ()", &clear_cache_op);
   m.def("weight_cache_size() -> int", &cache_size_op);
   m.def("conv2d_route(int x_bits, int w_bits, int[] in_nhwc, int[] w_ohwi, int[] padding, int[] stride, "
@@ -1312,6 +1374,7 @@ TORCH_LIBRARY_IMPL(torch_mlu, CUDA, m) {  // ROCm tensors dispatch on the CUDA k
   m.impl("qconv2d_head", &qconv2d_head_op);
   m.impl("qconv2d_irb", &qconv2d_irb_op);
   m.impl("qconv2d_first_layers", &qconv2d_first_layers_op);
+  m.impl("qconv2d_avgpool", &qconv2d_avgpool_op);
   m.impl("qconv2d_chain", &qconv2d_chain_op);
   m.impl("qlinear", &qlinear_op);
   m.impl("maxpool_nhwc", &maxpool_nhwc_op);

@@ -163,7 +163,7 @@ def _decode(layer, sd, device, ci_dev, co_dev, fractional=False):
 class FusedNet(object):
     def __init__(self, layers, state_dict, device="cuda", out_half=False, fuse_shortcuts=True,
                  fractional_scale=False, chain_links=None, fuse_heads=True, fuse_blocks=False,
-                 fuse_first_layers=True):
+                 fuse_first_layers=True, fuse_avgpool=True):
         """fractional_scale: quantize activations and weights with position and fractional scale -- the
         general form the reference's fused (graph) mode hands to its backend per tensor / per axis
         (jit/utils/utils.cpp:81-167) -- instead of the eager ops' power-of-two steps.
@@ -183,7 +183,9 @@ class FusedNet(object):
         measured 2 % slower with it (one stream: 1.5 % faster).
         fuse_first_layers: the input quantizer, a few-channel first convolution + ReLU and the max pooling that is its
         only reader run as one launch (torch_mlu::qconv2d_first_layers) where the library's kernel serves the shape;
-        neither the quantized image nor the convolution's output is then stored."""
+        neither the quantized image nor the convolution's output is then stored.
+        fuse_avgpool: a 1x1 convolution whose only reader is the global average pooling runs inside the pooling's launch
+        (torch_mlu::qconv2d_avgpool) where the library's kernel serves the shape; its fp32 output is then never stored."""
         self.layers = list(layers)
         self.device = torch.device(device)
         self.outputs = outputs_of(self.layers)
@@ -316,6 +318,27 @@ class FusedNet(object):
                     and len(self.q_demand[pool.name]) == 1 and self.q_demand[pool.name][0][0] == 8
                     and self.q_demand[pool.name][0][2] == 1.0 and self.q_demand[l0.name] == self.q_demand[pool.name]):
                 self.first_pool = pool
+        # Global average pooling: pooled_conv[pooling layer name] = the 1x1 convolution in front of it, when nothing else
+        # reads that convolution.
+        self.pooled_conv = {}
+        if fuse_avgpool:
+            by_name = {l.name: l for l in self.layers}
+            for g in self.layers:
+                c = by_name.get(g.src) if g.kind == "gap" and isinstance(g.src, str) else None
+                if c is None or c.kind != "conv":
+                    continue
+                cq = self.q[c.name]
+                readers = [m for m in self.layers
+                           if m.src == c.name or (isinstance(m.src, tuple) and c.name in m.src) or m.add == c.name]
+                if (readers == [g] and c.k == 1 and c.pad == 0 and c.stride == 1 and c.groups == 1
+                        and c.act in ("none", "relu", "relu6") and not c.add_after and (cq.bw_x, cq.bw_w) == (8, 8)
+                        and cq.chan_div is not None and cq.bias is not None and -64 <= cq.exp2 <= 64
+                        and c.name not in self.outputs and not self.q_demand[c.name]
+                        and c.name not in self.chain_of and c.name not in self.shortcut_of and c.name not in self.block_of
+                        and c.name not in self._fused_away and c.name not in self._head_names
+                        and not (self.stem and self.stem["name"] == c.name)):
+                    self.pooled_conv[g.name] = c
+        self._pooled_names = set(c.name for c in self.pooled_conv.values())
         self._block_inner = {}
         for pname, (x, d) in self.block_of.items():
             self._block_inner[x.name] = pname
@@ -342,6 +365,14 @@ class FusedNet(object):
         l0, pool = self.layers[0], self.first_pool
         return bool(torch.ops.torch_mlu.first_layers_fuse(n, c, h, w, self.cdev[l0.name], l0.k, l0.stride, l0.pad, pool.k,
                                                           pool.stride, pool.pad))
+
+    def avgpool_fuses(self, gap, n, h, w):
+        """whether the 1x1 convolution in front of the pooling layer `gap` runs inside the pooling's launch over n images
+        of h x w"""
+        c = self.pooled_conv.get(gap.name)
+        if c is None:
+            return False
+        return bool(torch.ops.torch_mlu.conv1x1_avgpool_fuses(n, h * w, self.cdev[c.src], self.cdev[c.name]))
 
     def head_fuses(self, head, n, h, w):
         """whether the 1x1 layer `head` and the 3x3 layer behind it run as one launch over n images of h x w"""
@@ -482,11 +513,19 @@ class FusedNet(object):
                 env[("input",) + d] = ops.quantize_nhwc(x, d[0], d[1], self.cdev["input"], d[2])
         skipped_heads = set()
         skipped_inner = set()
+        pooled_inside = set()
         by_name = {l.name: l for l in self.layers}
         for l in self.layers:
             name = l.name
             if name in first_fused:
                 continue
+            if l.kind == "conv" and not tracing and name in self._pooled_names:
+                lq = self.q[name]
+                px = env[(l.src, lq.bw_x, lq.pos_x, lq.scale_x)]
+                gap = next(g for g in self.layers if self.pooled_conv.get(g.name) is l)
+                if self.avgpool_fuses(gap, px.shape[0], px.shape[1], px.shape[2]):
+                    pooled_inside.add(name)  # computed inside the launch of the pooling behind it
+                    continue
             if l.kind == "conv" and not tracing and name in self._block_inner:
                 pl = by_name[self._block_inner[name]]
                 x_, d_ = self.block_of[pl.name]
@@ -600,6 +639,23 @@ class FusedNet(object):
             elif l.kind == "maxpool":
                 for form in self._forms(name):
                     env[(name,) + form] = ops.maxpool_nhwc(env[(l.src,) + form], l.k, l.stride, l.pad)
+            elif l.kind == "gap" and l.src in pooled_inside:
+                c = self.pooled_conv[name]
+                cq = self.q[c.name]
+                qds = self.q_demand[name]
+                want_mean = self.f_demand[name] or len(qds) != 1
+                qd = qds[0] if qds else None
+                tick(c.name)
+                mean, q = ops.qconv2d_avgpool(env[(c.src, cq.bw_x, cq.pos_x, cq.scale_x)], cq.qw, cq.exp2, cq.chan_div, cq.bias,
+                                              env[(c.add, "f")] if c.add else None, _ACT_CODE[c.act], want_mean,
+                                              qd[0] if qd else 0, qd[1] if qd else 0, qd[2] if qd else 1.0)
+                tick(c.name)
+                if want_mean:
+                    env[(name, "f")] = mean.reshape(mean.shape[0], 1, 1, mean.shape[1])
+                if qd:
+                    env[(name,) + qd] = q.reshape(q.shape[0], 1, 1, q.shape[1])
+                for d in qds[1:]:
+                    env[(name,) + d] = ops.quantize(env[(name, "f")], d[0], d[1], d[2])
             elif l.kind == "gap":
                 if self.f_demand[name] or tracing or not self.q_demand[name]:
                     g = ops.global_avgpool_nhwc(env[(l.src, "f")])

@@ -355,6 +355,28 @@ int catchq_first_layers_nchw(const float *x, int n, int c, int h, int w, int x_p
                              int pool_stride, int pool_pad, void *q, int sharing, void *workspace,
                              size_t workspace_bytes, catchq_stream_t stream);
 
+/* A 1x1 convolution and the global average pooling behind it in one launch (the end of a classifier's feature
+ * extractor).  In the reference: torch_mlu::conv2d (cnnl_conv2d, operators/cnnl/quantify_conv_forward.cpp:56-147), the
+ * block's float add (cnnl_add, operators/cnnl/add.cpp) and ReLU (operators/cnnl/activation.cpp) where it has them,
+ * adaptive_avg_pool2d((1,1)) (operators/cnnl/pooling.cpp), and the quantization of the classifier's input
+ * (cnnl_linear, operators/cnnl/linear.cpp:40-167).  For x [n, hw, ci] (int8) and w [co, ci] (int8):
+ *   v[i, p, c] = `epilogue` applied to the sums of the 1x1 convolution exactly as catchq_conv2d_nhwc applies it (exp2,
+ *                chan_div, chan_rcp, bias, resid [n, hw, co] fp32, act none / ReLU / ReLU6; its y, q and acc_out must be
+ *                NULL and resid_after_act 0: the convolution's output is never stored)
+ *   mean[i, c] = (sum of v[i, p, c] over p in storage order, one fp32 addition each) / hw      fp32 [n, co], may be NULL
+ *   q[i, c]    = sat(rne(mean[i, c] * q_scale * 2^-q_position))        int8 / int16 (q_bitwidth 8 / 16) [n, co], may be NULL
+ * -- the values of catchq_conv2d_nhwc with an fp32 output followed by catchq_global_avgpool_nhwc /
+ * catchq_global_avgpool_quantize_nhwc, bit for bit.  The fused kernel serves hw <= 64, ci % 32 == 0 (ci <= 4096),
+ * co % 32 == 0, an epilogue with chan_div, chan_rcp and bias (-64 <= exp2 <= 64) and no exp2_dev
+ * (catchq_conv1x1_avgpool_workspace_size reports 0 then); anything else runs as the two launches with the convolution's
+ * fp32 output (n * hw * co * 4 bytes) in the caller's workspace. */
+int catchq_conv1x1_avgpool_workspace_size(int n, int hw, int ci, int co, const catchq_epilogue_t *epilogue,
+                                          size_t *bytes);
+int catchq_conv1x1_avgpool_nhwc(const void *x, const void *w, int n, int hw, int ci, int co,
+                                const catchq_epilogue_t *epilogue, float *mean, void *q, int q_bitwidth,
+                                int q_position, float q_scale, void *workspace, size_t workspace_bytes,
+                                catchq_stream_t stream);
+
 /* Residual chain of a stage of bottleneck blocks, recomputed from its int8 inputs in one launch.
  * In the reference every residual block ends in torch_mlu::conv2d (cnnl_conv2d,
  * operators/cnnl/quantify_conv_forward.cpp:56-147) followed by a float add (cnnl_add, operators/cnnl/add.cpp)

@@ -213,6 +213,22 @@ def first_layers_nchw(x, x_pos, conv, k, stride=2, pad=3, pool=(3, 2, 1), x_scal
     return q, need.value
 
 
+def conv1x1_avgpool_nhwc(x, w, exp2=0, chan_div=None, bias=None, resid=None, act=0, chan_rcp=None, want_mean=True, q_bw=0,
+                         q_pos=0, q_scale=1.0):
+    """x [N,H,W,Ci] int8, w [Co,Ci] int8 -> ({"mean": fp32 [N,Co] or None, "q": int8 / int16 [N,Co] or None},
+    workspace bytes the library asked for)"""
+    n, hw, ci, co = x.shape[0], x.shape[1] * x.shape[2], x.shape[3], w.shape[0]
+    e, _ = _epilogue((n, hw, 1, co), x.device, exp2, chan_div, bias, resid, act, None, False, 0, 0, 1.0, chan_rcp)
+    need = ctypes.c_size_t()
+    check(lib().catchq_conv1x1_avgpool_workspace_size(n, hw, ci, co, ctypes.byref(e), ctypes.byref(need)))
+    ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=x.device)
+    mean = torch.empty((n, co), dtype=torch.float32, device=x.device) if want_mean else None
+    q = torch.empty((n, co), dtype=_INT[q_bw], device=x.device) if q_bw else None
+    check(lib().catchq_conv1x1_avgpool_nhwc(ptr(x), ptr(w), n, hw, ci, co, ctypes.byref(e), ptr(mean), ptr(q), q_bw, q_pos,
+                                            q_scale, ptr(ws), need.value, stream()))
+    return {"mean": mean, "q": q}, need.value
+
+
 def conv1x1_chain_nhwc(links, want_y=True, want_q=True, q_pos=0, sharing=0):
     """links: dicts with x [N,H,W,Ci] int8, w [Co,Ci] int8, stride, exp2, chan_div, chan_rcp, bias (device tensors);
     links[0] is the projection shortcut.  -> {"y": fp32 or None, "q": int8 or None}"""

@@ -77,6 +77,24 @@ def check_plan_rows(fused, x, images, rows_per_layer=3):
                     assert np.array_equal(want, got[n:n + 1].cpu().numpy()), "first layers: image %d" % n
                     checked += 1
                 continue
+            if l.name in fused._pooled_names and (l.name, "f") not in keep:
+                # computed inside the launch of the global average pooling behind it: the pooled values of the sampled
+                # images against the oracle's convolution, epilogue, ordered mean and quantizer
+                gap = next(g for g in fused.layers if fused.pooled_conv.get(g.name) is l)
+                qx = keep[(l.src, lq.bw_x, lq.pos_x, lq.scale_x)]
+                for n in images:
+                    acc, ovf = orc.conv2d_nhwc(qx[n:n + 1].cpu().numpy(), lq.qw.cpu().numpy(), (0, 0), (1, 1), (1, 1), 1)
+                    assert ovf == 0
+                    resid = keep[(l.add, "f")][n:n + 1].float().cpu().numpy() if l.add else None
+                    mean = orc.global_avgpool_nhwc(orc.epilogue(acc, lq.exp2, _np(lq.chan_div), _np(lq.bias), resid, _ACT[l.act]))
+                    if (gap.name, "f") in keep:
+                        assert np.array_equal(mean, keep[(gap.name, "f")][n:n + 1].reshape(mean.shape).cpu().numpy()), gap.name
+                        checked += 1
+                    for d in fused.q_demand[gap.name]:
+                        got = keep[(gap.name,) + tuple(d)][n:n + 1].reshape(mean.shape).cpu().numpy()
+                        assert np.array_equal(orc.quantize(mean, d[0], d[1], d[2]), got), gap.name
+                        checked += 1
+                continue
             if l.name in fused._head_names and (l.name, 8, fused.q_demand[l.name][0][1], 1.0) not in keep:
                 continue  # a 1x1 head computed inside the launch of the 3x3 layer behind it: covered there
             head = fused.head_of.get(l.name)
@@ -152,6 +170,8 @@ def check_plan_rows(fused, x, images, rows_per_layer=3):
                     want = orc.maxpool_nhwc(src[n:n + 1].float().cpu().numpy(), l.k, l.stride, l.pad)
                     assert np.array_equal(want, got[n:n + 1].float().cpu().numpy()), l.name
                     checked += 1
+        elif l.kind == "gap" and (l.src, "f") not in keep:
+            assert l.name in fused.pooled_conv  # pooled inside the launch that computes the convolution: covered there
         elif l.kind == "gap":
             src = keep[(l.src, "f")]
             mean = orc.global_avgpool_nhwc(src[list(images)].cpu().numpy())

@@ -1078,6 +1078,55 @@ def test_first_layers(case):
     assert same_bits(want, got.cpu().numpy())
 
 
+CONV_AVGPOOL_CASES = [
+    # N, H, W, Ci, Co, residual?, activation, fused in one launch?
+    (32, 7, 7, 512, 2048, True, 1, True),     # ResNet-50's last block: eight waves per block
+    (3, 7, 7, 512, 2048, True, 1, True),      # few images: four waves per block
+    (5, 7, 7, 320, 1280, False, 2, True),     # MobileNetV2's last convolution: ReLU6, ten K steps
+    (2, 8, 8, 64, 96, False, 0, True),        # 64 pixels: both pixel groups full; three channel groups on four waves
+    (4, 5, 6, 96, 32, True, 2, True),         # 30 pixels: one pixel group
+    (2, 1, 1, 32, 64, False, 1, True),        # a single pixel
+    (2, 3, 3, 2048, 64, False, 1, True),      # long K: the filter ring wraps eight times
+    (2, 9, 9, 64, 64, False, 1, False),       # 81 pixels: two launches
+    (2, 4, 4, 48, 64, True, 1, False),        # Ci % 32 != 0
+]
+
+
+@pytest.mark.parametrize("case", CONV_AVGPOOL_CASES)
+def test_conv1x1_global_avgpool(case):
+    """catchq_conv1x1_avgpool_nhwc against the oracle's convolution, epilogue (dequantization, bias, fp32 residual,
+    activation), ordered global average and quantizer, bit for bit, with and without the fp32 mean / the int8 form."""
+    n, h, w, ci, co, shortcut, act, fused = case
+    note("conv1x1_avgpool", case)
+    r = rng(sum(case[:5]))
+    x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, 1, 1, ci), 8)
+    div = r.uniform(0.6, 3.5, co).astype(np.float32)
+    bias = (r.standard_normal(co) * 1.5).astype(np.float32)
+    e1 = -11 - int(np.log2(ci / 32) / 2 + 0.5)
+    acc, ovf = orc.conv2d_nhwc(x, wt, (0, 0), (1, 1), (1, 1), 1)
+    assert ovf == 0
+    resid = (r.standard_normal(acc.shape) * 4).astype(np.float32) if shortcut else None
+    y = orc.epilogue(acc, e1, div, bias, resid, act)
+    assert (act == 0 or 0.1 < (y == 0).mean() < 0.9) and (act != 2 or 0.02 < (y == 6).mean() < 0.9)
+    mean = orc.global_avgpool_nhwc(y)
+    qp = -4 if act != 2 else -3
+    q8 = orc.quantize(mean, 8, qp, 0.93)
+    assert len(np.unique(q8)) > 8
+    dv = cabi.dev
+    xd, wd, dd, rd, bd = dv(x), dv(wt.reshape(co, ci)), dv(div), dv(np.float32(1) / div), dv(bias)
+    sd = dv(resid) if shortcut else None
+    for want_mean, q_bw in ((True, 8), (False, 8), (True, 0), (True, 16)):
+        out, ws_bytes = cabi.conv1x1_avgpool_nhwc(xd, wd, exp2=e1, chan_div=dd, bias=bd, resid=sd, act=act, chan_rcp=rd,
+                                                  want_mean=want_mean, q_bw=q_bw, q_pos=qp if q_bw == 8 else qp - 8, q_scale=0.93)
+        assert (ws_bytes == 0) == fused, ws_bytes
+        if want_mean:
+            assert same_bits(mean, out["mean"].cpu().numpy()), (want_mean, q_bw)
+        if q_bw == 8:
+            assert same_bits(q8, out["q"].cpu().numpy()), (want_mean, q_bw)
+        if q_bw == 16:
+            assert same_bits(orc.quantize(mean, 16, qp - 8, 0.93), out["q"].cpu().numpy()), (want_mean, q_bw)
+
+
 CHAIN_CASES = [
     # N, Ho, Wo, Co, shortcut (Cs, stride), main channel counts (one per block)
     (2, 14, 14, 256, (64, 1), (64,)),                  # first block of stage 1: shortcut + one block

@@ -198,7 +198,7 @@ def test_resnet50_residual_chains(limit):
     x = torch.randn(3, 3, 96, 96, generator=torch.Generator().manual_seed(9))
     sd = pipeline.calibrate(net, x, "int8", True)
     fused = pipeline.FusedNet(layers, sd, chain_links=limit)
-    plain = pipeline.FusedNet(layers, sd, chain_links=0)
+    plain = pipeline.FusedNet(layers, sd, chain_links=0, fuse_avgpool=False)
     lens = {n: len(c) for n, c in fused.chain_of.items()}
     if limit == 0:
         assert not lens and sorted(fused.shortcut_of) == ["l1.0.c3", "l2.0.c3", "l3.0.c3", "l4.0.c3"]
@@ -293,6 +293,40 @@ def test_resnet50_first_layers_in_one_launch():
     x2 = torch.randn(2, 3, 64, 62, generator=torch.Generator().manual_seed(13)).cuda()
     assert torch.equal(fused.forward(x2), plain.forward(x2))
     check_against_oracle(layers, sd, x, plain)
+
+
+@pytest.mark.parametrize("arch", ["resnet50", "mobilenet_v2"])
+def test_last_convolution_inside_the_average_pooling(arch):
+    """fuse_avgpool (the default): the 1x1 convolution in front of the global average pooling runs inside the pooling's
+    launch (torch_mlu::qconv2d_avgpool) at 7 x 7; its fp32 output is not produced, every other tensor of the plan and the
+    logits equal those of the plan with the two launches, eagerly and from a captured graph on two streams; at a
+    resolution whose last feature map has more than 64 pixels the same plan runs the two launches."""
+    note(arch, "bs4 224x224, last convolution inside the average pooling")
+    layers = nets.NETS[arch]()
+    net = nets.FloatNet(layers, seed=21, weight_std=0.2 if arch == "mobilenet_v2" else 0.05).eval()
+    x = torch.randn(4, 3, 224, 224, generator=torch.Generator().manual_seed(22))
+    sd = pipeline.calibrate(net, x, "int8", True)
+    fused = pipeline.FusedNet(layers, sd)
+    plain = pipeline.FusedNet(layers, sd, fuse_avgpool=False)
+    (gname, conv), = fused.pooled_conv.items()
+    assert not plain.pooled_conv and conv.k == 1
+    ka, kb = {}, {}
+    a = fused.forward(x.cuda(), keep=ka)
+    b = plain.forward(x.cuda(), keep=kb)
+    torch.cuda.synchronize()
+    assert sorted(set(kb) - set(ka)) == [(conv.name, "f")] and set(ka) <= set(kb)
+    assert torch.equal(a, b)
+    for key, t in ka.items():
+        assert torch.equal(t, kb[key]), key
+    static_in, replay = fused.capture(x.cuda(), streams=2)
+    for i in range(2):
+        static_in.copy_(x.cuda())
+        assert torch.equal(replay(), b), "replay %d" % i
+        _ = fused.forward(torch.randn(4, 3, 224, 224, device="cuda"))  # eager work between the replays
+        torch.cuda.synchronize()
+    x2 = torch.randn(2, 3, 288, 288, generator=torch.Generator().manual_seed(23)).cuda()  # 9 x 9 at the end
+    k2 = {}
+    assert torch.equal(fused.forward(x2, keep=k2), plain.forward(x2)) and (conv.name, "f") in k2
 
 
 def test_darknet53_yolov3_int16_activations():
