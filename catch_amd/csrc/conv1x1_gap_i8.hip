@@ -188,24 +188,32 @@ __global__ __launch_bounds__(64 * NW) void conv1x1_gap_kernel(const int8_t *__re
   }
 }
 
-// images of at most 64 pixels, K a multiple of 32 up to 4096, Co a multiple of 32
+// waves per block and LDS bytes; false: not this kernel's shape (images of at most 64 pixels, K a multiple of 32, Co a
+// multiple of 32, pixels and output tiles within the LDS of a compute unit)
+static bool gap_plan(int N, int HW, int K, int Co, int &nw, int &lds_bytes) {
+  if (!(N > 0 && HW >= 1 && HW <= 64 && K >= 32 && K % 32 == 0 && K <= 4096 && Co >= 32 && Co % 32 == 0 &&
+        (int64_t)N * HW * K < (1ll << 31) && (int64_t)N * HW * Co < (1ll << 31) && (int64_t)Co * K < (1ll << 31)))
+    return false;
+  // eight waves (256 channels) per block, four where that leaves compute units without a block
+  nw = ((int64_t)N * ((Co + 255) / 256) >= 256) ? 8 : 4;
+  const int tile_x = HW * (K + 16), tile_y = nw * HW * GC_YP * 4;
+  lds_bytes = ((tile_x > tile_y ? tile_x : tile_y) + 255) / 256 * 256;
+  return lds_bytes <= 160 * 1024;
+}
+
 bool conv1x1_gap_i8_ok(int N, int HW, int K, int Co) {
-  return N > 0 && HW >= 1 && HW <= 64 && K >= 32 && K % 32 == 0 && K <= 4096 && Co >= 32 && Co % 32 == 0 &&
-         (int64_t)N * HW * K < (1ll << 31) && (int64_t)N * HW * Co < (1ll << 31) && (int64_t)Co * K < (1ll << 31);
+  int nw, lds;
+  return gap_plan(N, HW, K, Co, nw, lds);
 }
 
 // x [N, HW, K] int8, w [Co, K] int8; mean / q [N, Co].  -1: not this kernel's shape.
 int conv1x1_gap_i8(const void *x, const void *w, int N, int HW, int K, int Co, const GapConvDev &e, hipStream_t st) {
-  if (!conv1x1_gap_i8_ok(N, HW, K, Co)) return -1;
+  int nw, lds_bytes;
+  if (!gap_plan(N, HW, K, Co, nw, lds_bytes)) return -1;
   GapConvParams p = {};
   p.N = N; p.HW = HW; p.K = K; p.Co = Co;
   p.xs = K + 16;
   p.groups = (HW + 31) / 32;
-  // eight waves (256 channels) per block, four where that leaves compute units without a block
-  const int nw = ((int64_t)N * ((Co + 255) / 256) >= 256) ? 8 : 4;
-  const int tile_x = HW * p.xs, tile_y = nw * HW * GC_YP * 4;
-  const int lds_bytes = ((tile_x > tile_y ? tile_x : tile_y) + 255) / 256 * 256;
-  if (lds_bytes > 160 * 1024) return -1;
   auto launch = [&](auto kern) {
     if (lds_bytes > 64 * 1024) {
       static std::atomic<bool> raised[64];

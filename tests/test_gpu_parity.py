@@ -1089,6 +1089,7 @@ CONV_AVGPOOL_CASES = [
     (2, 3, 3, 2048, 64, False, 1, True),      # long K: the filter ring wraps eight times
     (2, 9, 9, 64, 64, False, 1, False),       # 81 pixels: two launches
     (2, 4, 4, 48, 64, True, 1, False),        # Ci % 32 != 0
+    (1, 8, 8, 4096, 32, False, 1, False),     # 64 pixels x 4096 channels: more than a compute unit's LDS holds
 ]
 
 
