@@ -1128,6 +1128,65 @@ def test_conv1x1_global_avgpool(case):
             assert same_bits(orc.quantize(mean, 16, qp - 8, 0.93), out["q"].cpu().numpy()), (want_mean, q_bw)
 
 
+@pytest.mark.parametrize("seed", range(2))
+def test_first_layers_and_pooled_convolution_random_sweep(seed):
+    """random shapes inside the one-launch kernels' domains: 30 convolutions with the average pooling inside (1 to 64
+    pixels, 32 to 256 input and up to 352 output channels, one to 70 images, every activation, with and without
+    residual) and 20 first-layer stacks (one to three input channels, heights 7 to 69, widths 8 to 68, 32 / 64 / 128 output
+    channels, with and without a fractional input scale), bit-exact against the oracle, none through the workspace."""
+    r = rng(4100 + seed)
+    dv = cabi.dev
+    for it in range(30):
+        n = int(r.choice([1, 2, 3, 5, 9, 33, 70]))
+        h, w = int(r.integers(1, 9)), int(r.integers(1, 9))
+        ci, co = 32 * int(r.integers(1, 9)), 32 * int(r.integers(1, 12))
+        if n >= 33:
+            ci, co = min(ci, 128), min(co, 128)
+        act, use_res = int(r.integers(0, 3)), bool(r.integers(0, 2))
+        case = ("conv1x1_avgpool sweep", seed, it, n, h, w, ci, co, act, use_res)
+        note(*case)
+        x, wt = _ints(r, (n, h, w, ci), 8), _ints(r, (co, 1, 1, ci), 8)
+        div = r.uniform(0.6, 3.5, co).astype(np.float32)
+        bias = (r.standard_normal(co) * 1.5).astype(np.float32)
+        e1 = -11 - int(np.log2(ci / 32) / 2 + 0.5)
+        acc, ovf = orc.conv2d_nhwc(x, wt, (0, 0), (1, 1), (1, 1), 1)
+        assert ovf == 0
+        resid = (r.standard_normal(acc.shape) * 4).astype(np.float32) if use_res else None
+        mean = orc.global_avgpool_nhwc(orc.epilogue(acc, e1, div, bias, resid, act))
+        out, ws_bytes = cabi.conv1x1_avgpool_nhwc(dv(x), dv(wt.reshape(co, ci)), exp2=e1, chan_div=dv(div), bias=dv(bias),
+                                                  resid=dv(resid) if use_res else None, act=act,
+                                                  chan_rcp=dv(np.float32(1) / div), want_mean=True, q_bw=8, q_pos=-4)
+        assert ws_bytes == 0, case
+        assert same_bits(mean, out["mean"].cpu().numpy()), case
+        assert same_bits(orc.quantize(mean, 8, -4), out["q"].cpu().numpy()), case
+    for it in range(20):
+        n, c = int(r.choice([1, 2, 3, 7, 20, 40])), int(r.integers(1, 4))
+        h, w, co = int(r.integers(7, 70)), 4 * int(r.integers(2, 18)), int(r.choice([32, 64, 128]))
+        if n >= 20:
+            h, w = min(h, 40), min(w, 40)
+        act = int(r.integers(1, 3))
+        x_scale = float(np.float32(r.uniform(0.8, 1.2))) if r.integers(0, 2) else 1.0
+        case = ("first_layers sweep", seed, it, n, c, h, w, co, act, x_scale)
+        note(*case)
+        x = (r.standard_normal((n, c, h, w)) * 1.5).astype(np.float32)
+        wt = _ints(r, (co, 7, 7, 4), 8)
+        wt[..., c:] = 0
+        div = r.uniform(0.6, 3.5, co).astype(np.float32)
+        bias = (r.standard_normal(co) * 2.0).astype(np.float32)
+        e1 = -11 - int(np.log2(c) / 2 + 0.5)
+        qx = orc.quantize_nchw_to_nhwc(x, 8, -5, x_scale, cpad=4)
+        acc, ovf = orc.conv2d_nhwc(qx, wt, (3, 3), (2, 2), (1, 1), 1)
+        assert ovf == 0
+        q1 = orc.quantize(orc.epilogue(acc, e1, div, bias, None, act), 8, -3)
+        want = orc.maxpool_nhwc(q1.astype(np.float32), 3, 2, 1).astype(np.int8)
+        wdev = np.zeros((co, 7, 8, 4), np.int8)
+        wdev[:, :, :7] = wt
+        conv = dict(w=dv(wdev), exp2=e1, chan_div=dv(div), chan_rcp=dv(np.float32(1) / div), bias=dv(bias), act=act, q_pos=-3)
+        got, ws_bytes = cabi.first_layers_nchw(dv(x), -5, conv, 7, 2, 3, (3, 2, 1), x_scale, 0)
+        assert ws_bytes == 0, case
+        assert same_bits(want, got.cpu().numpy()), case
+
+
 CHAIN_CASES = [
     # N, Ho, Wo, Co, shortcut (Cs, stride), main channel counts (one per block)
     (2, 14, 14, 256, (64, 1), (64,)),                  # first block of stage 1: shortcut + one block
