@@ -1082,14 +1082,14 @@ CONV_AVGPOOL_CASES = [
     # N, H, W, Ci, Co, residual?, activation, fused in one launch?
     (32, 7, 7, 512, 2048, True, 1, True),     # ResNet-50's last block: eight waves per block
     (3, 7, 7, 512, 2048, True, 1, True),      # few images: four waves per block
-    (5, 7, 7, 320, 1280, False, 2, True),     # MobileNetV2's last convolution: ReLU6, ten K steps
+    (5, 7, 7, 320, 1280, False, 2, True),     # MobileNetV2's last convolution: ReLU6, rows of 20 pieces (swizzle over 4)
     (2, 8, 8, 64, 96, False, 0, True),        # 64 pixels: both pixel groups full; three channel groups on four waves
-    (4, 5, 6, 96, 32, True, 2, True),         # 30 pixels: one pixel group
+    (4, 5, 6, 96, 32, True, 2, True),         # 30 pixels: one pixel group; rows of 6 pieces (swizzle over 2)
     (2, 1, 1, 32, 64, False, 1, True),        # a single pixel
-    (2, 3, 3, 2048, 64, False, 1, True),      # long K: the filter ring wraps eight times
+    (2, 3, 3, 2048, 64, False, 1, True),      # long K: four passes through LDS
     (2, 9, 9, 64, 64, False, 1, False),       # 81 pixels: two launches
     (2, 4, 4, 48, 64, True, 1, False),        # Ci % 32 != 0
-    (1, 8, 8, 4096, 32, False, 1, False),     # 64 pixels x 4096 channels: more than a compute unit's LDS holds
+    (1, 8, 8, 4096, 32, False, 1, True),      # 64 pixels x 4096 channels: eight passes of 512 bytes through LDS
 ]
 
 
