@@ -16,9 +16,10 @@
 //                 (reciprocal-form division, bias, the activation folded into the requantizer's clamp) and
 //                 writes one dword into the band's convolution tile in LDS.  The 2*PR + 1 convolution rows of a
 //                 band share one row with the band above: that row is computed twice;
-//   3  pool       a lane takes four channels of one pooled pixel: nine dwords of the tile, the bytes compared two
-//                 at a time as 16-bit halves (the activation leaves 0..127, unsigned order is the signed one),
-//                 one dword stored.  Window taps in the padding read a neighbour inside the window instead.
+//   3  pool       a lane takes four channels of one pooled column and walks down the band: three dwords of a
+//                 convolution row give the row's maximum, shared by the two windows that contain the row; bytes are
+//                 compared two at a time as 16-bit halves (the activation leaves 0..127, unsigned order is the
+//                 signed one).  Window taps in the padding read a neighbour inside the window instead.
 //
 // Neither the framed int8 image nor the convolution's output reaches memory.  Every integer is the one the three
 // separate launches produce: the same quantizer, the same sums, the same float operations in the same order, and
@@ -179,37 +180,51 @@ __global__ __launch_bounds__(64 * NW) void stem_pool_kernel(const float *__restr
   __syncthreads();
 
   // ---- 3: 3x3 stride-2 maximum over the tile -------------------------------------------------------------------------
+  // A lane owns four channels of one pooled column and walks down the band's pooled rows: the maximum over the three
+  // columns of a convolution row is taken once and shared by the two windows that contain the row.  Bytes are compared
+  // two at a time as 16-bit halves: the even bytes masked out, the odd bytes in place (the byte below them only
+  // breaks ties).
   {
     typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
     const int quads = p.Co >> 2;
-    const int items = prn * p.Wp * quads;
+    const int items = p.Wp * quads;
     const int8_t *tile = lds + p.off_tile;
     int8_t *out = Q + ((int64_t)img * p.Hp + pr0) * p.Wp * p.Co;
     for (int it = tid; it < items; it += NT) {
-      const int px = it / quads, q = it - px * quads;
-      const int i = px / p.Wp, j = px - i * p.Wp;
-      int rr[3], cc[3];
+      const int j = it / quads, q = it - j * quads;
+      int cofs[3];
 #pragma unroll
-      for (int a = 0; a < 3; ++a) {
-        int r = 2 * (pr0 + i) - 1 + a, c = 2 * j - 1 + a;
-        r = r < 0 ? 0 : (r > p.Hc - 1 ? p.Hc - 1 : r);
-        c = c < 0 ? 0 : (c > p.Wc - 1 ? p.Wc - 1 : c);
-        rr[a] = (r - cr0) * p.Wc;
-        cc[a] = c;
+      for (int b = 0; b < 3; ++b) {
+        int c = 2 * j - 1 + b;
+        c = c < 0 ? 0 : (c > p.Wc - 1 ? p.Wc - 1 : c);  // a tap in the padding reads a neighbour inside the window
+        cofs[b] = c * tp + 4 * q;
       }
-      unsigned raw[9];
-#pragma unroll
-      for (int a = 0; a < 3; ++a)
-#pragma unroll
-        for (int b = 0; b < 3; ++b) raw[a * 3 + b] = *reinterpret_cast<const unsigned *>(tile + (rr[a] + cc[b]) * tp + 4 * q);
-      u16x2 even = {0, 0}, odd = {0, 0};
-#pragma unroll
-      for (int k = 0; k < 9; ++k) {
-        even = __builtin_elementwise_max(even, __builtin_bit_cast(u16x2, raw[k] & 0x00ff00ffu));
-        odd = __builtin_elementwise_max(odd, __builtin_bit_cast(u16x2, raw[k] & 0xff00ff00u));
+      u16x2 even_r, odd_r;
+      auto row_max = [&](int conv_row) {
+        const int r = (conv_row < 0 ? 0 : (conv_row > p.Hc - 1 ? p.Hc - 1 : conv_row)) - cr0;
+        const int8_t *base = tile + r * p.Wc * tp;
+        const unsigned a = *reinterpret_cast<const unsigned *>(base + cofs[0]);
+        const unsigned b = *reinterpret_cast<const unsigned *>(base + cofs[1]);
+        const unsigned c = *reinterpret_cast<const unsigned *>(base + cofs[2]);
+        even_r = __builtin_elementwise_max(__builtin_elementwise_max(__builtin_bit_cast(u16x2, a & 0x00ff00ffu),
+                                                                     __builtin_bit_cast(u16x2, b & 0x00ff00ffu)),
+                                           __builtin_bit_cast(u16x2, c & 0x00ff00ffu));
+        odd_r = __builtin_elementwise_max(__builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)),
+                                          __builtin_bit_cast(u16x2, c));
+      };
+      row_max(2 * pr0 - 1);
+      u16x2 even_p = even_r, odd_p = odd_r;  // the row shared with the window above
+      for (int i = 0; i < prn; ++i) {
+        row_max(2 * (pr0 + i));
+        u16x2 even = __builtin_elementwise_max(even_p, even_r), odd = __builtin_elementwise_max(odd_p, odd_r);
+        row_max(2 * (pr0 + i) + 1);
+        even = __builtin_elementwise_max(even, even_r);
+        odd = __builtin_elementwise_max(odd, odd_r);
+        even_p = even_r;
+        odd_p = odd_r;
+        *reinterpret_cast<unsigned *>(out + ((int64_t)i * p.Wp + j) * p.Co + 4 * q) =
+            __builtin_bit_cast(unsigned, even) | (__builtin_bit_cast(unsigned, odd) & 0xff00ff00u);
       }
-      *reinterpret_cast<unsigned *>(out + (int64_t)px * p.Co + 4 * q) =
-          __builtin_bit_cast(unsigned, even) | __builtin_bit_cast(unsigned, odd);
     }
   }
 }
@@ -219,9 +234,9 @@ __global__ __launch_bounds__(64 * NW) void stem_pool_kernel(const float *__restr
 // Band height: a block's work grows with its 2 * PR + 1 convolution rows plus a fixed part (set-up, barriers, the
 // latency of its input rows), the launch takes as many rounds of blocks as the busiest compute unit gets, and a
 // compute unit that holds one block at a time (more than 80 KiB of LDS) cannot hide one block's input latency behind
-// another's arithmetic.  Measured on 32 x 3 x 224 x 224 (us): PR 1 34.8, 2 29.1, 3 30.2, 4 31.6, 5 36.7, 6 40.8 and,
-// with one block of sixteen waves per compute unit, 7 24.1 -- the estimate below ranks them in that order.  Blocks that
-// are alone on their compute unit run sixteen waves.
+// another's arithmetic.  Measured on 32 x 3 x 224 x 224 (us): PR 2 25.6, 3 25.7, 4 25.7, 5 28.9, 6 30.3 and, with one
+// block of sixteen waves per compute unit, 7 20.0 (64 images: 3 42.0, 7 39.3) -- the estimate below ranks them in that
+// order.  Blocks that are alone on their compute unit run sixteen waves.
 static bool stem_pool_plan(int N, int C, int H, int W, int Co, StemPoolParams &p, int &lds_bytes, int &waves) {
   if (N <= 0 || C < 1 || C > 3 || H < 7 || W < 8 || W % 4 != 0 || W > 2048) return false;
   if (Co != 32 && Co != 64 && Co != 128) return false;
@@ -248,7 +263,7 @@ static bool stem_pool_plan(int N, int C, int H, int W, int Co, StemPoolParams &p
     if (lds > 160 * 1024) break;
     const int bands = (p.Hp + pr - 1) / pr;
     const int64_t rounds = ((int64_t)N * bands + kDeviceCUs - 1) / kDeviceCUs;
-    const int64_t cost = rounds * (4 * pr + 5) * (lds > 80 * 1024 ? 150 : 115);
+    const int64_t cost = rounds * (4 * pr + 5) * (lds > 80 * 1024 ? 140 : 115);
     if (want > 0 ? (pr == want || !best) : (!best || cost < best_cost)) { best = pr; best_cost = cost; }
   }
   if (!best) return false;
