@@ -1090,6 +1090,8 @@ CONV_AVGPOOL_CASES = [
     (2, 9, 9, 64, 64, False, 1, False),       # 81 pixels: two launches
     (2, 4, 4, 48, 64, True, 1, False),        # Ci % 32 != 0
     (1, 8, 8, 4096, 32, False, 1, True),      # 64 pixels x 4096 channels: eight passes of 512 bytes through LDS
+    (300, 2, 2, 512, 64, True, 1, True),      # more blocks than compute units: passes of 256 bytes, two blocks a unit
+    (130, 3, 3, 320, 512, False, 2, True),    # the same with rows of 10 pieces (passes of 160 bytes)
 ]
 
 
